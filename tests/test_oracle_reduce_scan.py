@@ -1,0 +1,166 @@
+"""Pins the oracle's reduction / prefix-sum functions.
+
+Sources of truth used here, none of which restates the oracle's own loops:
+  * numpy's float32 cumsum (strictly sequential accumulation) for the reference CPU path,
+  * math.fsum (exactly rounded) and numpy float64 cumsum for the fp64 definition,
+  * the reference's constant-0.001 input fixture in closed form, within the tolerances
+    the reference's own (disabled) checks use: 0.1 reduce, 0.01 scan, 0.001 CUB/Thrust
+    (reference src/reduction/seg_wmma_16.cu:89, src/prefixsum/seg_wmma_16.cu:91,
+    src/reduction/seg_cub_block.cu:97-127),
+  * inputs on the k/2048 grid, whose partial sums are exact in fp32 and fp64,
+  * structural identities (one-hot -> step, zeros -> zeros, scan's last == reduce).
+"""
+import math
+
+import numpy as np
+import pytest
+
+SEGS = [16, 32, 256, 1024, 2048, 16384]
+C = 0.00100040435791015625  # fp16(0.001f), the reference's fill value
+
+
+def as_f(x16, dt):
+    return x16.view(np.float16).astype(dt)
+
+
+@pytest.mark.parametrize("seg", SEGS)
+def test_ref_path_matches_numpy_float32_sequential(oracle, seg):
+    n = 1 << 17
+    nseg = n // seg
+    x = oracle.generate_f16(n, 3, oracle.DIST_UNIFORM)
+    cs = np.cumsum(as_f(x, np.float32).reshape(nseg, seg), axis=1, dtype=np.float32)
+    assert np.array_equal(oracle.seg_scan_ref(x, nseg, seg), cs.astype(np.float16).view(np.uint16).ravel())
+    assert np.array_equal(oracle.seg_reduce_ref(x, nseg, seg), cs[:, -1].astype(np.float16).view(np.uint16))
+    # threaded split gives the same bits
+    assert np.array_equal(oracle.seg_reduce_ref(x, nseg, seg, nthreads=5), oracle.seg_reduce_ref(x, nseg, seg))
+    assert np.array_equal(oracle.seg_scan_ref(x, nseg, seg, nthreads=3), oracle.seg_scan_ref(x, nseg, seg))
+
+
+def test_config1_cpu_reference_case(oracle):
+    # N = 2^20, seed 0, segments of 16: the CPU-runnable configuration
+    n, seg = 1 << 20, 16
+    x = oracle.generate_f16(n, 0, oracle.DIST_UNIFORM)
+    out = oracle.seg_reduce_ref(x, n // seg, seg)
+    cs = np.cumsum(as_f(x, np.float32).reshape(-1, seg), axis=1, dtype=np.float32)[:, -1]
+    assert np.array_equal(out, cs.astype(np.float16).view(np.uint16))
+    # and it satisfies the tolerance rule against the fp64 definition
+    bad, worst, _ = oracle.check_f16(out, oracle.seg_reduce_f64(x, n // seg, seg), seg)
+    assert bad == 0 and worst < 0
+
+
+def test_full_ref_matches_numpy(oracle):
+    n = 50000
+    x = oracle.generate_f16(n, 5, oracle.DIST_UNIFORM)
+    cs = np.cumsum(as_f(x, np.float32), dtype=np.float32)
+    assert np.array_equal(oracle.full_scan_ref(x), cs.astype(np.float16).view(np.uint16))
+    assert oracle.full_reduce_ref(x)[0] == cs[-1:].astype(np.float16).view(np.uint16)[0]
+
+
+@pytest.mark.parametrize("seg", SEGS)
+def test_f64_definition_matches_fsum_and_numpy(oracle, seg):
+    n = 1 << 16
+    nseg = n // seg
+    x = oracle.generate_f16(n, 9, oracle.DIST_UNIFORM)
+    xd = as_f(x, np.float64).reshape(nseg, seg)
+    red = oracle.seg_reduce_f64(x, nseg, seg)
+    exact = np.array([math.fsum(row) for row in xd])
+    # fp16 values are multiples of 2^-24 below 1 in magnitude: fp64 sums of <= 2^14 of
+    # them are exact, so the sequential fp64 sum must equal the exactly rounded sum
+    assert np.array_equal(red, exact)
+    sc = oracle.seg_scan_f64(x, nseg, seg)
+    assert np.array_equal(sc.reshape(nseg, seg), np.cumsum(xd, axis=1))
+    assert np.array_equal(sc.reshape(nseg, seg)[:, -1], red)
+
+
+@pytest.mark.parametrize("seg", SEGS)
+def test_reference_fixture_closed_form(oracle, seg):
+    nseg = 8
+    x = oracle.fill_f16(nseg * seg, 0.001)
+    red64 = oracle.seg_reduce_f64(x, nseg, seg)
+    assert np.array_equal(red64, np.full(nseg, seg * C))  # exact in fp64
+    sc64 = oracle.seg_scan_f64(x, nseg, seg).reshape(nseg, seg)
+    assert np.array_equal(sc64, np.tile((np.arange(seg) + 1) * C, (nseg, 1)))
+    red = as_f(oracle.seg_reduce_ref(x, nseg, seg), np.float64)
+    sc = as_f(oracle.seg_scan_ref(x, nseg, seg), np.float64).reshape(nseg, seg)
+    assert np.all(np.abs(red - seg * C) <= 0.001 * max(1.0, seg * C))  # CUB/Thrust tolerance (relative above 1)
+    assert np.all(np.abs(red - seg * C) <= 0.1)                       # WMMA reduce tolerance
+    assert np.all(np.abs(sc - (np.arange(seg) + 1) * C) <= 0.01)       # WMMA scan tolerance
+
+
+@pytest.mark.parametrize("seg", [16, 256, 4096, 8192])
+def test_exact_grid_inputs_are_bitwise_determined(oracle, seg):
+    # k/2048 inputs: every partial sum is a multiple of 2^-11 below 2^13, exact in fp32,
+    # so the fp32 path and the fp64 definition must agree bit for bit after one rounding
+    n = 1 << 16
+    nseg = n // seg
+    x = oracle.generate_f16(n, 21, oracle.DIST_GRID)
+    sc64 = oracle.seg_scan_f64(x, nseg, seg)
+    want = sc64.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.seg_scan_ref(x, nseg, seg), want)
+    assert np.array_equal(oracle.seg_reduce_ref(x, nseg, seg), want.reshape(nseg, seg)[:, -1])
+    assert all(oracle.f64_to_f16(v) == w for v, w in zip(sc64[:2000].tolist(), want[:2000].tolist()))
+
+
+def test_structural_identities(oracle):
+    seg, nseg = 64, 32
+    z = np.zeros(seg * nseg, dtype=np.uint16)
+    assert not oracle.seg_reduce_ref(z, nseg, seg).any() and not oracle.seg_scan_ref(z, nseg, seg).any()
+    one_hot = z.copy()
+    one_hot[5 * seg + 17] = 0x3C00  # 1.0 in segment 5, position 17
+    sc = as_f(oracle.seg_scan_ref(one_hot, nseg, seg), np.float32).reshape(nseg, seg)
+    want = np.zeros((nseg, seg), np.float32)
+    want[5, 17:] = 1.0
+    assert np.array_equal(sc, want)
+    red = as_f(oracle.seg_reduce_ref(one_hot, nseg, seg), np.float32)
+    assert red[5] == 1.0 and red.sum() == 1.0
+    # a change in one segment leaves all others bit-identical
+    x = oracle.generate_f16(seg * nseg, 2, oracle.DIST_UNIFORM)
+    y = x.copy()
+    y[7 * seg + 3] ^= 0x0100
+    a, b = oracle.seg_scan_ref(x, nseg, seg).reshape(nseg, seg), oracle.seg_scan_ref(y, nseg, seg).reshape(nseg, seg)
+    assert np.array_equal(np.delete(a, 7, 0), np.delete(b, 7, 0)) and not np.array_equal(a[7], b[7])
+    # zero segments / zero-length is a no-op
+    assert oracle.seg_reduce_ref(x, 0, seg).size == 0 and oracle.seg_scan_ref(x, 0, seg).size == 0
+
+
+def test_add_partial_sums(oracle):
+    seg, nseg = 32, 9
+    out = oracle.generate_f16(seg * nseg, 4, oracle.DIST_UNIFORM)
+    ps = oracle.generate_f16(nseg, 6, oracle.DIST_UNIFORM)
+    got = oracle.add_partial_sums_ref(out, ps, nseg, seg)
+    want = (as_f(out, np.float32).reshape(nseg, seg) + as_f(ps, np.float32)[:, None]).astype(np.float16)
+    assert np.array_equal(got, want.view(np.uint16).ravel())
+
+
+def test_tolerance_rule(oracle):
+    ref = np.array([1.0, 1.0, 1.0, 100.0, 70000.0, 70000.0, -70000.0, 65400.0, 0.0])
+    f = lambda v: np.array([v], np.float16).view(np.uint16)[0]
+    got = np.array([f(1.0), f(1.0 + 2 * 2 ** -10), f(1.0 + 4 * 2 ** -10), f(100.0), 0x7C00, f(65504.0), 0xFC00, 0x7C00, 0x7E00], np.uint16)
+    bad, worst, first = oracle.check_f16(got, ref, 1, ulps=2.0, abs_per_sqrt=0.0)
+    # violations: +4ulp, finite where inf is due, inf where 65400 is due, NaN
+    assert bad == 4 and first == 2 and worst == float("inf")
+    # the sqrt(segment) slack admits the 4-ulp error
+    bad, _, _ = oracle.check_f16(got[:4], ref[:4], 16, ulps=2.0, abs_per_sqrt=1e-3)
+    assert bad == 0
+    bad, _, fb = oracle.check_f32_rel(np.float32([1.0, 2.0, 0.0]), np.array([1.005, 2.5, 1e-9]), 1e-2, 1.0)
+    assert bad == 1 and fb == 1
+
+
+def test_gemv_gemm_f64_against_numpy(oracle):
+    M, N, K = 48, 40, 96
+    A = oracle.generate_f16(M * K, 1, oracle.DIST_NORMAL)
+    B = oracle.generate_f16(N * K, 2, oracle.DIST_NORMAL)  # N rows of K: column-major K x N
+    x = oracle.generate_f16(K, 3, oracle.DIST_NORMAL)
+    Ad, Bd, xd = as_f(A, np.float64).reshape(M, K), as_f(B, np.float64).reshape(N, K), as_f(x, np.float64)
+    y0 = np.linspace(-1, 1, M).astype(np.float32)
+    np.testing.assert_allclose(oracle.gemv_f64(A, x, M, K), Ad @ xd, rtol=1e-13, atol=1e-13)
+    np.testing.assert_allclose(oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0), 1.5 * (Ad @ xd) - 0.5 * y0.astype(np.float64), rtol=1e-13, atol=1e-13)
+    Cm = np.arange(M * N, dtype=np.float32).reshape(M, N) / 7
+    np.testing.assert_allclose(oracle.gemm_f64(A, B, M, N, K), Ad @ Bd.T, rtol=1e-13, atol=1e-12)
+    np.testing.assert_allclose(oracle.gemm_f64(A, B, M, N, K, 1.1, 1.2, Cm, row0=8, rows=16), (1.1 * (Ad @ Bd.T) + 1.2 * Cm.astype(np.float64))[8:24], rtol=1e-13, atol=1e-12)
+    # integer-valued inputs (the reference's rand()%3 fill, src/gemm/wmma.cu:110-127): exact
+    Ai = oracle.generate_f16(M * K, 5, oracle.DIST_SMALLINT)
+    Bi = oracle.generate_f16(N * K, 6, oracle.DIST_SMALLINT)
+    want = as_f(Ai, np.int64).reshape(M, K) @ as_f(Bi, np.int64).reshape(N, K).T
+    assert np.array_equal(oracle.gemm_f64(Ai, Bi, M, N, K), want.astype(np.float64))
+    # a transposed B operand would fail this: B is not symmetric in shape (N != K)
