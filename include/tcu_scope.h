@@ -1,0 +1,182 @@
+/*
+ * tcu_scope_amd — C ABI of the MI355X (gfx950) implementation of the tcu_scope hot path:
+ * fp16 segmented / full reduction and inclusive prefix sum (as contractions against
+ * constant ones / triangular matrices on MFMA, and as DPP / LDS wave and block
+ * collectives), and the fp16 GEMV / GEMM kernels.
+ *
+ * The reference (c3sr/tcu_scope) has no FFI layer; its boundary is the set of device
+ * kernels its benchmark harnesses launch, all of the form
+ *     kernel<<<grid, WARPS_PER_BLOCK*32>>>(const half *d_in, half *d_out, size_t num_segments)
+ * with the segment size, tiles/segments per warp and warps per block as template
+ * arguments.  Each entry point below replaces one such family; the template arguments
+ * become run-time arguments.
+ *
+ * Conventions
+ *   - every pointer named d_* is DEVICE memory owned by the caller; nothing here
+ *     allocates, frees or retains it.  Reduction/scan inputs and outputs must be
+ *     16-byte aligned unless the variant is TCU_VARIANT_AUTO.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
+ *     enqueue work; they do not synchronise.
+ *   - the return value is a tcu_status; on failure tcu_last_error() describes it (per
+ *     host thread).  TCU_ERR_UNSUPPORTED is what the reference's harness turns into
+ *     state.SkipWithError (e.g. "segment size must be 16").
+ *   - thread-compatible: concurrent calls must use different streams and, where a
+ *     workspace is taken, different workspaces.
+ *   - results: fp32 accumulation, one round-to-nearest-even conversion to fp16.
+ */
+#ifndef TCU_SCOPE_H
+#define TCU_SCOPE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TCU_SCOPE_ABI_VERSION 1
+
+typedef enum {
+  TCU_OK = 0,
+  TCU_ERR_INVALID_ARG = 1, /* null pointer, misalignment, bad enumerator, overflow */
+  TCU_ERR_UNSUPPORTED = 2, /* (variant, size) pair this kernel family does not cover */
+  TCU_ERR_RUNTIME = 3,     /* a HIP call failed; tcu_last_error() carries hipGetErrorString */
+  TCU_ERR_WORKSPACE = 4    /* workspace missing or smaller than the size query reports */
+} tcu_status;
+
+/* Kernel families.  The MFMA_* values keep the reference's naming of its WMMA kernels
+ * (one per benchmark family); WAVE_SHUFFLE and BLOCK_LDS are the counterparts of its
+ * cub::Warp* and cub::Block* comparators. */
+typedef enum {
+  TCU_VARIANT_AUTO = 0,            /* fastest measured family for the size; any segment size >= 1 */
+  TCU_VARIANT_MFMA_16 = 1,         /* segment size 16      (reference *_16)          */
+  TCU_VARIANT_MFMA_16N = 2,        /* power of two >= 16   (reference *_16N, _16N_OPT) */
+  TCU_VARIANT_MFMA_16N_BLOCK = 3,  /* >= 512, 16 segments per block (reference *_16N_BLOCK) */
+  TCU_VARIANT_MFMA_256 = 4,        /* segment size 256     (reference *_256)         */
+  TCU_VARIANT_MFMA_256N = 5,       /* power of two >= 256  (reference *_256N)        */
+  TCU_VARIANT_MFMA_256N_BLOCK = 6, /* >= 512, block per segment (reference *_256N_BLOCK) */
+  TCU_VARIANT_WAVE_SHUFFLE = 7,    /* DPP wavefront collectives (reference CUB_WARP_*) */
+  TCU_VARIANT_BLOCK_LDS = 8        /* >= 512, block collectives through LDS (reference CUB_BLOCK_*) */
+} tcu_variant;
+
+/* Strategies of the full-array entry points. */
+typedef enum {
+  TCU_FULL_AUTO = 0,
+  TCU_FULL_SINGLE_PASS = 1, /* one kernel: atomic ticket + carry (reduce), decoupled look-back (scan);
+                               replaces reference *_ATOMIC_W_BLOCK_SYNC / _ATOMIC_BALLOT / _CG */
+  TCU_FULL_MULTI_KERNEL = 2 /* reference "2 kernels" (reduce) / "3 kernels" (scan) sequences */
+} tcu_full_strategy;
+
+typedef enum {
+  TCU_DIST_UNIFORM = 0, /* uniform [-1,1) */
+  TCU_DIST_GRID = 1,    /* k/2048, exact in fp16 */
+  TCU_DIST_NORMAL = 2,  /* N(0,1) */
+  TCU_DIST_SMALLINT = 3 /* {0,1,2} */
+} tcu_dist;
+
+/* ---- library ------------------------------------------------------------------------ */
+
+/* Selects the device and caches its properties.  Replaces reference init_cuda
+ * (src/init/cuda.cpp:23-67): an out-of-range id falls back to device 0 as there. */
+int tcu_init(int device_id);
+const char *tcu_last_error(void);
+int tcu_abi_version(void);
+/* Compute units, wavefront size, LDS bytes per CU, 1 if the device is gfx950. */
+int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int *is_gfx950);
+/* Tuning switches used by the benchmarks: "nontemporal" (0/1, default 1). */
+int tcu_set_option(const char *name, int value);
+
+/* ---- segmented reduction -------------------------------------------------------------- */
+
+/* d_out[j] = fp16( sum of d_in[j*segment_size .. (j+1)*segment_size) ), j < num_segments.
+ * Replaces compute_wmma_segmented_reduction_{16,16n,16n_opt,16n_block,256,256n,256n_block}
+ * (reference src/reduction/kernel.cuh:33-559) and compute_cub_{warp,block}_segmented_reduction
+ * (src/reduction/seg_cub_warp.cu:17-32, seg_cub_block.cu:13-29).
+ * tiles_per_wave: 1 KiB tiles each wave keeps in flight (1,2,4,8; 0 = default) — the
+ * reference's WMMA_TILES_PER_WARP / SEGMENTS_PER_WARP; waves_per_block: 1..16 (0 = default)
+ * — the reference's WARPS_PER_BLOCK. */
+int tcu_seg_reduce_f16(const void *d_in, void *d_out, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
+
+/* ---- segmented inclusive prefix sum ------------------------------------------------------ */
+
+/* d_out[j*S + i] = fp16( d_in[j*S] + ... + d_in[j*S + i] ).  d_totals (may be NULL)
+ * receives the fp16 total of every segment — the `_ps` kernels' partial_sums.
+ * Replaces compute_wmma_segmented_prefixsum_{16,16n,16n_block,16n_opt,256,256_ps,256n,
+ * 256n_ps,256n_block,256n_block_ps} (reference src/prefixsum/kernel.cuh:48-774) and
+ * compute_cub_{warp,block}_segmented_prefixsum (src/prefixsum/seg_cub_warp.cu:17-27,
+ * seg_cub_block.cu:13-51).  In-place (d_out == d_in) is allowed. */
+int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
+
+/* d_out[s*S + i] += d_partial_sums[s]  (one fp16 addition per element).
+ * Replaces add_partial_sums (reference src/prefixsum/kernel.cuh:31-43). */
+int tcu_add_partial_sums_f16(void *d_out, const void *d_partial_sums, size_t num_segments, size_t segment_size, void *stream);
+
+/* ---- full-array reduction and prefix sum ---------------------------------------------------- */
+
+/* Two-phase workspace protocol (as the reference uses cub's, src/reduction/wmma_2kers.cu:49-53):
+ * call with d_workspace == NULL to receive the byte count in *workspace_bytes, then again
+ * with a device buffer of at least that size (256-byte aligned).  The workspace needs no
+ * initialisation; its contents are scratch.
+ * segment_size is the tile each block/wave reduces before the cross-block step (the
+ * reference's SEGMENT_SIZE template argument of the *_2KERS_* / *_3KERS / *_ATOMIC_*
+ * benchmarks); 0 = default. */
+
+/* d_out[0] = fp16(sum of all n elements).  Replaces compute_wmma_reduction_cg /
+ * _atomic_w_syncthreads / _atomic_w_atomicballot (reference src/reduction/kernel.cuh:564-786)
+ * and the segmented-kernel + cub::DeviceReduce sequence (src/reduction/wmma_2kers.cu:63-88). */
+int tcu_full_reduce_f16(const void *d_in, void *d_out, size_t n, void *d_workspace, size_t *workspace_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream);
+
+/* d_out[i] = fp16(d_in[0] + ... + d_in[i]).  Replaces compute_wmma_prefixsum_cg /
+ * _atomic_w_atomicballot (reference src/prefixsum/kernel.cuh:779-972) and the 3-kernel
+ * sequence (src/prefixsum/wmma_3kers.cu:60-82). */
+int tcu_full_scan_f16(const void *d_in, void *d_out, size_t n, void *d_workspace, size_t *workspace_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream);
+
+/* ---- dense contractions -------------------------------------------------------------------- */
+
+/* y = alpha * A x + beta * y.  A: M x K row-major fp16, x: K fp16, y: M fp32.
+ * Replaces compute_wmma_gemv_naive / compute_wmma_gemv_sharedmem (reference
+ * src/gemv/wmma_naive.cu:29-94, wmma_sharedmem.cu:43-137); note the reference stores A
+ * column-major and returns y as column 0 of an M x 16 matrix.
+ * variant: TCU_VARIANT_AUTO, TCU_VARIANT_WAVE_SHUFFLE (dot products + DPP) or
+ * TCU_VARIANT_MFMA_16N (16-row strips on MFMA with x as a replicated B operand). */
+int tcu_gemv_f16_f32(const void *d_A, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, int variant, void *stream);
+
+/* D = alpha * A B + beta * C.  A: M x K row-major fp16; B: K x N column-major fp16
+ * (element (k,n) at d_B[n*K + k]); C, D: M x N row-major fp32 (C may equal D, may be
+ * NULL when beta == 0).  Operand layouts of reference compute_gemm (src/gemm/wmma.cu:15-18,
+ * 171-365).  variant: TCU_VARIANT_AUTO / TCU_VARIANT_BLOCK_LDS = LDS-tiled MFMA kernel
+ * (reference compute_gemm, compute_gemm_sharedmem); TCU_VARIANT_WAVE_SHUFFLE is not
+ * defined here; TCU_VARIANT_MFMA_16N = one tile per wave straight from global memory
+ * (reference compute_gemm_naive, src/gemm/wmma_naive.cu:33-88). */
+int tcu_gemm_f16_f32(const void *d_A, const void *d_B, const void *d_C, void *d_D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream);
+
+/* ---- fills, conversions, inputs ---------------------------------------------------------------- */
+
+/* d[i] = (half) value.  Replaces cuda_memory_set / setFP16 (reference
+ * src/utils/cuda_helpers.cuh:123-181). */
+int tcu_fill_f16(void *d, float value, size_t n, void *stream);
+/* d_out[i] = (half) d_in[i].  Replaces convertFp32ToFp16 (src/utils/cuda_helpers.cuh:116-121). */
+int tcu_convert_f32_to_f16(void *d_out, const void *d_in, size_t n, void *stream);
+/* Counter-based seeded inputs (element i depends on (seed, first + i) only).  Stands in
+ * for the reference's cuRAND / rand() fills (src/gemm/wmma_naive.cu:177-181,
+ * src/gemm/wmma.cu:110-127), which are not reproducible without cuRAND.  UNIFORM, GRID
+ * and SMALLINT are bit-identical to the host generator used by the tests. */
+int tcu_generate_f16(void *d, size_t n, uint64_t seed, int dist, size_t first, void *stream);
+
+/* ---- measurement aids ---------------------------------------------------------------------------- */
+
+/* Plain streaming kernels with the same access shape as the reductions/scans: mode 0
+ * copies `bytes` from d_src to d_dst, mode 1 only reads d_src (one word per block is
+ * written to d_dst), mode 2 only writes d_dst.  Used to calibrate hardware counters and
+ * to report what fraction of peak a pure copy reaches.  bytes must be a multiple of 16. */
+int tcu_stream_probe(void *d_dst, const void *d_src, size_t bytes, int mode, int tiles_per_wave, int waves_per_block, void *stream);
+/* Runs every cross-lane primitive the kernels rely on (MFMA 16x16x32 / 32x32x16 operand
+ * layouts, DPP controls, lane swaps) on lane-indexed inputs and writes the raw results
+ * to d_out (fp32 / u32 words; see tcu_scope_amd/csrc/probe.hpp for the record layout).
+ * *out_words receives the number of 32-bit words (call with d_out == NULL to query). */
+int tcu_lane_probe(void *d_out, size_t *out_words, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TCU_SCOPE_H */

@@ -95,10 +95,31 @@ def splitmix64(seed, i):
     return lib().tcu_oracle_splitmix64(seed & 0xFFFFFFFFFFFFFFFF, i)
 
 
+_THREADS = min(16, os.cpu_count() or 1)
+_PAR_MIN = 1 << 22
+
+
+def _split(n_items, fn):
+    """Runs fn(lo, hi) over contiguous pieces of range(n_items) on a few threads (the C
+    functions release the GIL; every piece is computed independently, so results do not
+    depend on the split)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    t = _THREADS
+    bounds = [n_items * i // t for i in range(t + 1)]
+    with ThreadPoolExecutor(t) as ex:
+        list(ex.map(lambda i: fn(bounds[i], bounds[i + 1]), range(t)))
+
+
 def generate_f16(n, seed, dist=DIST_UNIFORM, first=0):
     """n fp16 bit patterns (uint16) of the counter-based generator."""
     out = np.empty(n, dtype=np.uint16)
-    lib().tcu_oracle_generate_f16_range(_p(out, ctypes.c_uint16), first, n, seed & 0xFFFFFFFFFFFFFFFF, dist)
+    L = lib()
+    seed &= 0xFFFFFFFFFFFFFFFF
+    if n >= _PAR_MIN:
+        _split(n, lambda lo, hi: L.tcu_oracle_generate_f16_range(_p(out[lo:hi], ctypes.c_uint16), first + lo, hi - lo, seed, dist))
+    else:
+        L.tcu_oracle_generate_f16_range(_p(out, ctypes.c_uint16), first, n, seed, dist)
     return out
 
 
@@ -155,7 +176,11 @@ def seg_reduce_f64(x, num_segments, segment_size):
     x = _u16(x)
     assert x.size >= num_segments * segment_size
     out = np.empty(num_segments, dtype=np.float64)
-    lib().tcu_oracle_seg_reduce_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), num_segments, segment_size)
+    L, S = lib(), segment_size
+    if num_segments * S >= _PAR_MIN and num_segments >= 64:
+        _split(num_segments, lambda lo, hi: L.tcu_oracle_seg_reduce_f64(_p(x[lo * S:], ctypes.c_uint16), _p(out[lo:], ctypes.c_double), hi - lo, S))
+    else:
+        L.tcu_oracle_seg_reduce_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), num_segments, S)
     return out
 
 
@@ -163,7 +188,11 @@ def seg_scan_f64(x, num_segments, segment_size):
     x = _u16(x)
     assert x.size >= num_segments * segment_size
     out = np.empty(num_segments * segment_size, dtype=np.float64)
-    lib().tcu_oracle_seg_scan_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), num_segments, segment_size)
+    L, S = lib(), segment_size
+    if num_segments * S >= _PAR_MIN and num_segments >= 64:
+        _split(num_segments, lambda lo, hi: L.tcu_oracle_seg_scan_f64(_p(x[lo * S:], ctypes.c_uint16), _p(out[lo * S:], ctypes.c_double), hi - lo, S))
+    else:
+        L.tcu_oracle_seg_scan_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), num_segments, S)
     return out
 
 
@@ -198,9 +227,20 @@ def check_f16(got, ref, segment_size, ulps=2.0, abs_per_sqrt=1e-3):
     got = _u16(got).ravel()
     ref = np.ascontiguousarray(ref, dtype=np.float64).ravel()
     assert got.size == ref.size, (got.size, ref.size)
+    L = lib()
+    if got.size >= _PAR_MIN:
+        res = []
+
+        def piece(lo, hi):
+            w, f = ctypes.c_double(), ctypes.c_size_t()
+            b = L.tcu_oracle_check_f16(_p(got[lo:hi], ctypes.c_uint16), _p(ref[lo:hi], ctypes.c_double), hi - lo, ulps, abs_per_sqrt, segment_size, ctypes.byref(w), ctypes.byref(f))
+            res.append((b, w.value, lo + f.value if b else got.size))
+
+        _split(got.size, piece)
+        return sum(r[0] for r in res), max(r[1] for r in res), min(r[2] for r in res)
     worst = ctypes.c_double()
     fb = ctypes.c_size_t()
-    bad = lib().tcu_oracle_check_f16(_p(got, ctypes.c_uint16), _p(ref, ctypes.c_double), got.size, ulps, abs_per_sqrt, segment_size, ctypes.byref(worst), ctypes.byref(fb))
+    bad = L.tcu_oracle_check_f16(_p(got, ctypes.c_uint16), _p(ref, ctypes.c_double), got.size, ulps, abs_per_sqrt, segment_size, ctypes.byref(worst), ctypes.byref(fb))
     return bad, worst.value, fb.value
 
 

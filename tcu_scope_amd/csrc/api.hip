@@ -1,0 +1,140 @@
+// C ABI of libtcu_scope_amd.so (declared in include/tcu_scope.h): thin wrappers that
+// validate, pick a kernel (dispatch.hpp) and report launch errors.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "dispatch.hpp"
+
+namespace {
+
+struct DeviceState {
+  bool initialised = false;
+  int device = 0;
+  int compute_units = 0;
+  int wavefront = 0;
+  int lds_bytes = 0;
+  bool gfx950 = false;
+};
+DeviceState &state() {
+  static DeviceState s;
+  return s;
+}
+
+int runtime_error(const char *what, hipError_t e) { return tcu::fail(TCU_ERR_RUNTIME, std::string(what) + ": " + hipGetErrorString(e)); }
+
+// Kernel launches are asynchronous; what can be caught here is a launch that the runtime
+// rejected (bad configuration, no code object for the device).
+int after_launch(const char *what, unsigned long launches_before, int rc) {
+  if (rc != TCU_OK || tcu::launch_count() == launches_before) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return runtime_error(what, e);
+  return TCU_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tcu_abi_version(void) { return TCU_SCOPE_ABI_VERSION; }
+
+const char *tcu_last_error(void) { return tcu::last_error_string().c_str(); }
+
+int tcu_init(int device_id) {
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess) return runtime_error("tcu_init: hipGetDeviceCount", e);
+  if (count <= 0) return tcu::fail(TCU_ERR_RUNTIME, "tcu_init: no HIP device");
+  if (device_id < 0 || device_id >= count) device_id = 0;  // as the reference does for --cuda_device_id
+  e = hipSetDevice(device_id);
+  if (e != hipSuccess) return runtime_error("tcu_init: hipSetDevice", e);
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, device_id);
+  if (e != hipSuccess) return runtime_error("tcu_init: hipGetDeviceProperties", e);
+  DeviceState &s = state();
+  s.device = device_id;
+  s.compute_units = prop.multiProcessorCount;
+  s.wavefront = prop.warpSize;
+  s.lds_bytes = (int)prop.sharedMemPerBlock;
+  s.gfx950 = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+  s.initialised = true;
+  if (!s.gfx950) return tcu::fail(TCU_ERR_UNSUPPORTED, std::string("tcu_init: this library is built for gfx950 only, device is ") + prop.gcnArchName);
+  return TCU_OK;
+}
+
+int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int *is_gfx950) {
+  DeviceState &s = state();
+  if (!s.initialised) {
+    int rc = tcu_init(0);
+    if (rc != TCU_OK && rc != TCU_ERR_UNSUPPORTED) return rc;
+  }
+  if (compute_units) *compute_units = s.compute_units;
+  if (wavefront_size) *wavefront_size = s.wavefront;
+  if (lds_bytes) *lds_bytes = s.lds_bytes;
+  if (is_gfx950) *is_gfx950 = s.gfx950 ? 1 : 0;
+  return TCU_OK;
+}
+
+int tcu_set_option(const char *name, int value) {
+  if (!name) return tcu::fail(TCU_ERR_INVALID_ARG, "tcu_set_option: null name");
+  if (std::strcmp(name, "nontemporal") == 0) {
+    tcu::options().nontemporal = value != 0;
+    return TCU_OK;
+  }
+  return tcu::fail(TCU_ERR_INVALID_ARG, std::string("tcu_set_option: unknown option ") + name);
+}
+
+int tcu_seg_reduce_f16(const void *d_in, void *d_out, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_seg_reduce_f16", before, tcu::seg_reduce_dispatch(d_in, d_out, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, stream));
+}
+
+int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_seg_scan_f16", before, tcu::seg_scan_dispatch(d_in, d_out, d_totals, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, stream));
+}
+
+int tcu_add_partial_sums_f16(void *d_out, const void *d_partial_sums, size_t num_segments, size_t segment_size, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_add_partial_sums_f16", before, tcu::add_partial_sums_dispatch(d_out, d_partial_sums, num_segments, segment_size, stream));
+}
+
+int tcu_full_reduce_f16(const void *d_in, void *d_out, size_t n, void *d_workspace, size_t *workspace_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_full_reduce_f16", before, tcu::full_reduce_dispatch(d_in, d_out, n, d_workspace, workspace_bytes, strategy, segment_size, waves_per_block, stream));
+}
+
+int tcu_full_scan_f16(const void *d_in, void *d_out, size_t n, void *d_workspace, size_t *workspace_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_full_scan_f16", before, tcu::full_scan_dispatch(d_in, d_out, n, d_workspace, workspace_bytes, strategy, segment_size, waves_per_block, stream));
+}
+
+int tcu_gemv_f16_f32(const void *d_A, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_gemv_f16_f32", before, tcu::gemv_dispatch(d_A, d_x, d_y, M, K, alpha, beta, variant, stream));
+}
+
+int tcu_gemm_f16_f32(const void *d_A, const void *d_B, const void *d_C, void *d_D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_gemm_f16_f32", before, tcu::gemm_dispatch(d_A, d_B, d_C, d_D, M, N, K, alpha, beta, variant, stream));
+}
+
+int tcu_fill_f16(void *d, float value, size_t n, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_fill_f16", before, tcu::fill_dispatch(d, value, n, stream)); }
+
+int tcu_convert_f32_to_f16(void *d_out, const void *d_in, size_t n, void *stream) { const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_convert_f32_to_f16", before, tcu::convert_dispatch(d_out, d_in, n, stream)); }
+
+int tcu_generate_f16(void *d, size_t n, uint64_t seed, int dist, size_t first, void *stream) { const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_generate_f16", before, tcu::generate_dispatch(d, n, seed, dist, first, stream)); }
+
+int tcu_stream_probe(void *d_dst, const void *d_src, size_t bytes, int mode, int tiles_per_wave, int waves_per_block, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_stream_probe", before, tcu::stream_probe_dispatch(d_dst, d_src, bytes, mode, tiles_per_wave, waves_per_block, stream));
+}
+
+int tcu_lane_probe(void *d_out, size_t *out_words, void *stream) { const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_lane_probe", before, tcu::lane_probe_dispatch(d_out, out_words, stream)); }
+
+}  // extern "C"

@@ -1,0 +1,591 @@
+// Host-side argument validation and kernel selection for the C entry points.
+// Mirrors the preconditions of the reference's harnesses (segment-size checks ->
+// "unsupported", num_elements % segment_size, grid limits: reference
+// src/reduction/seg_wmma_16.cu:16-18, seg_wmma_16n.cu:17-22,44-49,
+// src/reduction/wmma_2kers.cu:23-26).
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include <string>
+
+#include "../../include/tcu_scope.h"
+#include "launch.hpp"
+#include "seg_reduce.hpp"
+#include "seg_scan.hpp"
+#include "full_array.hpp"
+#include "gemv.hpp"
+#include "gemm.hpp"
+#include "util_kernels.hpp"
+
+namespace tcu {
+
+inline std::string &last_error_string() {
+  static thread_local std::string s;
+  return s;
+}
+inline int fail(int code, const std::string &msg) {
+  last_error_string() = msg;
+  return code;
+}
+
+struct Options {
+  bool nontemporal = true;
+};
+inline Options &options() {
+  static Options o;
+  return o;
+}
+
+inline bool is_pow2(size_t x) { return x && !(x & (x - 1)); }
+inline int ilog2(size_t x) {
+  int l = 0;
+  while (x > 1) {
+    x >>= 1;
+    l++;
+  }
+  return l;
+}
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr size_t kMaxGrid = 0x7fffffffu;
+
+struct SegArgs {
+  size_t num_segments, segment_size;
+  int variant, tiles_per_wave, waves_per_block;
+  bool mfma;
+};
+
+// Common validation for the segmented entry points.  On success `a` holds defaults
+// resolved and *generic says whether only the scalar kernel applies.
+inline int validate_segmented(const char *what, const void *in, const void *out, SegArgs &a, bool *generic) {
+  *generic = false;
+  if (a.segment_size == 0) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": segment_size must be positive");
+  if (a.num_segments != 0 && (in == nullptr || out == nullptr)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  if (a.num_segments > ((size_t)1 << 62) / a.segment_size) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": num_segments * segment_size overflows");
+  if (a.variant < TCU_VARIANT_AUTO || a.variant > TCU_VARIANT_BLOCK_LDS) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown variant");
+  const int u = a.tiles_per_wave, w = a.waves_per_block;
+  if (!(u == 0 || u == 1 || u == 2 || u == 4 || u == 8)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": tiles_per_wave must be 0 (default), 1, 2, 4 or 8");
+  if (!(w == 0 || w == 1 || w == 2 || w == 4 || w == 8 || w == 16)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": waves_per_block must be 0 (default), 1, 2, 4, 8 or 16");
+  const size_t S = a.segment_size;
+  const bool fast_ok = is_pow2(S) && S >= 16 && aligned16(in) && aligned16(out);
+  switch (a.variant) {
+    case TCU_VARIANT_AUTO:
+      if (!fast_ok) *generic = true;
+      break;
+    case TCU_VARIANT_MFMA_16:
+      if (S != 16) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment size must be 16");
+      break;
+    case TCU_VARIANT_MFMA_256:
+      if (S != 256) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment size must be 256");
+      break;
+    case TCU_VARIANT_MFMA_256N:
+      if (!is_pow2(S) || S < 256) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment size must be a power-of-two multiple of 256");
+      break;
+    case TCU_VARIANT_MFMA_16N_BLOCK:
+    case TCU_VARIANT_MFMA_256N_BLOCK:
+    case TCU_VARIANT_BLOCK_LDS:
+      if (!is_pow2(S) || S < 512) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": block-per-segment variants need a power-of-two segment size >= 512");
+      break;
+    default:
+      if (!is_pow2(S) || S < 16) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment size must be a power of two >= 16");
+  }
+  if (a.variant != TCU_VARIANT_AUTO && !(aligned16(in) && aligned16(out))) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": device pointers must be 16-byte aligned");
+  a.mfma = a.variant >= TCU_VARIANT_MFMA_16 && a.variant <= TCU_VARIANT_MFMA_256N_BLOCK;
+  return TCU_OK;
+}
+
+inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || v == TCU_VARIANT_MFMA_256N_BLOCK || v == TCU_VARIANT_BLOCK_LDS; }
+
+// ----- segmented reduction ----------------------------------------------------------------
+
+template <int LPS_LOG2, int U, bool MFMA>
+inline void launch_reduce_small(unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg) {
+  if (options().nontemporal)
+    launch(seg_reduce_small_kernel<LPS_LOG2, U, MFMA, true>, grid, block, stream, in, out, n_chunks, nseg);
+  else
+    launch(seg_reduce_small_kernel<LPS_LOG2, U, MFMA, false>, grid, block, stream, in, out, n_chunks, nseg);
+}
+template <int LPS_LOG2, bool MFMA>
+inline void launch_reduce_small_u(int u, unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg) {
+  switch (u) {
+    case 1: return launch_reduce_small<LPS_LOG2, 1, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
+    case 2: return launch_reduce_small<LPS_LOG2, 2, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
+    case 4: return launch_reduce_small<LPS_LOG2, 4, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
+    default: return launch_reduce_small<LPS_LOG2, 8, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
+  }
+}
+template <bool MFMA>
+inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg) {
+  switch (lps_log2) {
+    case 1: return launch_reduce_small_u<1, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
+    case 2: return launch_reduce_small_u<2, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
+    case 3: return launch_reduce_small_u<3, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
+    case 4: return launch_reduce_small_u<4, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
+    case 5: return launch_reduce_small_u<5, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
+    default: return launch_reduce_small_u<6, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
+  }
+}
+
+#define TCU_SWITCH_U_MFMA_NT(KERNEL, u, mfma, nt, ...)                    \
+  do {                                                                     \
+    const int _k = ((u) == 1 ? 0 : (u) == 2 ? 1 : (u) == 4 ? 2 : 3) * 4 + ((mfma) ? 2 : 0) + ((nt) ? 1 : 0); \
+    switch (_k) {                                                          \
+      case 0: launch(KERNEL<1, false, false>, __VA_ARGS__); break;         \
+      case 1: launch(KERNEL<1, false, true>, __VA_ARGS__); break;          \
+      case 2: launch(KERNEL<1, true, false>, __VA_ARGS__); break;          \
+      case 3: launch(KERNEL<1, true, true>, __VA_ARGS__); break;           \
+      case 4: launch(KERNEL<2, false, false>, __VA_ARGS__); break;         \
+      case 5: launch(KERNEL<2, false, true>, __VA_ARGS__); break;          \
+      case 6: launch(KERNEL<2, true, false>, __VA_ARGS__); break;          \
+      case 7: launch(KERNEL<2, true, true>, __VA_ARGS__); break;           \
+      case 8: launch(KERNEL<4, false, false>, __VA_ARGS__); break;         \
+      case 9: launch(KERNEL<4, false, true>, __VA_ARGS__); break;          \
+      case 10: launch(KERNEL<4, true, false>, __VA_ARGS__); break;         \
+      case 11: launch(KERNEL<4, true, true>, __VA_ARGS__); break;          \
+      case 12: launch(KERNEL<8, false, false>, __VA_ARGS__); break;        \
+      case 13: launch(KERNEL<8, false, true>, __VA_ARGS__); break;         \
+      case 14: launch(KERNEL<8, true, false>, __VA_ARGS__); break;         \
+      default: launch(KERNEL<8, true, true>, __VA_ARGS__); break;          \
+    }                                                                      \
+  } while (0)
+
+inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
+  SegArgs a{num_segments, segment_size, variant, tiles_per_wave, waves_per_block, false};
+  bool generic = false;
+  if (int rc = validate_segmented("tcu_seg_reduce_f16", d_in, d_out, a, &generic)) return rc;
+  if (num_segments == 0) return TCU_OK;
+  const size_t S = segment_size, N = num_segments * S;
+  const int wpb = waves_per_block ? waves_per_block : 4;
+  const unsigned block = (unsigned)wpb * 64u;
+  const half8_t *in = static_cast<const half8_t *>(d_in);
+  uint16_t *out = static_cast<uint16_t *>(d_out);
+  const bool nt = options().nontemporal;
+
+  if (generic) {
+    const size_t grid = (num_segments + wpb - 1) / wpb;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
+    launch(seg_reduce_generic_kernel, (unsigned)grid, block, stream, static_cast<const uint16_t *>(d_in), out, num_segments, S);
+    return TCU_OK;
+  }
+  const size_t n_chunks = N / 8;
+  int u = tiles_per_wave ? tiles_per_wave : 8;
+
+  if (is_block_variant(variant)) {
+    const size_t tiles_per_seg = S / kTileHalves;
+    const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;  // the reference's 16n_block owns 16 segments per block
+    const size_t grid = (num_segments + spb - 1) / spb;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
+    TCU_SWITCH_U_MFMA_NT(seg_reduce_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tiles_per_seg, spb);
+    return TCU_OK;
+  }
+  if (S <= 512) {
+    const size_t tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
+    const size_t waves = (tiles + u - 1) / u;
+    const size_t grid = (waves + wpb - 1) / wpb;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
+    const int lps_log2 = ilog2(S) - 3;
+    if (a.mfma)
+      launch_reduce_small_s<true>(lps_log2, u, (unsigned)grid, block, stream, in, out, n_chunks, num_segments);
+    else
+      launch_reduce_small_s<false>(lps_log2, u, (unsigned)grid, block, stream, in, out, n_chunks, num_segments);
+    return TCU_OK;
+  }
+  // S >= 1024: each wave walks max(S, u tiles) of data
+  const int tps_log2 = ilog2(S) - 9;
+  const size_t tiles_per_seg = (size_t)1 << tps_log2;
+  const size_t tiles = num_segments * tiles_per_seg;
+  const size_t iters = tiles_per_seg > (size_t)u ? tiles_per_seg / u : 1;
+  if (iters > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: segment too long for the wave-per-segment kernel; use a block variant");
+  const size_t tiles_per_wave_total = iters * u;
+  const size_t waves = (tiles + tiles_per_wave_total - 1) / tiles_per_wave_total;
+  const size_t grid = (waves + wpb - 1) / wpb;
+  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
+  TCU_SWITCH_U_MFMA_NT(seg_reduce_long_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tps_log2, (unsigned)iters);
+  return TCU_OK;
+}
+
+// ----- segmented inclusive prefix sum -------------------------------------------------------
+
+template <int LPS_LOG2, bool MFMA>
+inline void launch_scan_wave_u(int u, bool nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg, int tps_log2,
+                               unsigned iters) {
+#define TCU_SCAN_CASE(UU)                                                                                                          \
+  if (nt)                                                                                                                          \
+    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, true>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters); \
+  else                                                                                                                             \
+    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, false>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters); \
+  return
+  switch (u) {
+    case 1: TCU_SCAN_CASE(1);
+    case 2: TCU_SCAN_CASE(2);
+    case 4: TCU_SCAN_CASE(4);
+    default: TCU_SCAN_CASE(8);
+  }
+#undef TCU_SCAN_CASE
+}
+template <bool MFMA>
+inline void launch_scan_wave_s(int lps_log2, int u, bool nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg,
+                               int tps_log2, unsigned iters) {
+  switch (lps_log2) {
+    case 1: return launch_scan_wave_u<1, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
+    case 2: return launch_scan_wave_u<2, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
+    case 3: return launch_scan_wave_u<3, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
+    case 4: return launch_scan_wave_u<4, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
+    case 5: return launch_scan_wave_u<5, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
+    default: return launch_scan_wave_u<6, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
+  }
+}
+
+inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
+  SegArgs a{num_segments, segment_size, variant, tiles_per_wave, waves_per_block, false};
+  bool generic = false;
+  if (int rc = validate_segmented("tcu_seg_scan_f16", d_in, d_out, a, &generic)) return rc;
+  if (num_segments == 0) return TCU_OK;
+  const size_t S = segment_size, N = num_segments * S;
+  const int wpb = waves_per_block ? waves_per_block : 4;
+  const unsigned block = (unsigned)wpb * 64u;
+  const half8_t *in = static_cast<const half8_t *>(d_in);
+  uint4_t *out = static_cast<uint4_t *>(d_out);
+  uint16_t *totals = static_cast<uint16_t *>(d_totals);
+  const bool nt = options().nontemporal;
+
+  if (generic) {
+    const size_t grid = (num_segments + wpb - 1) / wpb;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: grid exceeds the launch limit");
+    launch(seg_scan_generic_kernel, (unsigned)grid, block, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), totals, num_segments, S);
+    return TCU_OK;
+  }
+  const size_t n_chunks = N / 8;
+  const int u = tiles_per_wave ? tiles_per_wave : 4;
+
+  if (is_block_variant(variant)) {
+    const size_t tiles_per_seg = S / kTileHalves;
+    const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;
+    const size_t grid = (num_segments + spb - 1) / spb;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: grid exceeds the launch limit");
+    TCU_SWITCH_U_MFMA_NT(seg_scan_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, spb);
+    return TCU_OK;
+  }
+  int lps_log2, tps_log2 = 0;
+  size_t iters = 1;
+  const size_t tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
+  if (S < 512) {
+    lps_log2 = ilog2(S) - 3;
+  } else {
+    lps_log2 = 6;
+    tps_log2 = ilog2(S) - 9;
+    const size_t tiles_per_seg = (size_t)1 << tps_log2;
+    iters = tiles_per_seg > (size_t)u ? tiles_per_seg / u : 1;
+    if (iters > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: segment too long for the wave-per-segment kernel; use a block variant");
+  }
+  const size_t per_wave = iters * u;
+  const size_t waves = (tiles + per_wave - 1) / per_wave;
+  const size_t grid = (waves + wpb - 1) / wpb;
+  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: grid exceeds the launch limit");
+  if (a.mfma)
+    launch_scan_wave_s<true>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters);
+  else
+    launch_scan_wave_s<false>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters);
+  return TCU_OK;
+}
+
+inline int add_partial_sums_dispatch(void *d_out, const void *d_ps, size_t num_segments, size_t segment_size, void *stream) {
+  if (segment_size == 0) return fail(TCU_ERR_INVALID_ARG, "tcu_add_partial_sums_f16: segment_size must be positive");
+  if (num_segments == 0) return TCU_OK;
+  if (!d_out || !d_ps) return fail(TCU_ERR_INVALID_ARG, "tcu_add_partial_sums_f16: null device pointer");
+  const size_t n = num_segments * segment_size;
+  if (is_pow2(segment_size) && segment_size >= 8 && aligned16(d_out)) {
+    const size_t n_chunks = n / 8;
+    const size_t grid = (n_chunks + 255) / 256;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_add_partial_sums_f16: grid exceeds the launch limit");
+    launch(add_partial_sums_kernel, (unsigned)grid, 256u, stream, static_cast<uint4_t *>(d_out), static_cast<const uint16_t *>(d_ps), n_chunks, ilog2(segment_size) - 3);
+  } else {
+    const size_t grid = (n + 255) / 256;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_add_partial_sums_f16: grid exceeds the launch limit");
+    launch(add_partial_sums_generic_kernel, (unsigned)grid, 256u, stream, static_cast<uint16_t *>(d_out), static_cast<const uint16_t *>(d_ps), n, segment_size);
+  }
+  return TCU_OK;
+}
+
+// ----- full-array reduction / prefix sum ------------------------------------------------------
+
+constexpr size_t kWorkspaceAlign = 256;
+inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct FullPlan {
+  int u, wpb;
+  size_t part_halves;  // halves per block step / partition
+};
+// segment_size = halves one block takes per step (0 = default); must be wpb * u * 512 with u in {1,2,4,8}
+inline int plan_full(const char *what, size_t segment_size, int waves_per_block, size_t default_part, FullPlan *p) {
+  int wpb = waves_per_block ? waves_per_block : 4;
+  if (!(wpb == 1 || wpb == 2 || wpb == 4 || wpb == 8 || wpb == 16)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": waves_per_block must be 0 (default), 1, 2, 4, 8 or 16");
+  size_t part = segment_size ? segment_size : default_part;
+  if (!is_pow2(part) || part < (size_t)wpb * 512) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment_size must be a power of two >= 512 * waves_per_block");
+  size_t u = part / ((size_t)wpb * 512);
+  while (u > 8 && wpb < 16) {  // more data per block than 8 tiles per wave: widen the block
+    wpb *= 2;
+    u /= 2;
+  }
+  if (u > 8) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment_size too large (at most 65536)");
+  p->u = (int)u;
+  p->wpb = wpb;
+  p->part_halves = part;
+  return TCU_OK;
+}
+
+constexpr unsigned kFullReduceMaxBlocks = 2048;
+
+inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d_ws, size_t *ws_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream) {
+  const char *what = "tcu_full_reduce_f16";
+  if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
+  if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
+  if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
+  const bool nt = options().nontemporal;
+  if (strategy == TCU_FULL_SINGLE_PASS) {
+    FullPlan p;
+    if (int rc = plan_full(what, segment_size, waves_per_block, 16384, &p)) return rc;
+    const size_t need = 256 + 4 * (size_t)kFullReduceMaxBlocks;
+    if (!d_ws) {
+      *ws_bytes = need;
+      return TCU_OK;
+    }
+    if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
+    if (!d_out || (n && !d_in)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+    if ((n % 8) != 0 || !aligned16(d_in)) {
+      // odd sizes: one block over scalar loads
+      launch(sum_f16_kernel, 1u, 1024u, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), n);
+      return TCU_OK;
+    }
+    const size_t n_chunks = n / 8;
+    const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
+    size_t grid = (n_tiles + (size_t)p.wpb * p.u - 1) / ((size_t)p.wpb * p.u);
+    if (grid > kFullReduceMaxBlocks) grid = kFullReduceMaxBlocks;
+    if (grid == 0) grid = 1;
+    unsigned *ws = static_cast<unsigned *>(d_ws);
+    launch(zero_words_kernel, 1u, 256u, stream, ws, (size_t)64);
+    TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, false, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws);
+    return TCU_OK;
+  }
+  // the reference's two-kernel sequence: segmented reduction into fp16 totals, then a sum of the totals
+  const size_t S = segment_size ? segment_size : 2048;
+  if (!is_pow2(S) || S < 16) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment_size must be a power of two >= 16");
+  if (n % S != 0) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": num_elements must be a multiple of segment_size");
+  const size_t nseg = n / S;
+  const size_t need = round_up(2 * (nseg ? nseg : 1), kWorkspaceAlign);
+  if (!d_ws) {
+    *ws_bytes = need;
+    return TCU_OK;
+  }
+  if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
+  if (!d_out || (n && !d_in)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  if (int rc = seg_reduce_dispatch(d_in, d_ws, nseg, S, S == 16 ? TCU_VARIANT_MFMA_16 : TCU_VARIANT_MFMA_16N, 0, waves_per_block, stream)) return rc;
+  launch(sum_f16_kernel, 1u, 1024u, stream, static_cast<const uint16_t *>(d_ws), static_cast<uint16_t *>(d_out), nseg);
+  return TCU_OK;
+}
+
+inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_ws, size_t *ws_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream) {
+  const char *what = "tcu_full_scan_f16";
+  if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
+  if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
+  if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
+  const bool nt = options().nontemporal;
+  if (strategy == TCU_FULL_SINGLE_PASS) {
+    FullPlan p;
+    if (int rc = plan_full(what, segment_size, waves_per_block, 8192, &p)) return rc;
+    if (n % 8 != 0 || !aligned16(d_in) || !aligned16(d_out)) {
+      if (!d_ws) {
+        *ws_bytes = kWorkspaceAlign;
+        return TCU_OK;
+      }
+      if (!n) return TCU_OK;
+      if (!d_in || !d_out) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+      launch(seg_scan_generic_kernel, 1u, 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), static_cast<uint16_t *>(nullptr), (size_t)1, n);
+      return TCU_OK;
+    }
+    const size_t n_chunks = n / 8;
+    const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
+    const size_t parts = (n_tiles + (size_t)p.wpb * p.u - 1) / ((size_t)p.wpb * p.u);
+    const size_t need = round_up(256 + 8 * (parts ? parts : 1), kWorkspaceAlign);
+    if (!d_ws) {
+      *ws_bytes = need;
+      return TCU_OK;
+    }
+    if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
+    if (!n) return TCU_OK;
+    if (!d_in || !d_out) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+    if (parts > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    unsigned *ws = static_cast<unsigned *>(d_ws);
+    const size_t words = 64 + 2 * parts;
+    launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
+    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, false, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws);
+    return TCU_OK;
+  }
+  // the reference's three-kernel sequence: segmented scan + totals, exclusive scan of the totals, add
+  const size_t S = segment_size ? segment_size : 2048;
+  if (!is_pow2(S) || S < 256) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment_size must be a power-of-two multiple of 256");
+  if (n % S != 0) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": num_elements must be a multiple of segment_size");
+  const size_t nseg = n / S;
+  const size_t need = round_up(2 * (nseg ? nseg : 1), kWorkspaceAlign);
+  if (!d_ws) {
+    *ws_bytes = need;
+    return TCU_OK;
+  }
+  if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
+  if (!n) return TCU_OK;
+  if (!d_in || !d_out) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  if (int rc = seg_scan_dispatch(d_in, d_out, d_ws, nseg, S, TCU_VARIANT_MFMA_256N, 0, waves_per_block, stream)) return rc;
+  launch(exclusive_scan_f16_kernel, 1u, 1024u, stream, static_cast<uint16_t *>(d_ws), nseg);
+  return add_partial_sums_dispatch(d_out, d_ws, nseg, S, stream);
+}
+
+// ----- GEMV / GEMM -----------------------------------------------------------------------------
+
+inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
+  const char *what = "tcu_gemv_f16_f32";
+  if (!(variant == TCU_VARIANT_AUTO || variant == TCU_VARIANT_WAVE_SHUFFLE || variant == TCU_VARIANT_MFMA_16N)) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": variant must be AUTO, WAVE_SHUFFLE or MFMA_16N");
+  if (M == 0) return TCU_OK;
+  if (!y || (K && (!A || !x))) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  const bool vec_ok = K % 8 == 0 && K > 0 && aligned16(A) && aligned16(x);
+  const bool nt = options().nontemporal;
+  const unsigned block = 256;
+  if (!vec_ok) {
+    if (variant != TCU_VARIANT_AUTO) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": K must be a positive multiple of 8 and A, x 16-byte aligned");
+    const size_t grid = (M + 3) / 4;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    launch(gemv_generic_kernel, (unsigned)grid, block, stream, static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(x), static_cast<float *>(y), M, K, alpha, beta);
+    return TCU_OK;
+  }
+  const half8_t *a = static_cast<const half8_t *>(A), *xv = static_cast<const half8_t *>(x);
+  float *yy = static_cast<float *>(y);
+  if (variant == TCU_VARIANT_MFMA_16N) {
+    const size_t strips = (M + 15) / 16;
+    const size_t grid = (strips + 3) / 4;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    if (nt)
+      launch(gemv_mfma_kernel<true>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+    else
+      launch(gemv_mfma_kernel<false>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+    return TCU_OK;
+  }
+  constexpr int ROWS = 2, UK = 4;
+  const size_t waves = (M + ROWS - 1) / ROWS;
+  const size_t grid = (waves + 3) / 4;
+  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+  if (nt)
+    launch(gemv_dot_kernel<ROWS, UK, true>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+  else
+    launch(gemv_dot_kernel<ROWS, UK, false>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+  return TCU_OK;
+}
+
+inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream) {
+  const char *what = "tcu_gemm_f16_f32";
+  if (!(variant == TCU_VARIANT_AUTO || variant == TCU_VARIANT_BLOCK_LDS || variant == TCU_VARIANT_MFMA_16N)) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": variant must be AUTO, BLOCK_LDS or MFMA_16N");
+  if (M == 0 || N == 0) return TCU_OK;
+  if (!D || (K && (!A || !B)) || (beta != 0.0f && !C)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  const bool al = aligned16(A) && aligned16(B);
+  const bool lds_ok = al && M % kGemmBM == 0 && N % kGemmBN == 0 && K % kGemmBK == 0 && K > 0;
+  const bool direct_ok = al && M % 32 == 0 && N % 32 == 0 && K % 16 == 0 && K > 0;
+  const half8_t *a = static_cast<const half8_t *>(A), *b = static_cast<const half8_t *>(B);
+  const float *c = static_cast<const float *>(C);
+  float *d = static_cast<float *>(D);
+  if (variant == TCU_VARIANT_BLOCK_LDS && !lds_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the LDS kernel needs M, N multiples of 128 and K a multiple of 32");
+  if (variant == TCU_VARIANT_MFMA_16N && !direct_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the direct kernel needs M, N multiples of 32 and K a multiple of 16");
+  if (lds_ok && variant != TCU_VARIANT_MFMA_16N) {
+    const size_t grid = (M / kGemmBM) * (N / kGemmBN);
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    launch(gemm_lds_kernel, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+  } else if (direct_ok) {
+    const size_t tiles = (M / 32) * (N / 32);
+    const size_t grid = (tiles + 3) / 4;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    launch(gemm_direct_kernel, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+  } else {
+    const size_t grid = (M * N + 255) / 256;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    launch(gemm_generic_kernel, (unsigned)grid, 256u, stream, static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B), c, d, M, N, K, alpha, beta);
+  }
+  return TCU_OK;
+}
+
+// ----- fills, conversions, inputs, probes --------------------------------------------------------
+
+inline unsigned fill_grid(size_t n) {
+  size_t g = (n + 255) / 256;
+  return (unsigned)(g > 65536 ? 65536 : (g ? g : 1));
+}
+inline int fill_dispatch(void *d, float value, size_t n, void *stream) {
+  if (!n) return TCU_OK;
+  if (!d) return fail(TCU_ERR_INVALID_ARG, "tcu_fill_f16: null device pointer");
+  launch(fill_f16_kernel, fill_grid(n), 256u, stream, static_cast<uint16_t *>(d), value, n);
+  return TCU_OK;
+}
+inline int convert_dispatch(void *d_out, const void *d_in, size_t n, void *stream) {
+  if (!n) return TCU_OK;
+  if (!d_out || !d_in) return fail(TCU_ERR_INVALID_ARG, "tcu_convert_f32_to_f16: null device pointer");
+  launch(convert_f32_to_f16_kernel, fill_grid(n), 256u, stream, static_cast<uint16_t *>(d_out), static_cast<const float *>(d_in), n);
+  return TCU_OK;
+}
+inline int generate_dispatch(void *d, size_t n, uint64_t seed, int dist, size_t first, void *stream) {
+  if (dist < TCU_DIST_UNIFORM || dist > TCU_DIST_SMALLINT) return fail(TCU_ERR_INVALID_ARG, "tcu_generate_f16: unknown distribution");
+  if (!n) return TCU_OK;
+  if (!d) return fail(TCU_ERR_INVALID_ARG, "tcu_generate_f16: null device pointer");
+  launch(generate_f16_kernel, fill_grid(n), 256u, stream, static_cast<uint16_t *>(d), n, seed, dist, first);
+  return TCU_OK;
+}
+
+template <int U>
+inline void launch_probe(int mode, bool nt, unsigned grid, unsigned block, void *stream, uint4_t *dst, const half8_t *src, size_t n_chunks) {
+#define TCU_PROBE_CASE(MODE)                                                                   \
+  if (nt)                                                                                      \
+    launch(stream_probe_kernel<U, MODE, true>, grid, block, stream, dst, src, n_chunks);       \
+  else                                                                                         \
+    launch(stream_probe_kernel<U, MODE, false>, grid, block, stream, dst, src, n_chunks);      \
+  return
+  switch (mode) {
+    case 0: TCU_PROBE_CASE(0);
+    case 1: TCU_PROBE_CASE(1);
+    default: TCU_PROBE_CASE(2);
+  }
+#undef TCU_PROBE_CASE
+}
+inline int stream_probe_dispatch(void *d_dst, const void *d_src, size_t bytes, int mode, int tiles_per_wave, int waves_per_block, void *stream) {
+  const char *what = "tcu_stream_probe";
+  if (mode < 0 || mode > 2) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": mode must be 0, 1 or 2");
+  if (bytes % 16 != 0) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": bytes must be a multiple of 16");
+  const int u = tiles_per_wave ? tiles_per_wave : 4, wpb = waves_per_block ? waves_per_block : 4;
+  if (!(u == 1 || u == 2 || u == 4 || u == 8) || !(wpb == 1 || wpb == 2 || wpb == 4 || wpb == 8 || wpb == 16)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": bad tiles_per_wave / waves_per_block");
+  if (!bytes) return TCU_OK;
+  if (!d_dst || (mode != 2 && !d_src) || !aligned16(d_dst) || !aligned16(d_src)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null or misaligned device pointer");
+  const size_t n_chunks = bytes / 16;
+  const size_t tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
+  const size_t waves = (tiles + u - 1) / u;
+  const size_t grid = (waves + wpb - 1) / wpb;
+  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+  const bool nt = options().nontemporal;
+  uint4_t *dst = static_cast<uint4_t *>(d_dst);
+  const half8_t *src = static_cast<const half8_t *>(d_src);
+  switch (u) {
+    case 1: launch_probe<1>(mode, nt, (unsigned)grid, wpb * 64u, stream, dst, src, n_chunks); break;
+    case 2: launch_probe<2>(mode, nt, (unsigned)grid, wpb * 64u, stream, dst, src, n_chunks); break;
+    case 4: launch_probe<4>(mode, nt, (unsigned)grid, wpb * 64u, stream, dst, src, n_chunks); break;
+    default: launch_probe<8>(mode, nt, (unsigned)grid, wpb * 64u, stream, dst, src, n_chunks); break;
+  }
+  return TCU_OK;
+}
+inline int lane_probe_dispatch(void *d_out, size_t *out_words, void *stream) {
+  if (!out_words) return fail(TCU_ERR_INVALID_ARG, "tcu_lane_probe: out_words must not be null");
+  if (!d_out) {
+    *out_words = kLaneProbeWords;
+    return TCU_OK;
+  }
+  if (*out_words < kLaneProbeWords) return fail(TCU_ERR_WORKSPACE, "tcu_lane_probe: output buffer too small");
+  launch(lane_probe_kernel, 1u, 64u, stream, static_cast<unsigned *>(d_out));
+  return TCU_OK;
+}
+
+}  // namespace tcu

@@ -1,0 +1,195 @@
+// Full-array (unsegmented) sum and inclusive prefix sum over fp16, fp32 carries.
+//
+// Single-pass kernels:
+//   full_reduce_kernel : persistent blocks stride over the array; every block leaves one
+//     fp32 partial in the workspace and takes an atomic ticket; the block that draws the
+//     last ticket adds the partials in index order (deterministic) and writes the fp16
+//     result.  Replaces the reference's atomic / cooperative-groups full reductions
+//     (src/reduction/kernel.cuh:564-786), whose combine step is an atomicAdd on one
+//     half (or a serial loop in global thread 0).
+//   full_scan_kernel   : decoupled look-back.  Partitions are handed out by an atomic
+//     ticket (so a partition's predecessors are always running or done); each block
+//     publishes {flag, fp32 aggregate} as one 64-bit word, wave 0 looks back 64
+//     descriptors at a time, then the block scans its tiles from registers.  Replaces
+//     the reference's grid-sync / spin-barrier full scans (src/prefixsum/kernel.cuh:779-972;
+//     both disabled upstream: the first needs more shared memory than exists, the second
+//     deadlocks) and its 3-kernel sequence, which moves 8+ bytes per element.
+// Multi-kernel helpers (the reference's "2 kernels" / "3 kernels" sequences):
+//   sum_f16_kernel, exclusive_scan_f16_kernel over the per-segment totals.
+#pragma once
+
+#include "seg_scan.hpp"
+
+namespace tcu {
+
+constexpr unsigned long long kFlagAggregate = 1ull << 32;
+constexpr unsigned long long kFlagPrefix = 2ull << 32;
+
+// words[0..n) = 0
+__global__ __launch_bounds__(256) void zero_words_kernel(unsigned *words, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) words[i] = 0u;
+}
+
+// workspace: counter at words[0]; partials (float) start at word 64
+template <int U, bool MFMA, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, unsigned *ws) {
+  __shared__ float partial[kMaxWaves];
+  __shared__ unsigned ticket;
+  const int lane = lane_id();
+  const int wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  float *partials = reinterpret_cast<float *>(ws + 64);
+  const half8_t ones = splat8(1.0f);
+  const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
+  const size_t stride = (size_t)gridDim.x * WPB * U;
+
+  float accs[2] = {0.0f, 0.0f};
+  float4_t accm = {0, 0, 0, 0};
+  for (size_t t0 = ((size_t)blockIdx.x * WPB + wave) * U; t0 < n_tiles; t0 += stride) {
+    half8_t v[U];
+    load_tiles<U, NT>(v, in, t0 * kTileChunks, n_chunks, lane);
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+      if constexpr (MFMA)
+        accm = mfma_16x16x32(v[j], ones, accm);
+      else
+        accs[j & 1] = sum8(v[j], accs[j & 1]);
+    }
+  }
+  float total;
+  if constexpr (MFMA)
+    total = add_xor32(add_xor16((accm[0] + accm[1]) + (accm[2] + accm[3])));
+  else
+    total = lane_group_sum<6>(accs[0] + accs[1]);
+  if (lane == 63) partial[wave] = total;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.0f;
+    for (int w = 0; w < WPB; w++) s += partial[w];
+    partials[blockIdx.x] = s;
+    device_fence_release();
+    ticket = atomic_add_u32_acq_rel(ws, 1u);
+  }
+  __syncthreads();
+  if (ticket != gridDim.x - 1) return;  // block-uniform
+  if (wave == 0) {
+    device_fence_acquire();
+    float s = 0.0f;
+    for (unsigned i = lane; i < gridDim.x; i += 64) s += atomic_load_f32(partials + i);
+    s = lane_group_sum<6>(s);
+    if (lane == 63) out[0] = f16_bits(s);
+  }
+}
+
+// One partition (blockDim/64 * U tiles) per block.  workspace: ticket counter at word 0,
+// descriptors (64-bit: flag << 32 | float bits) from byte 256.
+template <int U, bool MFMA, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws) {
+  __shared__ float wave_total[kMaxWaves];
+  __shared__ unsigned s_part;
+  __shared__ float s_prefix;
+  const int lane = lane_id();
+  const int wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  unsigned long long *desc = reinterpret_cast<unsigned long long *>(ws + 64);
+  ScanOperands ops;
+  if constexpr (MFMA) ops = make_scan_operands(lane);
+
+  if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
+  __syncthreads();
+  const unsigned part = s_part;
+  const size_t t0 = ((size_t)part * WPB + wave) * U;
+
+  half8_t v[U];
+  load_tiles<U, NT>(v, in, t0 * kTileChunks, n_chunks, lane);
+  float acc = 0.0f;
+#pragma unroll
+  for (int j = 0; j < U; j++) acc = sum8(v[j], acc);
+  acc = lane_group_sum<6>(acc);
+  if (lane == 63) wave_total[wave] = acc;
+  __syncthreads();
+
+  if (wave == 0) {
+    float aggregate = 0.0f;
+    for (int w = 0; w < WPB; w++) aggregate += wave_total[w];
+    float prefix = 0.0f;
+    if (part == 0) {
+      if (lane == 0) atomic_store_u64(desc, kFlagPrefix | __float_as_uint(aggregate));
+    } else {
+      if (lane == 0) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
+      long long base = (long long)part - 1;
+      while (true) {  // every lane of wave 0 takes the same path
+        const long long idx = base - lane;
+        unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : kFlagPrefix;
+        const unsigned flag = (unsigned)(d >> 32);
+        const unsigned long long is_prefix = ballot(flag == 2u);
+        const unsigned long long is_empty = ballot(flag == 0u);
+        const int first_prefix = is_prefix ? __builtin_ctzll(is_prefix) : 64;
+        const unsigned long long needed = first_prefix >= 63 ? ~0ull : ((2ull << first_prefix) - 1ull);
+        if (is_empty & needed) {
+          spin_pause();
+          continue;
+        }
+        float val = lane <= first_prefix ? __uint_as_float((unsigned)d) : 0.0f;
+        val = lane_group_sum<6>(val);
+        prefix += readlane(val, 63);
+        if (first_prefix < 64) break;
+        base -= 64;
+      }
+      if (lane == 0) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
+    }
+    if (lane == 0) s_prefix = prefix;
+  }
+  __syncthreads();
+  float carry = s_prefix;
+  for (int w = 0; w < wave; w++) carry += wave_total[w];
+#pragma unroll
+  for (int j = 0; j < U; j++) {
+    float tile_total;
+    scan_tile<6, MFMA, NT>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    carry += tile_total;
+  }
+}
+
+// out[0] = fp16(sum of n halves), one block
+__global__ __launch_bounds__(1024) void sum_f16_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, size_t n) {
+  __shared__ float partial[16];
+  const int lane = lane_id(), wave = wave_in_block();
+  float acc = 0.0f;
+  for (size_t i = threadIdx.x; i < n; i += blockDim.x) acc += (float)__builtin_bit_cast(half_t, in[i]);
+  acc = lane_group_sum<6>(acc);
+  if (lane == 63) partial[wave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.0f;
+    for (unsigned w = 0; w < (blockDim.x >> 6); w++) s += partial[w];
+    out[0] = f16_bits(s);
+  }
+}
+
+// in-place exclusive prefix sum of n halves (fp32 running sum, fp16 storage), one block
+__global__ __launch_bounds__(1024) void exclusive_scan_f16_kernel(uint16_t *data, size_t n) {
+  __shared__ float wave_total[16];
+  const int lane = lane_id(), wave = wave_in_block();
+  const int waves = (int)(blockDim.x >> 6);
+  float carry = 0.0f;
+  for (size_t base = 0; base < n; base += blockDim.x) {
+    const size_t i = base + threadIdx.x;
+    const float x = i < n ? (float)__builtin_bit_cast(half_t, data[i]) : 0.0f;
+    const float excl = lane_group_exclusive_scan<6>(x, lane);
+    if (lane == 63) wave_total[wave] = excl + x;
+    __syncthreads();
+    float offset = carry, all = 0.0f;
+    for (int w = 0; w < waves; w++) {
+      const float wt = wave_total[w];
+      if (w < wave) offset += wt;
+      all += wt;
+    }
+    if (i < n) data[i] = f16_bits(excl + offset);
+    carry += all;
+    __syncthreads();
+  }
+}
+
+}  // namespace tcu

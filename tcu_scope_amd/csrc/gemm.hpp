@@ -1,0 +1,135 @@
+// D = alpha * A B + beta * C.  A: M x K row-major fp16; B: K x N column-major fp16 (stored
+// as N rows of K, so both operands are K-contiguous); C, D: M x N row-major fp32.
+// Operand layouts of the reference's compute_gemm (src/gemm/wmma.cu:15-18).
+//
+//   gemm_lds_kernel    : 128 x 128 block tile, K step 32, 4 waves in a 2 x 2 grid, each wave
+//                        a 64 x 64 tile = 2 x 2 v_mfma_f32_32x32x16_f16 accumulators.
+//                        A/B tiles go global -> registers -> LDS (rows padded to 40 halves
+//                        so that the 128-bit fragment reads of 16 lanes hit distinct banks)
+//                        with the next step's global loads in flight during the MFMAs and
+//                        two LDS buffers (one barrier per step).  Counterpart of the
+//                        reference's shared-memory kernels (src/gemm/wmma.cu:171-365,
+//                        wmma_sharedmem.cu:43-123).
+//   gemm_direct_kernel : one 32 x 32 tile per wave, fragments loaded straight from global
+//                        memory (reference compute_gemm_naive, src/gemm/wmma_naive.cu:33-88).
+//   gemm_generic_kernel: any M, N, K; one thread per output element.
+#pragma once
+
+#include "wave_ops.hpp"
+
+namespace tcu {
+
+constexpr int kGemmBM = 128, kGemmBN = 128, kGemmBK = 32;
+constexpr int kGemmLdsStride = 40;  // halves per LDS row (32 + 8 pad)
+
+TCU_DEVICE void gemm_store_tile(float *D, const float *C, size_t ldc, size_t row0, size_t col0, const float16_t &acc, int lane, float alpha, float beta) {
+  const size_t col = col0 + (lane & 31);
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    const size_t row = row0 + 8 * (i / 4) + 4 * (lane >> 5) + (i % 4);
+    const size_t idx = row * ldc + col;
+    D[idx] = beta == 0.0f ? alpha * acc[i] : alpha * acc[i] + beta * C[idx];
+  }
+}
+
+// M % 128 == 0, N % 128 == 0, K % 32 == 0; 256 threads.
+__global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+  __shared__ __attribute__((aligned(16))) half_t lds_a[2][kGemmBM * kGemmLdsStride];
+  __shared__ __attribute__((aligned(16))) half_t lds_b[2][kGemmBN * kGemmLdsStride];
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // block -> tile: consecutive blocks walk down a column of tiles so that they share B
+  const size_t tiles_m = M / kGemmBM;
+  const size_t tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+  const size_t k_chunks = K / 8;
+  // global -> LDS copy assignment: 128 rows x 4 chunks = 512 chunks per operand, 2 per thread
+  const int crow = tid >> 2, cchunk = tid & 3;  // rows crow and crow + 64
+  const half8_t *ga0 = A + (tile_m * kGemmBM + crow) * k_chunks + cchunk;
+  const half8_t *ga1 = ga0 + 64 * k_chunks;
+  const half8_t *gb0 = B + (tile_n * kGemmBN + crow) * k_chunks + cchunk;
+  const half8_t *gb1 = gb0 + 64 * k_chunks;
+  const int so0 = crow * kGemmLdsStride + cchunk * 8, so1 = so0 + 64 * kGemmLdsStride;
+
+  float16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+  half8_t ra0 = ga0[0], ra1 = ga1[0], rb0 = gb0[0], rb1 = gb1[0];
+  *reinterpret_cast<half8_t *>(&lds_a[0][so0]) = ra0;
+  *reinterpret_cast<half8_t *>(&lds_a[0][so1]) = ra1;
+  *reinterpret_cast<half8_t *>(&lds_b[0][so0]) = rb0;
+  *reinterpret_cast<half8_t *>(&lds_b[0][so1]) = rb1;
+  __syncthreads();
+
+  const size_t steps = K / kGemmBK;
+  // fragment read offsets: lane l -> row l%32 of the 32-row tile, halves 8*(l/32) .. +7 of a 16-k substep
+  const int frow = lane & 31, fk = (lane >> 5) * 8;
+  for (size_t s = 0; s < steps; s++) {
+    const int cur = (int)(s & 1);
+    if (s + 1 < steps) {
+      const size_t o = (s + 1) * (kGemmBK / 8);
+      ra0 = ga0[o];
+      ra1 = ga1[o];
+      rb0 = gb0[o];
+      rb1 = gb1[o];
+    }
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+      half8_t fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) fa[i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][(wm * 64 + i * 32 + frow) * kGemmLdsStride + kk * 16 + fk]);
+#pragma unroll
+      for (int j = 0; j < 2; j++) fb[j] = *reinterpret_cast<const half8_t *>(&lds_b[cur][(wn * 64 + j * 32 + frow) * kGemmLdsStride + kk * 16 + fk]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = mfma_32x32x16(fa[i], fb[j], acc[i][j]);
+    }
+    if (s + 1 < steps) {
+      const int nxt = cur ^ 1;
+      *reinterpret_cast<half8_t *>(&lds_a[nxt][so0]) = ra0;
+      *reinterpret_cast<half8_t *>(&lds_a[nxt][so1]) = ra1;
+      *reinterpret_cast<half8_t *>(&lds_b[nxt][so0]) = rb0;
+      *reinterpret_cast<half8_t *>(&lds_b[nxt][so1]) = rb1;
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) gemm_store_tile(D, C, N, tile_m * kGemmBM + wm * 64 + i * 32, tile_n * kGemmBN + wn * 64 + j * 32, acc[i][j], lane, alpha, beta);
+}
+
+// M % 32 == 0, N % 32 == 0, K % 16 == 0; one 32 x 32 tile per wave.
+__global__ __launch_bounds__(kWave * 4) void gemm_direct_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
+                                                                 float beta) {
+  const int lane = lane_id();
+  const size_t tiles_m = M / 32, tiles_n = N / 32;
+  const size_t tile = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  if (tile >= tiles_m * tiles_n) return;
+  const size_t tile_m = tile % tiles_m, tile_n = tile / tiles_m;
+  const size_t k_chunks = K / 8;
+  const half8_t *ga = A + (tile_m * 32 + (lane & 31)) * k_chunks + (lane >> 5);
+  const half8_t *gb = B + (tile_n * 32 + (lane & 31)) * k_chunks + (lane >> 5);
+  float16_t acc;
+#pragma unroll
+  for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+  for (size_t c = 0; c < k_chunks; c += 2) acc = mfma_32x32x16(ga[c], gb[c], acc);
+  gemm_store_tile(D, C, N, tile_m * 32, tile_n * 32, acc, lane, alpha, beta);
+}
+
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
+                                                            float beta) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= M * N) return;
+  const size_t m = idx / N, n = idx % N;
+  float acc = 0.0f;
+  for (size_t k = 0; k < K; k++) acc += (float)__builtin_bit_cast(half_t, A[m * K + k]) * (float)__builtin_bit_cast(half_t, B[n * K + k]);
+  D[idx] = beta == 0.0f ? alpha * acc : alpha * acc + beta * C[idx];
+}
+
+}  // namespace tcu

@@ -1,0 +1,118 @@
+// y = alpha * A x + beta * y;  A: M x K row-major fp16, x: K fp16, y: M fp32.
+//
+// The operation streams A once (2*M*K bytes) and is bound by HBM bandwidth.
+//   gemv_dot_kernel  : each wave owns ROWS consecutive rows; per step every lane loads one
+//                      128-bit chunk of x and the matching chunk of each row (a wave reads
+//                      1 KiB of a row contiguously), multiplies with packed fp16 dot
+//                      products into fp32, and finishes with a DPP wave reduction.
+//   gemv_mfma_kernel : the reference's formulation (GEMV as a 16-wide GEMM,
+//                      src/gemv/wmma_naive.cu:29-94): a wave owns a 16-row strip, the strip
+//                      is the A operand of v_mfma_f32_16x16x32_f16 and x, replicated over
+//                      the 16 columns, the B operand.  Lane (r, b) reads 64 contiguous
+//                      bytes of row r per 4 MFMAs (k order inside a step is permuted
+//                      identically for A and x, which a contraction does not see).
+//   gemv_generic_kernel : any M, K (scalar loads).
+#pragma once
+
+#include "seg_reduce.hpp"
+
+namespace tcu {
+
+TCU_DEVICE float dot8(half8_t a, half8_t x, float acc) {
+  acc = fdot2(__builtin_shufflevector(a, a, 0, 1), __builtin_shufflevector(x, x, 0, 1), acc);
+  acc = fdot2(__builtin_shufflevector(a, a, 2, 3), __builtin_shufflevector(x, x, 2, 3), acc);
+  acc = fdot2(__builtin_shufflevector(a, a, 4, 5), __builtin_shufflevector(x, x, 4, 5), acc);
+  acc = fdot2(__builtin_shufflevector(a, a, 6, 7), __builtin_shufflevector(x, x, 6, 7), acc);
+  return acc;
+}
+
+// K must be a multiple of 8; rows are 16-byte aligned.
+template <int ROWS, int UK, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, float *__restrict__ y, size_t M, size_t k_chunks, float alpha,
+                                                              float beta) {
+  const int lane = lane_id();
+  const size_t row0 = ((size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block()) * ROWS;
+  if (row0 >= M) return;
+  float acc[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+  const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (size_t c0 = 0; c0 < k_chunks; c0 += (size_t)64 * UK) {
+    half8_t xv[UK], av[UK][ROWS];
+#pragma unroll
+    for (int u = 0; u < UK; u++) {
+      const size_t c = c0 + (size_t)u * 64 + lane;
+      const bool ok = c < k_chunks;
+      xv[u] = ok ? x[c] : zero;
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        const size_t row = row0 + r < M ? row0 + r : M - 1;  // clamp: duplicates are discarded below
+        av[u][r] = ok ? load_chunk<NT>(A + row * k_chunks + c) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UK; u++)
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) acc[r] = dot8(av[u][r], xv[u], acc[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) {
+    const float s = lane_group_sum<6>(acc[r]);
+    if (lane == 63 && row0 + r < M) {
+      float *p = y + row0 + r;
+      *p = beta == 0.0f ? alpha * s : alpha * s + beta * *p;
+    }
+  }
+}
+
+// K must be a multiple of 128.  One wave per 16-row strip.
+template <bool NT>
+__global__ __launch_bounds__(kMaxBlock) void gemv_mfma_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, float *__restrict__ y, size_t M, size_t k_chunks, float alpha,
+                                                               float beta) {
+  const int lane = lane_id();
+  const int r = lane & 15, b = lane >> 4;
+  const size_t strip = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  const size_t row0 = strip * 16;
+  if (row0 >= M) return;
+  const size_t row = row0 + r < M ? row0 + r : M - 1;
+  const half8_t *arow = A + row * k_chunks;
+  float4_t acc = {0, 0, 0, 0};
+  // a step covers 128 k = 16 chunks; lane (r, b) takes chunks 4b .. 4b+3 of the step
+  for (size_t c0 = 0; c0 < k_chunks; c0 += 32) {
+    half8_t av[2][4], xv[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int s = 0; s < 4; s++) {
+        const size_t c = c0 + (size_t)h * 16 + 4 * b + s;
+        const bool ok = c < k_chunks;
+        const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+        av[h][s] = ok ? load_chunk<NT>(arow + c) : zero;
+        xv[h][s] = ok ? x[c] : zero;
+      }
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int s = 0; s < 4; s++) acc = mfma_16x16x32(av[h][s], xv[h][s], acc);
+  }
+  // every column of D holds the strip's 16 results; column 0 writes them
+  if (r == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const size_t m = row0 + 4 * b + i;
+      if (m < M) y[m] = beta == 0.0f ? alpha * acc[i] : alpha * acc[i] + beta * y[m];
+    }
+  }
+}
+
+__global__ __launch_bounds__(kMaxBlock) void gemv_generic_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ x, float *__restrict__ y, size_t M, size_t K, float alpha, float beta) {
+  const int lane = lane_id();
+  const size_t row = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  if (row >= M) return;
+  float acc = 0.0f;
+  for (size_t k = lane; k < K; k += 64) acc += (float)__builtin_bit_cast(half_t, A[row * K + k]) * (float)__builtin_bit_cast(half_t, x[k]);
+  acc = lane_group_sum<6>(acc);
+  if (lane == 63) y[row] = beta == 0.0f ? alpha * acc : alpha * acc + beta * y[row];
+}
+
+}  // namespace tcu

@@ -1,0 +1,326 @@
+// Segmented inclusive prefix sum over fp16, fp32 accumulation, fp16 output of length N.
+//
+// Same HBM layout, chunk (8 halves) and tile (64 chunks, lane l <-> chunk l) as the
+// reduction.  A tile is scanned in three steps:
+//   1. chunk totals          T[c], c = 0..63
+//   2. exclusive scan of the totals over each segment's chunks (+ the carry that enters
+//      the tile when a segment spans several tiles)              E[c]
+//   3. inclusive scan inside every chunk, started at E[c]        out[c][i]
+// Flavour MFMA = false does 1 and 3 with packed fp16 dot products in the owning lane and
+// 2 with DPP row shifts / broadcasts (the counterpart of the reference's cub::WarpScan /
+// cub::BlockScan rows, src/prefixsum/seg_cub_warp.cu:17-27, seg_cub_block.cu:13-51).
+// Flavour MFMA = true takes the tile as the B operand of v_mfma_f32_16x16x32_f16:
+//   1. D0 = P * X with P[m][k] = [k/8 == m%4]: every lane of column n gets the four
+//      totals of chunks n, 16+n, 32+n, 48+n;
+//   3. D1 = U1 * X + C1 and D2 = U2 * X + C2 with block upper-triangular ones
+//      U1[m][k] = [k/8 == m/8][k%8 <= m%8], U2[m][k] = [k/8 == 2 + m/8][k%8 <= m%8] and the
+//      carries E broadcast in the accumulator inputs C1/C2 — scan == multiplication by a
+//      triangular ones matrix with the cross-tile carry entering through the accumulator,
+//      the formulation of reference src/prefixsum/kernel.cuh:48-83 (seg 16), :87-150
+//      (16n), :303-363 (256: L*A*O + A*U), :442-506 (256n, carry via fill_fragment);
+//   2. stays on DPP, on the four replicated totals.
+// Lane (n, g) of D1/D2 holds 4 consecutive outputs of chunk (n, g/2) / (n, 2 + g/2); two
+// v_permlane16_swap turn that into one 128-bit store per lane.
+#pragma once
+
+#include "seg_reduce.hpp"
+
+namespace tcu {
+
+// Exclusive scan of `t` over groups of 2^LOG2 adjacent lanes (lane order), LOG2 = 1..6.
+template <int LOG2>
+TCU_DEVICE float lane_group_exclusive_scan(float t, int lane) {
+  constexpr int LPS = 1 << LOG2;
+  float e = dpp<DPP_WAVE_SHR1>(0.0f, t);
+  if ((lane & (LPS - 1)) == 0) e = 0.0f;
+  if constexpr (LOG2 >= 2) {
+    float s = dpp<DPP_ROW_SHR0 + 1>(0.0f, e);
+    if (LPS < 16 && (lane & (LPS - 1)) < 1) s = 0.0f;
+    e += s;
+  }
+  if constexpr (LOG2 >= 2) {
+    float s = dpp<DPP_ROW_SHR0 + 2>(0.0f, e);
+    if (LPS < 16 && (lane & (LPS - 1)) < 2) s = 0.0f;
+    e += s;
+  }
+  if constexpr (LOG2 >= 3) {
+    float s = dpp<DPP_ROW_SHR0 + 4>(0.0f, e);
+    if (LPS < 16 && (lane & (LPS - 1)) < 4) s = 0.0f;
+    e += s;
+  }
+  if constexpr (LOG2 >= 4) e += dpp<DPP_ROW_SHR0 + 8>(0.0f, e);
+  if constexpr (LOG2 >= 5) e += dpp<DPP_ROW_BCAST15, 0xA, 0xF, false>(0.0f, e);
+  if constexpr (LOG2 >= 6) e += dpp<DPP_ROW_BCAST31, 0xC, 0xF, false>(0.0f, e);
+  return e;
+}
+
+// Exclusive scan of t over groups of 2^LOG2 lanes inside each 16-lane row, LOG2 = 1..4.
+template <int LOG2>
+TCU_DEVICE float row_group_exclusive_scan(float t, int n) {
+  constexpr int LPS = 1 << LOG2;
+  float e = dpp<DPP_ROW_SHR0 + 1>(0.0f, t);
+  if ((n & (LPS - 1)) == 0) e = 0.0f;
+  if constexpr (LOG2 >= 2) {
+    float s = dpp<DPP_ROW_SHR0 + 1>(0.0f, e);
+    if (LPS < 16 && (n & (LPS - 1)) < 1) s = 0.0f;
+    e += s;
+  }
+  if constexpr (LOG2 >= 2) {
+    float s = dpp<DPP_ROW_SHR0 + 2>(0.0f, e);
+    if (LPS < 16 && (n & (LPS - 1)) < 2) s = 0.0f;
+    e += s;
+  }
+  if constexpr (LOG2 >= 3) {
+    float s = dpp<DPP_ROW_SHR0 + 4>(0.0f, e);
+    if (LPS < 16 && (n & (LPS - 1)) < 4) s = 0.0f;
+    e += s;
+  }
+  if constexpr (LOG2 >= 4) e += dpp<DPP_ROW_SHR0 + 8>(0.0f, e);
+  return e;
+}
+
+// 8 inclusive prefixes of one chunk started at `e`, rounded to fp16 and packed.
+TCU_DEVICE uint4_t chunk_scan_packed(half8_t v, float e) {
+  const half2_t one_zero = {(half_t)1.0f, (half_t)0.0f};
+  const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
+  const half2_t h01 = __builtin_shufflevector(v, v, 0, 1), h23 = __builtin_shufflevector(v, v, 2, 3);
+  const half2_t h45 = __builtin_shufflevector(v, v, 4, 5), h67 = __builtin_shufflevector(v, v, 6, 7);
+  const float x0 = fdot2(h01, one_zero, e), x1 = fdot2(h01, ones, e);
+  const float x2 = fdot2(h23, one_zero, x1), x3 = fdot2(h23, ones, x1);
+  const float x4 = fdot2(h45, one_zero, x3), x5 = fdot2(h45, ones, x3);
+  const float x6 = fdot2(h67, one_zero, x5), x7 = fdot2(h67, ones, x5);
+  uint4_t r = {pack_f16x2(x0, x1), pack_f16x2(x2, x3), pack_f16x2(x4, x5), pack_f16x2(x6, x7)};
+  return r;
+}
+
+// Constant A operands of the MFMA flavour (see the header comment).
+struct ScanOperands {
+  half8_t totals;  // P
+  half8_t tri_lo;  // U1
+  half8_t tri_hi;  // U2
+};
+TCU_DEVICE ScanOperands make_scan_operands(int lane) {
+  const int m = lane & 15, b = lane >> 4;
+  ScanOperands o;
+  o.totals = splat8(b == (m & 3) ? 1.0f : 0.0f);
+  half8_t lo, hi;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    lo[i] = (half_t)((b == (m >> 3) && i <= (m & 7)) ? 1.0f : 0.0f);
+    hi[i] = (half_t)((b == 2 + (m >> 3) && i <= (m & 7)) ? 1.0f : 0.0f);
+  }
+  o.tri_lo = lo;
+  o.tri_hi = hi;
+  return o;
+}
+
+// One tile.  `carry` (wave-uniform) is what precedes the tile inside its segment; on
+// return *tile_total is the sum of the whole tile (only meaningful for LPS_LOG2 == 6).
+// Writes the scanned tile to out[chunk_base ..] (chunks >= n_chunks are skipped) and, when
+// totals != nullptr and the tile holds whole segments (LPS_LOG2 < 6), their totals.
+template <int LPS_LOG2, bool MFMA, bool NT>
+TCU_DEVICE void scan_tile(half8_t v, float carry, const ScanOperands &ops, int lane, uint4_t *out, size_t chunk_base, size_t n_chunks, uint16_t *totals, size_t tile_seg0,
+                          size_t num_segments, float *tile_total) {
+  constexpr int LPS = 1 << LPS_LOG2;
+  if constexpr (!MFMA) {
+    const float t = sum8(v, 0.0f);
+    const float e0 = lane_group_exclusive_scan<LPS_LOG2>(t, lane);
+    const float e = e0 + carry;
+    const uint4_t r = chunk_scan_packed(v, e);
+    const size_t c = chunk_base + lane;
+    if (c < n_chunks) store_chunk<NT>(out + c, r);
+    const float incl = e + t;
+    if constexpr (LPS_LOG2 == 6) {
+      *tile_total = readlane(e0 + t, 63);
+    } else {
+      *tile_total = 0.0f;
+      if (totals != nullptr && (lane & (LPS - 1)) == LPS - 1) {
+        const size_t s = tile_seg0 + (size_t)(lane >> LPS_LOG2);
+        if (s < num_segments) totals[s] = f16_bits(incl);
+      }
+    }
+  } else {
+    const int n = lane & 15, g = lane >> 4;
+    const float4_t zero = {0, 0, 0, 0};
+    const float4_t T = mfma_16x16x32(ops.totals, v, zero);  // T[i] = total of chunk 16*i + n
+    float e[4];
+    if constexpr (LPS_LOG2 <= 4) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) e[i] = row_group_exclusive_scan<LPS_LOG2>(T[i], n);
+      *tile_total = 0.0f;
+      if (totals != nullptr && g == 0 && (n & (LPS - 1)) == LPS - 1) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const size_t s = tile_seg0 + (size_t)((16 * i + n) >> LPS_LOG2);
+          if (s < num_segments) totals[s] = f16_bits(e[i] + T[i]);
+        }
+      }
+    } else {
+      float rowsum[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        e[i] = row_group_exclusive_scan<4>(T[i], n);
+        rowsum[i] = readlane(e[i] + T[i], 15);
+      }
+      if constexpr (LPS_LOG2 == 5) {
+        e[1] += rowsum[0];
+        e[3] += rowsum[2];
+        *tile_total = 0.0f;
+        if (totals != nullptr && lane < 2) {
+          const size_t s = tile_seg0 + (size_t)lane;
+          if (s < num_segments) totals[s] = f16_bits(lane == 0 ? rowsum[0] + rowsum[1] : rowsum[2] + rowsum[3]);
+        }
+      } else {
+        const float r01 = rowsum[0] + rowsum[1];
+        e[0] += carry;
+        e[1] += carry + rowsum[0];
+        e[2] += carry + r01;
+        e[3] += carry + (r01 + rowsum[2]);
+        *tile_total = r01 + (rowsum[2] + rowsum[3]);
+      }
+    }
+    const float c1 = g < 2 ? e[0] : e[1];
+    const float c2 = g < 2 ? e[2] : e[3];
+    const float4_t d1 = mfma_16x16x32(ops.tri_lo, v, float4_t{c1, c1, c1, c1});
+    const float4_t d2 = mfma_16x16x32(ops.tri_hi, v, float4_t{c2, c2, c2, c2});
+    unsigned a_lo = pack_f16x2(d1[0], d1[1]), a_hi = pack_f16x2(d1[2], d1[3]);
+    unsigned b_lo = pack_f16x2(d2[0], d2[1]), b_hi = pack_f16x2(d2[2], d2[3]);
+    permlane16_swap(a_lo, b_lo);
+    permlane16_swap(a_hi, b_hi);
+    // rows 0..3 now hold chunks n, 32+n, 16+n, 48+n
+    const int dst = n + 16 * (((g & 1) << 1) | (g >> 1));
+    const size_t c = chunk_base + dst;
+    const uint4_t r = {a_lo, a_hi, b_lo, b_hi};
+    if (c < n_chunks) store_chunk<NT>(out + c, r);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Wave-owned spans.  LPS_LOG2 = 1..5: S = 16..256, segments inside a tile.  LPS_LOG2 = 6:
+// S = 512 << tiles_per_seg_log2, a wave walks its segment(s) carrying the running sum.
+// Each wave owns iters*U consecutive tiles.
+// ---------------------------------------------------------------------------------------
+template <int LPS_LOG2, int U, bool MFMA, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, int tiles_per_seg_log2, unsigned iters) {
+  const int lane = lane_id();
+  const size_t gw = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  const size_t tile0 = gw * (size_t)iters * U;
+  if (tile0 * kTileChunks >= n_chunks) return;
+  const size_t tmask = ((size_t)1 << tiles_per_seg_log2) - 1;
+  ScanOperands ops;
+  if constexpr (MFMA) ops = make_scan_operands(lane);
+  constexpr int SEGS_PER_TILE = 64 >> LPS_LOG2;
+
+  float carry = 0.0f;
+  for (unsigned it = 0; it < iters; it++) {
+    const size_t t_it = tile0 + (size_t)it * U;
+    half8_t v[U];
+    load_tiles<U, NT>(v, in, t_it * kTileChunks, n_chunks, lane);
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+      const size_t t = t_it + j;
+      if (LPS_LOG2 < 6 || (t & tmask) == 0) carry = 0.0f;
+      float tile_total;
+      scan_tile<LPS_LOG2, MFMA, NT>(v[j], carry, ops, lane, out, t * kTileChunks, n_chunks, totals, t * SEGS_PER_TILE, num_segments, &tile_total);
+      if constexpr (LPS_LOG2 == 6) {
+        carry += tile_total;
+        if (totals != nullptr && ((t + 1) & tmask) == 0) {
+          const size_t s = t >> tiles_per_seg_log2;
+          if (lane == 0 && s < num_segments) totals[s] = f16_bits(carry);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// S >= 512: a block of waves shares each segment.  Per step the block takes WPB*U tiles,
+// wave w the U consecutive tiles starting at w*U; wave totals meet in LDS.
+// ---------------------------------------------------------------------------------------
+template <int U, bool MFMA, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, size_t tiles_per_seg,
+                                                                    unsigned segs_per_block) {
+  __shared__ float wave_total[2][kMaxWaves];
+  const int lane = lane_id();
+  const int wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  ScanOperands ops;
+  if constexpr (MFMA) ops = make_scan_operands(lane);
+  unsigned parity = 0;
+  for (unsigned sb = 0; sb < segs_per_block; sb++) {
+    const size_t seg = (size_t)blockIdx.x * segs_per_block + sb;
+    if (seg >= num_segments) break;  // block-uniform
+    const size_t tile_base = seg * tiles_per_seg;
+    size_t lim = (tile_base + tiles_per_seg) * kTileChunks;
+    if (lim > n_chunks) lim = n_chunks;
+    float block_carry = 0.0f;
+    for (size_t step0 = 0; step0 < tiles_per_seg; step0 += (size_t)WPB * U) {
+      const size_t t0 = step0 + (size_t)wave * U;  // first tile of this wave (may lie past the segment)
+      half8_t v[U];
+      load_tiles<U, NT>(v, in, (tile_base + t0) * kTileChunks, t0 < tiles_per_seg ? lim : 0, lane);
+      // pass 1: this wave's total
+      float acc = 0.0f;
+#pragma unroll
+      for (int j = 0; j < U; j++) acc = sum8(v[j], acc);
+      acc = lane_group_sum<6>(acc);
+      if (lane == 63) wave_total[parity][wave] = acc;
+      __syncthreads();
+      float carry = block_carry, all = 0.0f;
+      for (int w = 0; w < WPB; w++) {
+        const float x = wave_total[parity][w];
+        if (w < wave) carry += x;
+        all += x;
+      }
+      block_carry += all;
+      parity ^= 1u;
+      // pass 2: scan the tiles held in registers
+#pragma unroll
+      for (int j = 0; j < U; j++) {
+        float tile_total;
+        scan_tile<6, MFMA, NT>(v[j], carry, ops, lane, out, (tile_base + t0 + j) * kTileChunks, t0 + j < tiles_per_seg ? lim : 0, nullptr, 0, 0, &tile_total);
+        carry += tile_total;
+      }
+    }
+    if (totals != nullptr && threadIdx.x == 0) totals[seg] = f16_bits(block_carry);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// any S >= 1: one wave per segment, 64 elements per step
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kMaxBlock) void seg_scan_generic_kernel(const uint16_t *in, uint16_t *out, uint16_t *totals, size_t num_segments, size_t segment_size) {
+  const int lane = lane_id();
+  const size_t seg = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  if (seg >= num_segments) return;
+  const uint16_t *p = in + seg * segment_size;
+  uint16_t *q = out + seg * segment_size;
+  float carry = 0.0f;
+  for (size_t base = 0; base < segment_size; base += 64) {
+    const size_t i = base + lane;
+    const float x = i < segment_size ? (float)__builtin_bit_cast(half_t, p[i]) : 0.0f;
+    const float incl = lane_group_exclusive_scan<6>(x, lane) + x + carry;
+    if (i < segment_size) q[i] = f16_bits(incl);
+    carry = readlane(incl, 63);
+  }
+  if (totals != nullptr && lane == 0) totals[seg] = f16_bits(carry);
+}
+
+// out[s*S + i] += partial_sums[s], one fp16 addition per element (8 per lane per step)
+__global__ __launch_bounds__(256) void add_partial_sums_kernel(uint4_t *out, const uint16_t *partial_sums, size_t n_chunks, int seg_log2_chunks) {
+  const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n_chunks) return;
+  const float ps = (float)__builtin_bit_cast(half_t, partial_sums[c >> seg_log2_chunks]);
+  uint4_t raw = out[c];
+  half8_t v = __builtin_bit_cast(half8_t, raw);
+  uint4_t r = {pack_f16x2((float)v[0] + ps, (float)v[1] + ps), pack_f16x2((float)v[2] + ps, (float)v[3] + ps), pack_f16x2((float)v[4] + ps, (float)v[5] + ps),
+               pack_f16x2((float)v[6] + ps, (float)v[7] + ps)};
+  out[c] = r;
+}
+__global__ __launch_bounds__(256) void add_partial_sums_generic_kernel(uint16_t *out, const uint16_t *partial_sums, size_t n, size_t segment_size) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float ps = (float)__builtin_bit_cast(half_t, partial_sums[i / segment_size]);
+  out[i] = f16_bits((float)__builtin_bit_cast(half_t, out[i]) + ps);
+}
+
+}  // namespace tcu

@@ -3,6 +3,11 @@ import sys
 
 import pytest
 
+try:  # paid once here, outside any per-test time limit (the first import on a fresh box is slow)
+    import torch  # noqa: F401
+except Exception:  # pragma: no cover
+    torch = None
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

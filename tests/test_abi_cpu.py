@@ -1,0 +1,66 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header
+declares, and validates arguments without touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import tcu_scope_amd
+
+    if not os.path.exists(tcu_scope_amd.library_path()):
+        tcu_scope_amd.build()
+    return tcu_scope_amd.lib()
+
+
+def test_header_and_library_agree(lib):
+    import tcu_scope_amd.binding as b
+
+    text = open(os.path.join(ROOT, "include", "tcu_scope.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(tcu_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(b.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.tcu_abi_version() == 1
+
+
+def test_argument_validation_needs_no_gpu(lib):
+    sz = ctypes.c_size_t
+    err = lambda: lib.tcu_last_error().decode()
+    buf = ctypes.create_string_buffer(4096 + 16)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+    assert lib.tcu_seg_reduce_f16(p, p, 0, 16, 0, 0, 0, None) == 0          # empty: no launch
+    assert lib.tcu_seg_reduce_f16(p, p, 4, 0, 0, 0, 0, None) == 1 and "segment_size" in err()
+    assert lib.tcu_seg_reduce_f16(p, p, 4, 32, 1, 0, 0, None) == 2 and "must be 16" in err()
+    assert lib.tcu_seg_reduce_f16(p, p, 4, 16, 4, 0, 0, None) == 2 and "must be 256" in err()
+    assert lib.tcu_seg_reduce_f16(p, p, 4, 16, 99, 0, 0, None) == 1
+    assert lib.tcu_seg_reduce_f16(None, p, 4, 16, 0, 0, 0, None) == 1
+    assert lib.tcu_seg_scan_f16(p, p, None, 4, 48, 7, 0, 0, None) == 2
+    assert lib.tcu_seg_scan_f16(p, p, None, 4, 16, 7, 5, 0, None) == 1
+    need = sz(0)
+    assert lib.tcu_full_scan_f16(None, None, 1 << 30, None, ctypes.byref(need), 0, 0, 0, None) == 0
+    assert need.value == 256 + 8 * ((1 << 30) // 8192)
+    assert lib.tcu_full_reduce_f16(None, None, 1 << 30, None, ctypes.byref(need), 0, 0, 0, None) == 0 and need.value > 0
+    assert lib.tcu_full_reduce_f16(None, None, 1000, None, ctypes.byref(need), 2, 2048, 0, None) == 2  # n % segment_size
+    assert lib.tcu_full_scan_f16(None, None, 1 << 20, None, None, 0, 0, 0, None) == 1
+    assert lib.tcu_gemv_f16_f32(p, p, p, 4, 8, 1.0, 0.0, 5, None) == 2
+    assert lib.tcu_gemm_f16_f32(p, p, None, p, 64, 64, 64, 1.0, 0.0, 8, None) == 2  # LDS kernel needs multiples of 128
+    assert lib.tcu_set_option(b"no_such_option", 1) == 1
+    assert lib.tcu_set_option(b"nontemporal", 1) == 0
+    words = sz(0)
+    assert lib.tcu_lane_probe(None, ctypes.byref(words), None) == 0 and words.value == 2560
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    import tcu_scope_amd.binding as b
+
+    monkeypatch.setattr(b, "_lib", None)
+    monkeypatch.setattr(b, "_LIB", str(tmp_path / "nope.so"))
+    with pytest.raises(ImportError):
+        b.lib()

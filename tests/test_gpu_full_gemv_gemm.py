@@ -1,0 +1,160 @@
+"""GPU parity of the full-array reduction / prefix sum and of GEMV / GEMM."""
+import numpy as np
+import pytest
+
+from gpu_common import expect_ok, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tcu():
+    import tcu_scope_amd as t
+
+    t.init(0)
+    return t
+
+
+@pytest.mark.parametrize("n", [8, 1000, 1003, 1 << 12, (1 << 20) + 8 * 37, 1 << 24])
+def test_full_reduce_and_scan(tcu, oracle, n):
+    S = tcu.FullStrategy
+    x = oracle.generate_f16(n, 4, oracle.DIST_UNIFORM)
+    ref = oracle.seg_scan_f64(x, 1, n)
+    xd = to_dev(x)
+    for strategy, seg, w in [(S.AUTO, 0, 0), (S.SINGLE_PASS, 2048, 4), (S.SINGLE_PASS, 1024, 1), (S.SINGLE_PASS, 65536, 8), (S.MULTI_KERNEL, 0, 0), (S.MULTI_KERNEL, 256, 2)]:
+        try:
+            red = to_host(tcu.full_reduce(xd, strategy, seg, w))
+            sc = to_host(tcu.full_scan(xd, strategy, seg, w))
+        except tcu.TcuError as e:
+            assert e.status == 2 and strategy == S.MULTI_KERNEL and n % (seg or 2048) != 0, (strategy, seg, str(e))
+            continue
+        expect_ok(oracle, red, ref[-1:], n, f"full reduce n={n} {strategy.name} seg={seg}")
+        expect_ok(oracle, sc, ref, n, f"full scan n={n} {strategy.name} seg={seg}")
+
+
+def test_full_exact_grid_bitwise_and_repeatable(tcu, oracle):
+    import torch
+
+    n = 1 << 22  # |prefix| stays far below 8192: every fp32 partial sum is exact
+    x = oracle.generate_f16(n, 6, oracle.DIST_GRID)
+    ref = oracle.seg_scan_f64(x, 1, n)
+    assert np.abs(ref).max() < 8192
+    xd = to_dev(x)
+    want = ref.astype(np.float16).view(np.uint16)
+    assert np.array_equal(to_host(tcu.full_scan(xd)), want)
+    assert to_host(tcu.full_reduce(xd))[0] == want[-1]
+    # same workspace reused back to back (it needs no initialisation between calls)
+    ws = torch.empty(tcu.binding.full_workspace_bytes("scan", n), dtype=torch.uint8, device="cuda")
+    ws.fill_(0xAB)
+    for _ in range(3):
+        assert np.array_equal(to_host(tcu.full_scan(xd, workspace=ws)), want)
+    y = to_dev(oracle.generate_f16(n, 7, oracle.DIST_UNIFORM))
+    a, b = to_host(tcu.full_reduce(y)), to_host(tcu.full_reduce(y))
+    assert a[0] == b[0], "full reduction is deterministic"
+    with pytest.raises(tcu.TcuError) as e:
+        tcu.full_scan(xd, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))
+    assert e.value.status == 4
+
+
+def test_full_size_2p30(tcu, oracle):
+    """N = 2^30: reduction against the fp64 sum; scan through its last element, windows at
+    both ends and the overflow rule (fp16 saturates to inf only where the fp64 prefix does)."""
+    n = 1 << 30
+    xd = tcu.generate(n, 1, tcu.Dist.UNIFORM)
+    red = to_host(tcu.full_reduce(xd))
+    out = tcu.full_scan(xd)
+    # fp64 prefix at chunk boundaries, streamed on the host in 2^26 pieces
+    piece = 1 << 26
+    carry = 0.0
+    first_ref = last_ref = None
+    for p in range(n // piece):
+        xp = oracle.generate_f16(piece, 1, oracle.DIST_UNIFORM, first=p * piece)
+        sc = oracle.seg_scan_f64(xp, 1, piece) + carry
+        if p == 0:
+            first_ref = sc.copy()
+        if p == n // piece - 1:
+            last_ref = sc.copy()
+        got = to_host(out[p * piece + piece - 1:p * piece + piece])
+        expect_ok(oracle, got, sc[-1:], n, f"2^30 scan at element {p * piece + piece - 1}")
+        carry = sc[-1]
+    expect_ok(oracle, red, np.array([carry]), n, "2^30 full reduce")
+    expect_ok(oracle, to_host(out[:piece]), first_ref, n, "2^30 scan first window")
+    expect_ok(oracle, to_host(out[n - piece:]), last_ref, n, "2^30 scan last window")
+
+
+def test_add_partial_sums(tcu, oracle):
+    for seg, nseg in [(256, 100), (2048, 33), (24, 10)]:
+        out = oracle.generate_f16(seg * nseg, 4, oracle.DIST_UNIFORM)
+        ps = oracle.generate_f16(nseg, 6, oracle.DIST_UNIFORM)
+        d = to_dev(out)
+        tcu.add_partial_sums(d, to_dev(ps), seg)
+        assert np.array_equal(to_host(d), oracle.add_partial_sums_ref(out, ps, nseg, seg))
+
+
+@pytest.mark.parametrize("M,K", [(16384, 16384), (4096, 1024), (1000, 4096), (37, 264), (5, 20)])
+def test_gemv(tcu, oracle, M, K):
+    import torch
+
+    A = oracle.generate_f16(M * K, 1, oracle.DIST_NORMAL)
+    x = oracle.generate_f16(K, 2, oracle.DIST_NORMAL)
+    y0 = np.linspace(-1, 1, M).astype(np.float32)
+    Ad, xd = to_dev(A).view(M, K), to_dev(x)
+    for v in (tcu.Variant.AUTO, tcu.Variant.WAVE_SHUFFLE, tcu.Variant.MFMA_16N):
+        for alpha, beta in [(1.0, 0.0), (1.5, -0.5)]:
+            y = torch.from_numpy(y0.copy()).cuda()
+            try:
+                tcu.gemv(Ad, xd, alpha, beta, y=y, variant=v)
+            except tcu.TcuError as e:
+                assert e.status == 2 and K % 8 != 0
+                continue
+            torch.cuda.synchronize()
+            ref = oracle.gemv_f64(A, x, M, K, alpha, beta, y0)
+            # fp32 accumulation of K products of N(0,1) values: 1e-2 relative at the scale sqrt(K)
+            bad, worst, first = oracle.check_f32_rel(y.cpu().numpy(), ref, 1e-2, float(np.sqrt(K)))
+            assert bad == 0, (v.name, alpha, beta, bad, worst, first)
+            bad, worst, first = oracle.check_f32_rel(y.cpu().numpy(), ref, 1e-4, float(np.sqrt(K)))
+            assert bad == 0, ("tight", v.name, alpha, beta, bad, worst, first)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (512, 384, 160), (96, 64, 48), (33, 17, 20)])
+def test_gemm_small_exact_and_normal(tcu, oracle, M, N, K):
+    import torch
+
+    C0 = (np.arange(M * N) % 7).astype(np.float32)
+    for dist, exact in [(oracle.DIST_SMALLINT, True), (oracle.DIST_NORMAL, False)]:
+        A = oracle.generate_f16(M * K, 5, dist)
+        B = oracle.generate_f16(N * K, 6, dist)
+        Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
+        for v in (tcu.Variant.AUTO, tcu.Variant.BLOCK_LDS, tcu.Variant.MFMA_16N):
+            for alpha, beta in [(1.0, 0.0), (2.0, 3.0)]:
+                Cd = torch.from_numpy(C0.copy()).cuda().view(M, N)
+                try:
+                    D = tcu.gemm(Ad, Bd, alpha, beta, C=Cd, variant=v)
+                except tcu.TcuError as e:
+                    assert e.status == 2
+                    continue
+                torch.cuda.synchronize()
+                ref = oracle.gemm_f64(A, B, M, N, K, alpha, beta, C0)
+                got = D.cpu().numpy()
+                if exact:  # the reference's rand()%3 fill: integer sums are exact in fp32
+                    assert np.array_equal(got.astype(np.float64), ref), (v.name, alpha, beta)
+                else:
+                    bad, worst, first = oracle.check_f32_rel(got, ref, 1e-2, float(np.sqrt(K)))
+                    assert bad == 0, (v.name, alpha, beta, bad, worst, first)
+
+
+def test_gemm_8192(tcu, oracle):
+    """M = N = K = 8192, N(0,1) inputs, 1e-2 relative: 64 sampled rows against the fp64 oracle."""
+    import torch
+
+    M = N = K = 8192
+    Ad = tcu.generate(M * K, 11, tcu.Dist.NORMAL).view(M, K)
+    Bd = tcu.generate(N * K, 12, tcu.Dist.NORMAL).view(N, K)
+    D = tcu.gemm(Ad, Bd)
+    torch.cuda.synchronize()
+    A, B = to_host(Ad).ravel(), to_host(Bd).ravel()
+    rows = [0, 1, 127, 128, 4095, 4096, 8191] + list(range(300, 8192, 997))
+    for r in rows:
+        ref = oracle.gemm_f64(A, B, M, N, K, row0=r, rows=1)
+        bad, worst, first = oracle.check_f32_rel(D[r].cpu().numpy(), ref, 1e-2, float(np.sqrt(K)))
+        assert bad == 0, (r, bad, worst, first)

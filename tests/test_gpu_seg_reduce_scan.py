@@ -1,0 +1,230 @@
+"""GPU parity of the segmented reduction and inclusive prefix sum against the CPU oracle,
+through the C ABI.  Tolerance: |out - fp64 sum| <= 2 ulp_fp16(result) + 1e-3*sqrt(segment size);
+inputs on the k/2048 grid must match bit for bit (their fp32 partial sums are exact)."""
+import numpy as np
+import pytest
+
+from gpu_common import expect_ok, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+SEGS = [16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 16384]
+
+
+@pytest.fixture(scope="module")
+def tcu():
+    import tcu_scope_amd as t
+
+    t.init(0)
+    return t
+
+
+def variants_for(tcu, seg):
+    V = tcu.Variant
+    out = [V.AUTO, V.WAVE_SHUFFLE, V.MFMA_16N]
+    if seg == 16:
+        out.append(V.MFMA_16)
+    if seg == 256:
+        out.append(V.MFMA_256)
+    if seg >= 256:
+        out.append(V.MFMA_256N)
+    if seg >= 512:
+        out += [V.BLOCK_LDS, V.MFMA_256N_BLOCK, V.MFMA_16N_BLOCK]
+    return out
+
+
+@pytest.mark.parametrize("seg", SEGS)
+def test_seg_reduce_uniform_all_variants(tcu, oracle, seg):
+    n = 1 << 21
+    nseg = n // seg
+    x = oracle.generate_f16(n, 1, oracle.DIST_UNIFORM)
+    ref = oracle.seg_reduce_f64(x, nseg, seg)
+    xd = to_dev(x)
+    for v in variants_for(tcu, seg):
+        for u, w in [(0, 0), (1, 1), (2, 8), (4, 2), (8, 16)]:
+            got = to_host(tcu.seg_reduce(xd, seg, variant=v, tiles_per_wave=u, waves_per_block=w))
+            expect_ok(oracle, got, ref, seg, f"seg_reduce seg={seg} {v.name} u={u} w={w}")
+
+
+@pytest.mark.parametrize("seg", SEGS)
+def test_seg_scan_uniform_all_variants(tcu, oracle, seg):
+    import torch
+
+    n = 1 << 21
+    nseg = n // seg
+    x = oracle.generate_f16(n, 2, oracle.DIST_UNIFORM)
+    ref = oracle.seg_scan_f64(x, nseg, seg)
+    ref_tot = ref.reshape(nseg, seg)[:, -1]
+    xd = to_dev(x)
+    for v in variants_for(tcu, seg):
+        for u, w in [(0, 0), (1, 1), (2, 8), (4, 2), (8, 16)]:
+            tot = torch.zeros(nseg, dtype=torch.float16, device="cuda")
+            got = to_host(tcu.seg_scan(xd, seg, variant=v, tiles_per_wave=u, waves_per_block=w, totals=tot))
+            expect_ok(oracle, got, ref, seg, f"seg_scan seg={seg} {v.name} u={u} w={w}")
+            expect_ok(oracle, to_host(tot), ref_tot, seg, f"seg_scan totals seg={seg} {v.name} u={u} w={w}")
+
+
+@pytest.mark.parametrize("seg", [16, 256, 1024, 8192])
+def test_exact_grid_inputs_bitwise(tcu, oracle, seg):
+    n = 1 << 20
+    nseg = n // seg
+    x = oracle.generate_f16(n, 21, oracle.DIST_GRID)
+    sc = oracle.seg_scan_f64(x, nseg, seg)
+    want_scan = sc.astype(np.float16).view(np.uint16)
+    want_red = want_scan.reshape(nseg, seg)[:, -1]
+    assert np.array_equal(want_red, oracle.seg_reduce_ref(x, nseg, seg))  # the reference CPU path agrees bit for bit here
+    xd = to_dev(x)
+    for v in variants_for(tcu, seg):
+        assert np.array_equal(to_host(tcu.seg_reduce(xd, seg, variant=v)), want_red), f"reduce {v.name}"
+        assert np.array_equal(to_host(tcu.seg_scan(xd, seg, variant=v)), want_scan), f"scan {v.name}"
+
+
+def test_reference_fixture_constant_fill(tcu, oracle):
+    """The reference fills its inputs with (half)0.001f; closed forms seg*c and (i+1)*c."""
+    import torch
+
+    c = 0.00100040435791015625
+    for seg in (16, 256, 2048):
+        n = 1 << 18
+        nseg = n // seg
+        x = torch.empty(n, dtype=torch.float16, device="cuda")
+        tcu.fill(x, 0.001)
+        assert np.all(to_host(x) == 0x1419)
+        red = to_host(tcu.seg_reduce(x, seg)).view(np.float16).astype(np.float64)
+        sc = to_host(tcu.seg_scan(x, seg)).view(np.float16).astype(np.float64).reshape(nseg, seg)
+        expect_ok(oracle, to_host(tcu.seg_reduce(x, seg)), np.full(nseg, seg * c), seg, "fixture reduce")
+        expect_ok(oracle, to_host(tcu.seg_scan(x, seg)), np.tile((np.arange(seg) + 1) * c, nseg), seg, "fixture scan")
+        assert np.all(np.abs(red - seg * c) <= 0.1) and np.all(np.abs(sc - (np.arange(seg) + 1) * c) <= 0.01)  # the reference's own tolerances
+
+
+def test_ragged_and_edge_cases(tcu, oracle):
+    import torch
+
+    V = tcu.Variant
+    # tails: segment counts that do not fill a tile / wave / block
+    for seg, nseg in [(16, 1), (16, 3), (16, 33), (16, 257), (64, 5), (256, 7), (512, 3), (1024, 5), (2048, 3), (4096, 1)]:
+        x = oracle.generate_f16(nseg * seg, 7, oracle.DIST_UNIFORM)
+        xd = to_dev(x)
+        for v in variants_for(tcu, seg):
+            for u in (1, 8):
+                out = torch.full((nseg + 64,), 7.0, dtype=torch.float16, device="cuda")  # guard words after the end
+                tcu.seg_reduce(xd, seg, variant=v, tiles_per_wave=u, out=out, num_segments=nseg)
+                h = to_host(out)
+                expect_ok(oracle, h[:nseg], oracle.seg_reduce_f64(x, nseg, seg), seg, f"tail reduce seg={seg} nseg={nseg} {v.name}")
+                assert np.all(h[nseg:] == 0x4700), f"reduce wrote past the end: seg={seg} nseg={nseg} {v.name}"
+                outs = torch.full((nseg * seg + 512,), 7.0, dtype=torch.float16, device="cuda")
+                tcu.seg_scan(xd, seg, variant=v, tiles_per_wave=u, out=outs, num_segments=nseg)
+                h = to_host(outs)
+                expect_ok(oracle, h[: nseg * seg], oracle.seg_scan_f64(x, nseg, seg), seg, f"tail scan seg={seg} nseg={nseg} {v.name}")
+                assert np.all(h[nseg * seg:] == 0x4700), f"scan wrote past the end: seg={seg} nseg={nseg} {v.name}"
+    # segment sizes outside the fast kernels (AUTO only)
+    for seg, nseg in [(1, 100), (7, 91), (24, 50), (100, 33), (1000, 9)]:
+        x = oracle.generate_f16(nseg * seg, 8, oracle.DIST_UNIFORM)
+        xd = to_dev(x)
+        expect_ok(oracle, to_host(tcu.seg_reduce(xd, seg)), oracle.seg_reduce_f64(x, nseg, seg), seg, f"generic reduce seg={seg}")
+        expect_ok(oracle, to_host(tcu.seg_scan(xd, seg)), oracle.seg_scan_f64(x, nseg, seg), seg, f"generic scan seg={seg}")
+        with pytest.raises(tcu.TcuError) as e:
+            tcu.seg_reduce(xd, seg, variant=V.WAVE_SHUFFLE)
+        assert e.value.status == 2
+    # empty input is a no-op
+    empty = torch.empty(0, dtype=torch.float16, device="cuda")
+    assert tcu.seg_reduce(empty, 16).numel() == 0 and tcu.seg_scan(empty, 16).numel() == 0
+    # the reference's precondition failures map to "unsupported"
+    x = to_dev(oracle.generate_f16(4096, 9, oracle.DIST_UNIFORM))
+    for v, seg in [(V.MFMA_16, 32), (V.MFMA_256, 16), (V.MFMA_256N, 128), (V.BLOCK_LDS, 256)]:
+        with pytest.raises(tcu.TcuError) as e:
+            tcu.seg_reduce(x, seg, variant=v)
+        assert e.value.status == 2
+        with pytest.raises(tcu.TcuError) as e:
+            tcu.seg_scan(x, seg, variant=v)
+        assert e.value.status == 2
+    with pytest.raises(tcu.TcuError) as e:
+        tcu.seg_reduce(x, 0)
+    assert e.value.status == 1
+    with pytest.raises(tcu.TcuError) as e:
+        tcu.seg_reduce(x, 16, tiles_per_wave=3)
+    assert e.value.status == 1
+    with pytest.raises(tcu.TcuError) as e:
+        tcu.seg_reduce(x[1:], 16, variant=V.WAVE_SHUFFLE, num_segments=8)  # misaligned
+    assert e.value.status == 1
+    expect_ok(oracle, to_host(tcu.seg_reduce(x[1:], 16, num_segments=8)), oracle.seg_reduce_f64(to_host(x)[1:129], 8, 16), 16, "misaligned AUTO")
+
+
+def test_scan_in_place_and_structure(tcu, oracle):
+    import torch
+
+    seg, nseg = 2048, 512
+    x = oracle.generate_f16(seg * nseg, 11, oracle.DIST_UNIFORM)
+    xd = to_dev(x)
+    want = to_host(tcu.seg_scan(xd, seg))
+    y = xd.clone()
+    tcu.seg_scan(y, seg, out=y)
+    assert np.array_equal(to_host(y), want), "in-place scan differs"
+    # one-hot input gives an exact step, zeros give zeros
+    z = torch.zeros(seg * nseg, dtype=torch.float16, device="cuda")
+    assert not to_host(tcu.seg_scan(z, seg)).any() and not to_host(tcu.seg_reduce(z, seg)).any()
+    z[5 * seg + 1234] = 1.0
+    sc = to_host(tcu.seg_scan(z, seg)).view(np.float16).reshape(nseg, seg)
+    step = np.zeros((nseg, seg), np.float16)
+    step[5, 1234:] = 1.0
+    assert np.array_equal(sc, step)
+    # changing one segment leaves every other output bit-identical
+    x2 = x.copy()
+    x2[7 * seg + 3] ^= 0x0100
+    a, b = want.reshape(nseg, seg), to_host(tcu.seg_scan(to_dev(x2), seg)).reshape(nseg, seg)
+    assert np.array_equal(np.delete(a, 7, 0), np.delete(b, 7, 0)) and not np.array_equal(a[7], b[7])
+
+
+def test_device_generator_matches_oracle(tcu, oracle):
+    n = (1 << 20) + 13
+    for dist in (tcu.Dist.UNIFORM, tcu.Dist.GRID, tcu.Dist.SMALLINT):
+        got = to_host(tcu.generate(n, 12345, dist, first=99))
+        assert np.array_equal(got, oracle.generate_f16(n, 12345, int(dist), first=99)), dist.name
+    g = to_host(tcu.generate(1 << 20, 3, tcu.Dist.NORMAL)).view(np.float16).astype(np.float64)
+    h = oracle.generate_f16(1 << 20, 3, oracle.DIST_NORMAL).view(np.float16).astype(np.float64)
+    assert np.mean(g != h) < 1e-3 and np.max(np.abs(g - h)) <= 2 ** -7  # libm differences move at most a rounding boundary
+
+
+@pytest.mark.parametrize("seg", [16, 256, 1024, 4096, 16384])
+def test_full_size_seg_reduce(tcu, oracle, seg):
+    """N = 2^28 (the benchmark configuration): every variant against the oracle."""
+    n = 1 << 28
+    nseg = n // seg
+    xd = tcu.generate(n, 1, tcu.Dist.UNIFORM)
+    x = oracle.generate_f16(n, 1, oracle.DIST_UNIFORM)
+    ref = oracle.seg_reduce_f64(x, nseg, seg)
+    for v in variants_for(tcu, seg):
+        expect_ok(oracle, to_host(tcu.seg_reduce(xd, seg, variant=v)), ref, seg, f"2^28 reduce seg={seg} {v.name}")
+
+
+@pytest.mark.parametrize("seg", [16, 256, 2048, 16384])
+def test_full_size_seg_scan(tcu, oracle, seg):
+    """N = 2^28: the last element of every scanned segment against the fp64 segment sum,
+    adjacent differences against the inputs, a 2^24-element window against the oracle, and
+    all variants bit-identical on exact-grid inputs."""
+    import torch
+
+    n = 1 << 28
+    nseg = n // seg
+    xd = tcu.generate(n, 1, tcu.Dist.UNIFORM)
+    x = oracle.generate_f16(n, 1, oracle.DIST_UNIFORM)
+    red64 = oracle.seg_reduce_f64(x, nseg, seg)
+    win = 1 << 24
+    for v in variants_for(tcu, seg):
+        out = tcu.seg_scan(xd, seg, variant=v)
+        last = to_host(out.view(nseg, seg)[:, -1].contiguous())
+        expect_ok(oracle, last, red64, seg, f"2^28 scan last element seg={seg} {v.name}")
+        for lo in (0, n - win):
+            got = to_host(out[lo:lo + win])
+            expect_ok(oracle, got, oracle.seg_scan_f64(x[lo:lo + win], win // seg, seg), seg, f"2^28 scan window@{lo} seg={seg} {v.name}")
+        # scan[i] - scan[i-1] = x[i] up to the two roundings of the outputs
+        o32, x32 = out.float().view(nseg, seg), xd.float().view(nseg, seg)
+        d = (o32[:, 1:] - o32[:, :-1] - x32[:, 1:]).abs()
+        ulp = torch.maximum(o32[:, 1:].abs(), o32[:, :-1].abs()) * 2.0 ** -10 + 2.0 ** -24
+        assert bool((d <= 2 * ulp + 2e-3 * seg ** 0.5).all()), f"difference identity seg={seg} {v.name}"
+        del out, o32, x32, d, ulp
+    gd = tcu.generate(n, 5, tcu.Dist.GRID)
+    base = tcu.seg_scan(gd, seg, variant=tcu.Variant.WAVE_SHUFFLE)
+    if seg <= 8192:
+        for v in variants_for(tcu, seg):
+            assert torch.equal(tcu.seg_scan(gd, seg, variant=v), base), f"grid inputs: {v.name} differs from WAVE_SHUFFLE"
