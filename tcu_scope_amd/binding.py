@@ -6,7 +6,7 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB = os.path.join(_HERE, "libtcu_scope_amd.so")
+_LIB = os.environ.get("TCU_SCOPE_AMD_LIBRARY") or os.path.join(_HERE, "libtcu_scope_amd.so")
 _CSRC = os.path.join(_HERE, "csrc")
 
 EXPORTS = [
@@ -146,7 +146,7 @@ def seg_reduce(x, segment_size, variant=Variant.AUTO, tiles_per_wave=0, waves_pe
     """out[j] = sum of x[j*S:(j+1)*S] (fp32 accumulate, fp16 result)."""
     torch = _torch()
     _need_f16(x, "x")
-    nseg = x.numel() // segment_size if num_segments is None else num_segments
+    nseg = (x.numel() // segment_size if segment_size > 0 else 1) if num_segments is None else num_segments
     if out is None:
         out = torch.empty(nseg, dtype=torch.float16, device=x.device)
     _check(lib().tcu_seg_reduce_f16(_ptr(x), _ptr(out), nseg, segment_size, int(variant), tiles_per_wave, waves_per_block, _stream(stream)))
@@ -157,9 +157,9 @@ def seg_scan(x, segment_size, variant=Variant.AUTO, tiles_per_wave=0, waves_per_
     """Inclusive prefix sum inside every segment; `totals` (optional tensor) receives the segment totals."""
     torch = _torch()
     _need_f16(x, "x")
-    nseg = x.numel() // segment_size if num_segments is None else num_segments
+    nseg = (x.numel() // segment_size if segment_size > 0 else 1) if num_segments is None else num_segments
     if out is None:
-        out = torch.empty(nseg * segment_size, dtype=torch.float16, device=x.device)
+        out = torch.empty(nseg * max(segment_size, 0), dtype=torch.float16, device=x.device)
     _check(lib().tcu_seg_scan_f16(_ptr(x), _ptr(out), _ptr(totals), nseg, segment_size, int(variant), tiles_per_wave, waves_per_block, _stream(stream)))
     return out
 

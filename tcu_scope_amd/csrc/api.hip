@@ -81,6 +81,10 @@ int tcu_set_option(const char *name, int value) {
     tcu::options().nontemporal = value != 0;
     return TCU_OK;
   }
+  if (std::strcmp(name, "static_order") == 0) {
+    tcu::options().static_order = value != 0;
+    return TCU_OK;
+  }
   return tcu::fail(TCU_ERR_INVALID_ARG, std::string("tcu_set_option: unknown option ") + name);
 }
 

@@ -33,6 +33,7 @@ inline int fail(int code, const std::string &msg) {
 
 struct Options {
   bool nontemporal = true;
+  bool static_order = false;
 };
 inline Options &options() {
   static Options o;
@@ -97,6 +98,32 @@ inline int validate_segmented(const char *what, const void *in, const void *out,
   return TCU_OK;
 }
 
+// Launch shapes measured on MI355X at N = 2^28 (timings in profiles/): for each segment
+// size the family and (tiles per wave, waves per block) that moved the most bytes per
+// second.  MFMA and DPP flavours tie within run-to-run noise at every size (the kernels
+// are bound by HBM, not by issue slots), so AUTO takes the DPP flavour.
+struct Plan {
+  bool block;  // block-per-segment kernel
+  int u, w;
+};
+inline Plan auto_plan_reduce(size_t S) {
+  if (S <= 32) return {false, 2, 1};
+  if (S <= 512) return {false, 2, 4};
+  if (S == 1024) return {false, 4, 4};
+  if (S == 2048) return {false, 1, 1};
+  if (S == 4096) return {true, 2, 4};
+  if (S == 8192) return {true, 4, 8};
+  return {true, 1, 8};
+}
+inline Plan auto_plan_scan(size_t S) {
+  if (S <= 512) return {false, 1, 1};
+  if (S == 1024) return {false, 1, 2};
+  if (S == 2048) return {true, 4, 2};
+  if (S == 4096) return {true, 1, 2};
+  if (S == 8192) return {true, 4, 8};
+  return {true, 2, 16};
+}
+
 inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || v == TCU_VARIANT_MFMA_256N_BLOCK || v == TCU_VARIANT_BLOCK_LDS; }
 
 // ----- segmented reduction ----------------------------------------------------------------
@@ -158,22 +185,27 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
   if (int rc = validate_segmented("tcu_seg_reduce_f16", d_in, d_out, a, &generic)) return rc;
   if (num_segments == 0) return TCU_OK;
   const size_t S = segment_size, N = num_segments * S;
-  const int wpb = waves_per_block ? waves_per_block : 4;
-  const unsigned block = (unsigned)wpb * 64u;
   const half8_t *in = static_cast<const half8_t *>(d_in);
   uint16_t *out = static_cast<uint16_t *>(d_out);
   const bool nt = options().nontemporal;
 
   if (generic) {
-    const size_t grid = (num_segments + wpb - 1) / wpb;
+    const int gw = waves_per_block ? waves_per_block : 4;
+    const size_t grid = (num_segments + gw - 1) / gw;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
-    launch(seg_reduce_generic_kernel, (unsigned)grid, block, stream, static_cast<const uint16_t *>(d_in), out, num_segments, S);
+    launch(seg_reduce_generic_kernel, (unsigned)grid, (unsigned)gw * 64u, stream, static_cast<const uint16_t *>(d_in), out, num_segments, S);
     return TCU_OK;
   }
   const size_t n_chunks = N / 8;
-  int u = tiles_per_wave ? tiles_per_wave : 8;
+  const Plan plan = auto_plan_reduce(S);
+  const bool use_block = variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant);
+  // explicit families keep their own tuned shape; AUTO and matching families use the plan
+  const bool plan_fits = variant == TCU_VARIANT_AUTO || plan.block == use_block;
+  const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 2 : 4));
+  const int wpb = waves_per_block ? waves_per_block : (plan_fits ? plan.w : (use_block ? 8 : 4));
+  const unsigned block = (unsigned)wpb * 64u;
 
-  if (is_block_variant(variant)) {
+  if (use_block) {
     const size_t tiles_per_seg = S / kTileHalves;
     const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;  // the reference's 16n_block owns 16 segments per block
     const size_t grid = (num_segments + spb - 1) / spb;
@@ -245,23 +277,27 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   if (int rc = validate_segmented("tcu_seg_scan_f16", d_in, d_out, a, &generic)) return rc;
   if (num_segments == 0) return TCU_OK;
   const size_t S = segment_size, N = num_segments * S;
-  const int wpb = waves_per_block ? waves_per_block : 4;
-  const unsigned block = (unsigned)wpb * 64u;
   const half8_t *in = static_cast<const half8_t *>(d_in);
   uint4_t *out = static_cast<uint4_t *>(d_out);
   uint16_t *totals = static_cast<uint16_t *>(d_totals);
   const bool nt = options().nontemporal;
 
   if (generic) {
-    const size_t grid = (num_segments + wpb - 1) / wpb;
+    const int gw = waves_per_block ? waves_per_block : 4;
+    const size_t grid = (num_segments + gw - 1) / gw;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: grid exceeds the launch limit");
-    launch(seg_scan_generic_kernel, (unsigned)grid, block, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), totals, num_segments, S);
+    launch(seg_scan_generic_kernel, (unsigned)grid, (unsigned)gw * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), totals, num_segments, S);
     return TCU_OK;
   }
   const size_t n_chunks = N / 8;
-  const int u = tiles_per_wave ? tiles_per_wave : 4;
+  const Plan plan = auto_plan_scan(S);
+  const bool use_block = variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant);
+  const bool plan_fits = variant == TCU_VARIANT_AUTO || plan.block == use_block;
+  const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 4 : 4));
+  const int wpb = waves_per_block ? waves_per_block : (plan_fits ? plan.w : (use_block ? 4 : 1));
+  const unsigned block = (unsigned)wpb * 64u;
 
-  if (is_block_variant(variant)) {
+  if (use_block) {
     const size_t tiles_per_seg = S / kTileHalves;
     const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;
     const size_t grid = (num_segments + spb - 1) / spb;
@@ -337,8 +373,6 @@ inline int plan_full(const char *what, size_t segment_size, int waves_per_block,
   return TCU_OK;
 }
 
-constexpr unsigned kFullReduceMaxBlocks = 2048;
-
 inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d_ws, size_t *ws_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream) {
   const char *what = "tcu_full_reduce_f16";
   if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
@@ -347,26 +381,29 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {
     FullPlan p;
-    if (int rc = plan_full(what, segment_size, waves_per_block, 16384, &p)) return rc;
-    const size_t need = 256 + 4 * (size_t)kFullReduceMaxBlocks;
+    if (int rc = plan_full(what, segment_size, waves_per_block ? waves_per_block : 8, 16384, &p)) return rc;
+    const bool vec = n % 8 == 0 && aligned16(d_in);
+    const size_t n_chunks = n / 8;
+    const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
+    size_t grid = (n_tiles + (size_t)p.wpb * p.u - 1) / ((size_t)p.wpb * p.u);
+    if (grid == 0) grid = 1;
+    const size_t groups = (grid + kFullReduceGroup - 1) / kFullReduceGroup;
+    const size_t need = round_up(4 * (64 + groups + grid + groups), kWorkspaceAlign);
     if (!d_ws) {
       *ws_bytes = need;
       return TCU_OK;
     }
     if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
     if (!d_out || (n && !d_in)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
-    if ((n % 8) != 0 || !aligned16(d_in)) {
+    if (!vec) {
       // odd sizes: one block over scalar loads
       launch(sum_f16_kernel, 1u, 1024u, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), n);
       return TCU_OK;
     }
-    const size_t n_chunks = n / 8;
-    const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
-    size_t grid = (n_tiles + (size_t)p.wpb * p.u - 1) / ((size_t)p.wpb * p.u);
-    if (grid > kFullReduceMaxBlocks) grid = kFullReduceMaxBlocks;
-    if (grid == 0) grid = 1;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     unsigned *ws = static_cast<unsigned *>(d_ws);
-    launch(zero_words_kernel, 1u, 256u, stream, ws, (size_t)64);
+    const size_t words = 64 + groups;
+    launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
     TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, false, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws);
     return TCU_OK;
   }
@@ -395,7 +432,7 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {
     FullPlan p;
-    if (int rc = plan_full(what, segment_size, waves_per_block, 8192, &p)) return rc;
+    if (int rc = plan_full(what, segment_size, waves_per_block ? waves_per_block : 16, 65536, &p)) return rc;
     if (n % 8 != 0 || !aligned16(d_in) || !aligned16(d_out)) {
       if (!d_ws) {
         *ws_bytes = kWorkspaceAlign;
@@ -421,7 +458,7 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
     unsigned *ws = static_cast<unsigned *>(d_ws);
     const size_t words = 64 + 2 * parts;
     launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
-    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, false, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws);
+    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, false, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0);
     return TCU_OK;
   }
   // the reference's three-kernel sequence: segmented scan + totals, exclusive scan of the totals, add

@@ -31,7 +31,17 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned *words, size_t
   if (i < n) words[i] = 0u;
 }
 
-// workspace: counter at words[0]; partials (float) start at word 64
+// One partition (blockDim/64 * U tiles) per block, no loop: blocks dispatched in order sweep
+// the array as one moving window, which is what HBM serves fastest (a persistent
+// grid-stride version of this kernel measured 2-3x slower).  Completion is detected with
+// two levels of tickets so that no counter sees more than 64 + blocks/64 atomics
+// (same-address device-scope atomics retire at roughly one per 11 ns on this part):
+// groups of 64 consecutive blocks share a counter; the last block of a group adds the
+// group's partials, the last group adds the group sums and writes the result.  All sums
+// run in index order, so the result does not depend on timing.
+// workspace words: [0] top counter, [64 .. 64+groups) group counters, then
+// float partial[blocks], float group_sum[groups].
+constexpr unsigned kFullReduceGroup = 64;
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, unsigned *ws) {
   __shared__ float partial[kMaxWaves];
@@ -39,53 +49,64 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   const int lane = lane_id();
   const int wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
-  float *partials = reinterpret_cast<float *>(ws + 64);
+  const unsigned n_blocks = gridDim.x;
+  const unsigned n_groups = (n_blocks + kFullReduceGroup - 1) / kFullReduceGroup;
+  unsigned *group_counter = ws + 64;
+  float *partials = reinterpret_cast<float *>(ws + 64 + n_groups);
+  float *group_sum = partials + n_blocks;
   const half8_t ones = splat8(1.0f);
-  const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
-  const size_t stride = (size_t)gridDim.x * WPB * U;
 
-  float accs[2] = {0.0f, 0.0f};
-  float4_t accm = {0, 0, 0, 0};
-  for (size_t t0 = ((size_t)blockIdx.x * WPB + wave) * U; t0 < n_tiles; t0 += stride) {
-    half8_t v[U];
-    load_tiles<U, NT>(v, in, t0 * kTileChunks, n_chunks, lane);
-#pragma unroll
-    for (int j = 0; j < U; j++) {
-      if constexpr (MFMA)
-        accm = mfma_16x16x32(v[j], ones, accm);
-      else
-        accs[j & 1] = sum8(v[j], accs[j & 1]);
-    }
-  }
+  half8_t v[U];
+  load_tiles<U, NT>(v, in, ((size_t)blockIdx.x * WPB + wave) * U * kTileChunks, n_chunks, lane);
   float total;
-  if constexpr (MFMA)
+  if constexpr (MFMA) {
+    float4_t accm = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < U; j++) accm = mfma_16x16x32(v[j], ones, accm);
     total = add_xor32(add_xor16((accm[0] + accm[1]) + (accm[2] + accm[3])));
-  else
+  } else {
+    float accs[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < U; j++) accs[j & 1] = sum8(v[j], accs[j & 1]);
     total = lane_group_sum<6>(accs[0] + accs[1]);
+  }
   if (lane == 63) partial[wave] = total;
   __syncthreads();
+  const unsigned g = blockIdx.x / kFullReduceGroup;
   if (threadIdx.x == 0) {
     float s = 0.0f;
     for (int w = 0; w < WPB; w++) s += partial[w];
     partials[blockIdx.x] = s;
     device_fence_release();
-    ticket = atomic_add_u32_acq_rel(ws, 1u);
+    ticket = atomic_add_u32_acq_rel(group_counter + g, 1u);
   }
   __syncthreads();
-  if (ticket != gridDim.x - 1) return;  // block-uniform
-  if (wave == 0) {
-    device_fence_acquire();
-    float s = 0.0f;
-    for (unsigned i = lane; i < gridDim.x; i += 64) s += atomic_load_f32(partials + i);
-    s = lane_group_sum<6>(s);
-    if (lane == 63) out[0] = f16_bits(s);
+  const unsigned first = g * kFullReduceGroup;
+  const unsigned members = n_blocks - first < kFullReduceGroup ? n_blocks - first : kFullReduceGroup;
+  if (ticket != members - 1) return;  // block-uniform
+  if (wave != 0) return;
+  device_fence_acquire();
+  float s = lane < (int)members ? atomic_load_f32(partials + first + lane) : 0.0f;
+  s = lane_group_sum<6>(s);
+  unsigned top = 0;
+  if (lane == 63) {
+    group_sum[g] = s;
+    device_fence_release();
+    top = atomic_add_u32_acq_rel(ws, 1u);
   }
+  top = readlane_u32(top, 63);
+  if (top != n_groups - 1) return;  // wave-uniform
+  device_fence_acquire();
+  float t = 0.0f;
+  for (unsigned i = lane; i < n_groups; i += 64) t += atomic_load_f32(group_sum + i);
+  t = lane_group_sum<6>(t);
+  if (lane == 63) out[0] = f16_bits(t);
 }
 
 // One partition (blockDim/64 * U tiles) per block.  workspace: ticket counter at word 0,
 // descriptors (64-bit: flag << 32 | float bits) from byte 256.
 template <int U, bool MFMA, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws) {
+__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order) {
   __shared__ float wave_total[kMaxWaves];
   __shared__ unsigned s_part;
   __shared__ float s_prefix;
@@ -96,9 +117,11 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   ScanOperands ops;
   if constexpr (MFMA) ops = make_scan_operands(lane);
 
-  if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
-  __syncthreads();
-  const unsigned part = s_part;
+  if (!static_order) {
+    if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
+    __syncthreads();
+  }
+  const unsigned part = static_order ? blockIdx.x : s_part;
   const size_t t0 = ((size_t)part * WPB + wave) * U;
 
   half8_t v[U];
@@ -119,6 +142,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
     } else {
       if (lane == 0) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
       long long base = (long long)part - 1;
+      unsigned polls = 0;
       while (true) {  // every lane of wave 0 takes the same path
         const long long idx = base - lane;
         unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : kFlagPrefix;
@@ -128,6 +152,10 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
         const int first_prefix = is_prefix ? __builtin_ctzll(is_prefix) : 64;
         const unsigned long long needed = first_prefix >= 63 ? ~0ull : ((2ull << first_prefix) - 1ull);
         if (is_empty & needed) {
+          if (++polls > (1u << 20)) {  // give up: never spin without bound
+            if (lane == 0) atomic_add_u32(ws + 1, 1u);
+            break;
+          }
           spin_pause();
           continue;
         }

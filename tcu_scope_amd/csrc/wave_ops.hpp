@@ -127,9 +127,12 @@ TCU_DEVICE half8_t load_chunk(const half8_t *p) {
   if constexpr (NT) return __builtin_nontemporal_load(p);
   return *p;
 }
+#ifndef TCU_STORE_NT
+#define TCU_STORE_NT 1
+#endif
 template <bool NT>
 TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
-  if constexpr (NT)
+  if constexpr (NT && TCU_STORE_NT)
     __builtin_nontemporal_store(v, p);
   else
     *p = v;

@@ -1,0 +1,34 @@
+// GEMM / GEMV benchmarks under the reference's names (src/gemm/wmma.cu:776, wmma_naive.cu:339,
+// wmma_sharedmem.cu, src/gemv/wmma_naive.cu:357, wmma_sharedmem.cu) and the timed CPU path.
+#include "args.hpp"
+#include "harness.hpp"
+
+static void CUDA_WMMA_GEMM(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_BLOCK_LDS, "CUDA_WMMA_GEMM"); }
+static void CUDA_WMMA_GEMM_SHAREDMEM(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_BLOCK_LDS, "CUDA_WMMA_GEMM_SHAREDMEM"); }
+static void CUDA_WMMA_GEMM_NAIVE(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMM_NAIVE"); }
+BENCHMARK(CUDA_WMMA_GEMM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_GEMM_SHAREDMEM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_GEMM_NAIVE)->Apply(GemmArgs)->UseManualTime();
+
+static void CUDA_WMMA_GEMV_NAIVE(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMV_NAIVE"); }
+static void CUDA_WMMA_GEMV_SHAREDMEM(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMV_SHAREDMEM"); }
+static void TCU_WAVE_GEMV(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_WAVE_SHUFFLE, "TCU_WAVE_GEMV"); }
+BENCHMARK(CUDA_WMMA_GEMV_NAIVE)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_GEMV_SHAREDMEM)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(TCU_WAVE_GEMV)->Apply(GemvArgs)->UseManualTime();
+
+// The reference's CPU verification loop as a benchmark: N = 2^20 in segments of 16 (seed 0),
+// one thread (as the reference wrote it) and all host threads.
+static void CPU_SEQUENTIAL_SEGMENTED_REDUCTION(benchmark::State &state) { harness::run_cpu_segmented(state, false, 1); }
+static void CPU_THREADED_SEGMENTED_REDUCTION(benchmark::State &state) { harness::run_cpu_segmented(state, false, 0); }
+static void CPU_SEQUENTIAL_SEGMENTED_PREFIXSUM(benchmark::State &state) { harness::run_cpu_segmented(state, true, 1); }
+static void CPU_THREADED_SEGMENTED_PREFIXSUM(benchmark::State &state) { harness::run_cpu_segmented(state, true, 0); }
+static void CpuArgs(benchmark::internal::Benchmark *b) {
+  b->Args({65536, 16, 1 << 20});
+  for (int64_t seg : {16, 256, 1024, 4096, 16384}) b->Args({(int64_t(1) << 26) / seg, seg, int64_t(1) << 26});
+  b->ArgNames({"num_segments", "segment_size", "num_elements"});
+}
+BENCHMARK(CPU_SEQUENTIAL_SEGMENTED_REDUCTION)->Apply(CpuArgs)->UseManualTime();
+BENCHMARK(CPU_THREADED_SEGMENTED_REDUCTION)->Apply(CpuArgs)->UseManualTime();
+BENCHMARK(CPU_SEQUENTIAL_SEGMENTED_PREFIXSUM)->Apply(CpuArgs)->UseManualTime();
+BENCHMARK(CPU_THREADED_SEGMENTED_PREFIXSUM)->Apply(CpuArgs)->UseManualTime();

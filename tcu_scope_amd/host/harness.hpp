@@ -1,0 +1,97 @@
+// Shared host-side pieces of the benchmark harnesses: flags, HIP error plumbing, device
+// buffers, seeded inputs, verification against a CPU sum, and the timed loops.
+// The shape of every harness follows the reference's (e.g. src/reduction/seg_wmma_16n.cu:12-178):
+// validate arguments -> allocate -> fill -> [verify] -> timed loop with an event pair around
+// each launch -> counters; any failure becomes state.SkipWithError.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/tcu_scope.h"
+#include "minibench.hpp"
+
+namespace harness {
+
+struct Flags {
+  int cuda_device_id = 0;            // --cuda_device_id (name kept from the reference, src/init/flags.cpp:4)
+  std::string input = "uniform";     // --tcu_input=uniform|constant|grid   (constant = the reference's 0.001 fill)
+  std::string verify = "auto";       // --tcu_verify=auto|all|none          (auto: up to 2^26 elements)
+  uint64_t seed = 1;                 // --tcu_seed
+  int verbose = 0;                   // --v
+  bool help = false;                 // --help / -h
+};
+Flags &flags();
+// parses and removes the harness flags from argv (as the reference does before Google
+// Benchmark sees the command line, src/init/flags.cpp:9-23)
+void init_flags(int *argc, char **argv);
+// selects the device (--cuda_device_id, clamped to 0 when absent) and prints what it found
+bool init_device();
+
+struct hip_error : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+struct unsupported : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+void check_hip(hipError_t e, const char *expr, const char *file, int line);
+void check_tcu(int status, const char *expr);
+#define PRINT_IF_ERROR(expr) ::harness::check_hip((expr), #expr, __FILE__, __LINE__)
+#define TCU_CHECK(expr) ::harness::check_tcu((expr), #expr)
+
+class DeviceBuffer {
+ public:
+  DeviceBuffer() = default;
+  explicit DeviceBuffer(size_t bytes);
+  ~DeviceBuffer();
+  DeviceBuffer(const DeviceBuffer &) = delete;
+  DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+  void *get() const { return p_; }
+  size_t bytes() const { return n_; }
+
+ private:
+  void *p_ = nullptr;
+  size_t n_ = 0;
+};
+
+class EventPair {
+ public:
+  EventPair();
+  ~EventPair();
+  void start();
+  float stop_ms();  // records stop, waits for it, returns the elapsed time
+
+ private:
+  hipEvent_t a_, b_;
+};
+
+// host fp16 helpers (bit recipe of reference src/utils/fp16_conversion.hpp:91-114 for the
+// widening direction; round-to-nearest-even for the narrowing one)
+float half_to_float(uint16_t h);
+uint16_t float_to_half(float f);
+
+// fills d (n halves) according to --tcu_input
+void fill_input(void *d, size_t n, uint64_t seed);
+inline const char *input_dist_name() { return flags().input.c_str(); }
+bool should_verify(size_t num_elements);
+
+// |got - fp64 sum| <= 2 ulp_fp16(result) + 1e-3 * sqrt(segment size); throws on mismatch
+void verify_seg_reduce(const void *d_in, const void *d_out, size_t num_segments, size_t segment_size, const char *what);
+void verify_seg_scan(const void *d_in, const void *d_out, size_t num_segments, size_t segment_size, const char *what);
+
+// timed loops; `expected_segment_size` = 0 accepts any size the variant supports
+void run_seg_reduce(benchmark::State &state, int variant, int tiles_per_wave, int waves_per_block, const char *name);
+void run_seg_scan(benchmark::State &state, int variant, int tiles_per_wave, int waves_per_block, bool with_totals, const char *name);
+void run_full_reduce(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
+void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
+void run_gemv(benchmark::State &state, int variant, const char *name);
+void run_gemm(benchmark::State &state, int variant, const char *name);
+// the reference's CPU verification loop (fp32 running sum per segment, fp16 result) timed on
+// `threads` host threads; scan = prefix sums instead of totals
+void run_cpu_segmented(benchmark::State &state, bool scan, int threads);
+
+}  // namespace harness

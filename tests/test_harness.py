@@ -1,0 +1,70 @@
+"""The C++ benchmark harness: names and argument grammar on the CPU, real runs on the GPU."""
+import json
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BENCH = os.path.join(ROOT, "tcu_scope_amd", "host", "bench")
+
+
+def _bench():
+    if not os.path.exists(BENCH):
+        subprocess.check_call(["make", "-C", os.path.dirname(BENCH)], stdout=subprocess.DEVNULL)
+    return BENCH
+
+
+def test_benchmark_names_follow_the_reference_grammar():
+    names = subprocess.check_output([_bench(), "--benchmark_list_tests"], text=True).split("\n")
+    names = [n for n in names if n]
+    have = set(names)
+    # spot checks taken from the reference's registrations and plot specs
+    for n in [
+        "CUDA_WMMA_SEGMENTED_REDUCTION_16<1, 8>/num_segments:16777216/segment_size:16/num_elements:268435456/manual_time",
+        "CUDA_WMMA_SEGMENTED_REDUCTION_16N<8>/num_segments:16777216/segment_size:16/num_elements:268435456/manual_time",
+        "CUDA_WMMA_SEGMENTED_REDUCTION_256<4, 2>/num_segments:1048576/segment_size:256/num_elements:268435456/manual_time",
+        "CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK<16>/num_segments:16384/segment_size:16384/num_elements:268435456/manual_time",
+        "CUDA_WMMA_TUNE_SEGMENTED_REDUCTION_256N<4>/num_segments:4194304/segment_size:256/base_segment_size:256/max_elements_log2:30/manual_time",
+        "CUB_WARP_SEGMENTED_REDUCTION<256, 16>/num_segments:16777216/segment_size:16/num_elements:268435456/manual_time",
+        "CUB_BLOCK_SEGMENTED_PREFIXSUM<512, 32, BLOCK_SCAN_RAKING>/num_segments:16384/segment_size:16384/num_elements:268435456/manual_time",
+        "CUDA_WMMA_SEGMENTED_PREFIXSUM_16<4, 2>/num_segments:16777216/segment_size:16/num_elements:268435456/manual_time",
+        "CUDA_WMMA_SEGMENTED_PREFIXSUM_256N<2>/num_segments:131072/segment_size:2048/num_elements:268435456/manual_time",
+        "CUDA_WMMA_FULL_REDUCTION_2KERS_BASE_16<2 * 256, 1>/num_elements:4096/manual_time",
+        "CUDA_WMMA_FULL_REDUCTION_ATOMIC_W_ATOMIC_BALLOT<4 * 256, 4>/num_elements:1073741824/manual_time",
+        "CUDA_WMMA_FULL_PREFIXSUM_3KERS<8 * 256, 8>/num_elements:1073741824/manual_time",
+        "CUDA_WMMA_GEMM/M:8192/N:8192/K:8192/manual_time",
+        "CUDA_WMMA_GEMM_NAIVE/M:8192/N:8192/K:8192/manual_time",
+        "CUDA_WMMA_GEMV_NAIVE/M:16384/N:16384/manual_time",
+        "CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/segment_size:16/num_elements:1048576/manual_time",
+    ]:
+        assert n in have, n
+    # the filter is a regular expression over those names
+    out = subprocess.check_output([_bench(), "--benchmark_list_tests", "--benchmark_filter=CUDA_WMMA_SEGMENTED_REDUCTION_16N<(4|8)>.*segment_size:256/"], text=True).split()
+    assert len(out) == 2 * 19 and all(re.search(r"_16N<(4|8)>", n) for n in out)
+
+
+@pytest.mark.gpu
+def test_harness_runs_verifies_and_reports(tmp_path):
+    out = tmp_path / "out.json"
+    filt = ("(CUDA_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16<1, 4>|256<1, 4>|16N<4>|256N<4>|256N_BLOCK<4>)|CUB_(WARP|BLOCK)_SEGMENTED_(REDUCTION|PREFIXSUM)<(256, 16|512, 32, BLOCK_(SCAN|REDUCE)_RAKING)>"
+            "|TCU_AUTO_SEGMENTED_(REDUCTION|PREFIXSUM))/.*num_elements:4194304/"
+            "|CUDA_WMMA_FULL_(REDUCTION_(2KERS_BASE_16|ATOMIC_W_BLOCK_SYNC)|PREFIXSUM_(3KERS|CG))<8 \\* 256, 4>/num_elements:4194304/"
+            "|CUDA_WMMA_GEM[MV](_NAIVE)?/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/")
+    p = subprocess.run([BENCH, f"--benchmark_filter={filt}", "--benchmark_min_time=0.02", f"--benchmark_out={out}", "--benchmark_out_format=json", "--tcu_verify=all", "--v=1"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "ERROR OCCURRED" not in p.stdout, p.stdout
+    data = json.loads(out.read_text())
+    rows = data["benchmarks"]
+    assert len(rows) >= 40
+    for r in rows:
+        assert r["iterations"] >= 1 and r["real_time"] > 0 and r["flops"] > 0, r
+        assert r["name"].endswith("/manual_time")
+    # precondition failures surface as skipped benchmarks, as in the reference
+    p = subprocess.run([BENCH, "--benchmark_filter=CUDA_WMMA_FULL_REDUCTION_2KERS_BASE_16<16 \\* 256, 1>/num_elements:4096/", "--benchmark_min_time=0.01"], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0 and "ERROR OCCURRED" not in p.stdout  # 4096 is a multiple of 4096: runs
+    p = subprocess.run([BENCH, "--benchmark_filter=CUDA_WMMA_SEGMENTED_REDUCTION_16N_BLOCK<4>/.*segment_size:512/num_elements:4096/", "--tcu_input=constant", "--benchmark_min_time=0.01"],
+                       capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0 and "ERROR OCCURRED" not in p.stdout, p.stdout
