@@ -61,7 +61,8 @@ def main():
     ap.add_argument("--tiles-per-wave", type=int, default=0)
     ap.add_argument("--waves-per-block", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-n-log2", type=int, default=26, help="element count of the CPU-baseline sample")
+    ap.add_argument("--with-copy-probe", action="store_true", help="also launch the plain copy kernel over 2^n_log2 halves before timing (calibrates hardware counters)")
+    ap.add_argument("--cpu-n-log2", type=int, default=28, help="element count of the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (--gpus 1); segments are independent, so a multi-GPU run would be N copies of this one", file=sys.stderr)
@@ -101,6 +102,11 @@ def main():
             tcu.seg_reduce(x, seg, variant=v, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=red_out, stream=stream)
         else:
             tcu.seg_scan(x, seg, variant=v, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=scan_out, stream=stream)
+
+    if args.with_copy_probe:
+        for i in range(4):  # 2*n bytes read + 2*n bytes written per launch, same launch shape as the scan kernels
+            tcu.stream_probe(scan_out, inputs[i & 1], 2 * n, 0, 1, 1, stream=stream)
+        torch.cuda.synchronize()
 
     counter = 0
     for _ in range(args.warmup):
