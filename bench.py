@@ -27,6 +27,15 @@ REDUCE_SEGS = [16, 256, 1024, 4096, 16384]
 SCAN_SEGS = [16, 256, 2048, 16384]
 
 
+# HBM bytes per launch at N = 2^28 with the AUTO launch shapes, from rocprofv3 FETCH_SIZE /
+# WRITE_SIZE runs of this script, each counter scaled by what it reads for the plain copy
+# kernel of known size (profiles/seg_reduce_scan_2p28_hbm_traffic.md).
+MEASURED_TRAFFIC_2P28_AUTO = {
+    ("reduce", 16): 570418104, ("reduce", 256): 538967188, ("reduce", 1024): 537931321, ("reduce", 4096): 537926153, ("reduce", 16384): 537138026,
+    ("scan", 16): 1073751645, ("scan", 256): 1073705869, ("scan", 2048): 1073579459, ("scan", 16384): 1073566659,
+}
+
+
 def algorithmic_bytes(kind, n, seg):
     # reduce: read N halves, write N/seg halves; scan: read N, write N
     return 2 * n + (2 * n // seg if kind == "reduce" else 2 * n)
@@ -132,6 +141,7 @@ def main():
     elems_per_step = len(configs) * n
     value = args.steps * elems_per_step / total_s / 1e9
 
+    measured_shapes = args.n_log2 == 28 and variant == tcu.Variant.AUTO and args.tiles_per_wave == 0 and args.waves_per_block == 0
     per_config = []
     for c, (kind, seg) in enumerate(configs):
         ms = sorted(events[k][c][0].elapsed_time(events[k][c][1]) for k in range(args.steps))
@@ -141,12 +151,13 @@ def main():
             "op": kind, "segment_size": seg, "avg_ms": round(avg, 5), "min_ms": round(ms[0], 5), "median_ms": round(ms[len(ms) // 2], 5),
             "gelem_per_s": round(n / avg / 1e6, 1), "algorithmic_bytes": by, "gb_per_s": round(by / avg / 1e6, 1),
             "frac_hbm_peak": round(by / avg / 1e6 / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_2P28_AUTO.get((kind, seg)) if measured_shapes else None,
         })
     # the dominant kernel: the launch that takes the largest share of a step
     dom = max(per_config, key=lambda r: r["avg_ms"])
     roofline = {
         "bound": "hbm", "kernel": f"seg_{dom['op']} segment_size={dom['segment_size']}", "achieved": dom["gb_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": dom["frac_hbm_peak"], "traffic": None, "algorithmic_bytes_per_launch": dom["algorithmic_bytes"], "avg_launch_ms": dom["avg_ms"],
+        "frac": dom["frac_hbm_peak"], "traffic": dom["traffic"], "algorithmic_bytes_per_launch": dom["algorithmic_bytes"], "avg_launch_ms": dom["avg_ms"],
         "min_frac_over_sweep": min(r["frac_hbm_peak"] for r in per_config),
     }
 
