@@ -381,14 +381,16 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {
     FullPlan p;
-    if (int rc = plan_full(what, segment_size, waves_per_block ? waves_per_block : 8, 16384, &p)) return rc;
+    if (int rc = plan_full(what, segment_size, waves_per_block ? waves_per_block : 16, 65536, &p)) return rc;
     const bool vec = n % 8 == 0 && aligned16(d_in);
     const size_t n_chunks = n / 8;
     const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
     size_t grid = (n_tiles + (size_t)p.wpb * p.u - 1) / ((size_t)p.wpb * p.u);
     if (grid == 0) grid = 1;
     const size_t groups = (grid + kFullReduceGroup - 1) / kFullReduceGroup;
-    const size_t need = round_up(4 * (64 + groups + grid + groups), kWorkspaceAlign);
+    const size_t counter_words = 64 + ((groups + 1) & ~(size_t)1);
+    const size_t words = counter_words + 2 * (grid + groups);
+    const size_t need = round_up(4 * words, kWorkspaceAlign);
     if (!d_ws) {
       *ws_bytes = need;
       return TCU_OK;
@@ -402,7 +404,6 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
     }
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     unsigned *ws = static_cast<unsigned *>(d_ws);
-    const size_t words = 64 + groups;
     launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
     TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, false, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws);
     return TCU_OK;
@@ -506,6 +507,18 @@ inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t
       launch(gemv_mfma_kernel<true>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
     else
       launch(gemv_mfma_kernel<false>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+    return TCU_OK;
+  }
+  const size_t k_tiles = (K / 8 + 63) / 64;
+  if (k_tiles >= 8) {  // rows of 8 KiB and more: block per pair of rows
+    constexpr int BROWS = 2, BU = 4;
+    const unsigned bw = k_tiles >= 32 ? 8u : k_tiles >= 16 ? 4u : 2u;
+    const size_t bgrid = (M + BROWS - 1) / BROWS;
+    if (bgrid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    if (nt)
+      launch(gemv_block_kernel<BROWS, BU, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
+    else
+      launch(gemv_block_kernel<BROWS, BU, false>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
     return TCU_OK;
   }
   constexpr int ROWS = 2, UK = 4;

@@ -33,15 +33,37 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned *words, size_t
 
 // One partition (blockDim/64 * U tiles) per block, no loop: blocks dispatched in order sweep
 // the array as one moving window, which is what HBM serves fastest (a persistent
-// grid-stride version of this kernel measured 2-3x slower).  Completion is detected with
-// two levels of tickets so that no counter sees more than 64 + blocks/64 atomics
-// (same-address device-scope atomics retire at roughly one per 11 ns on this part):
-// groups of 64 consecutive blocks share a counter; the last block of a group adds the
-// group's partials, the last group adds the group sums and writes the result.  All sums
-// run in index order, so the result does not depend on timing.
-// workspace words: [0] top counter, [64 .. 64+groups) group counters, then
-// float partial[blocks], float group_sum[groups].
+// grid-stride version of this kernel measured 2-3x slower).
+// Completion is detected without fences (an agent-scope release/acquire pair per block costs
+// about 90 ns of L2 write-back/invalidate and made this kernel 20x slower than the data
+// movement) and without a hot counter (same-address device-scope atomics retire at about
+// one per 11 ns): every block publishes {1, partial} as ONE 64-bit word, then takes a
+// ticket from the counter of its group of 64 blocks; the block that draws the last ticket
+// of a group reads the group's 64 words (polling the few that may still be in flight),
+// publishes the group sum the same way and takes a ticket from the top counter; the last
+// group adds the group sums and writes the result.  All sums run in index order, so the
+// result does not depend on timing.
+// workspace words: [0] top counter, [64 .. 64+groups) group counters, then (8-byte
+// aligned) u64 partial[blocks], u64 group_sum[groups]; all zeroed before the launch.
 constexpr unsigned kFullReduceGroup = 64;
+constexpr unsigned long long kPublished = 1ull << 32;
+constexpr unsigned kPublishPollLimit = 1u << 22;
+
+// sum over lanes of the published values at p[lane], lane < count (count <= 64); false if a
+// value never showed up
+TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, int lane, float *sum) {
+  unsigned long long d = kPublished;
+  for (unsigned polls = 0;; polls++) {
+    if ((unsigned)lane < count) d = atomic_load_u64(p + lane);
+    if (ballot((d >> 32) == 1ull) == ~0ull) break;
+    if (polls > kPublishPollLimit) return false;
+    spin_pause();
+  }
+  const float v = (unsigned)lane < count ? __uint_as_float((unsigned)d) : 0.0f;
+  *sum = readlane(lane_group_sum<6>(v), 63);
+  return true;
+}
+
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, unsigned *ws) {
   __shared__ float partial[kMaxWaves];
@@ -52,8 +74,8 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   const unsigned n_blocks = gridDim.x;
   const unsigned n_groups = (n_blocks + kFullReduceGroup - 1) / kFullReduceGroup;
   unsigned *group_counter = ws + 64;
-  float *partials = reinterpret_cast<float *>(ws + 64 + n_groups);
-  float *group_sum = partials + n_blocks;
+  unsigned long long *partials = reinterpret_cast<unsigned long long *>(ws + 64 + ((n_groups + 1) & ~1u));
+  unsigned long long *group_sum = partials + n_blocks;
   const half8_t ones = splat8(1.0f);
 
   half8_t v[U];
@@ -76,31 +98,38 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   if (threadIdx.x == 0) {
     float s = 0.0f;
     for (int w = 0; w < WPB; w++) s += partial[w];
-    partials[blockIdx.x] = s;
-    device_fence_release();
-    ticket = atomic_add_u32_acq_rel(group_counter + g, 1u);
+    atomic_store_u64(partials + blockIdx.x, kPublished | __float_as_uint(s));
+    ticket = atomic_add_u32(group_counter + g, 1u);
   }
   __syncthreads();
   const unsigned first = g * kFullReduceGroup;
   const unsigned members = n_blocks - first < kFullReduceGroup ? n_blocks - first : kFullReduceGroup;
   if (ticket != members - 1) return;  // block-uniform
   if (wave != 0) return;
-  device_fence_acquire();
-  float s = lane < (int)members ? atomic_load_f32(partials + first + lane) : 0.0f;
-  s = lane_group_sum<6>(s);
+  const uint16_t failed = 0x7e00u;  // NaN: a published value never became visible
+  float s;
+  if (!gather_published(partials + first, members, lane, &s)) {
+    if (lane == 0) out[0] = failed;
+    return;
+  }
   unsigned top = 0;
   if (lane == 63) {
-    group_sum[g] = s;
-    device_fence_release();
-    top = atomic_add_u32_acq_rel(ws, 1u);
+    atomic_store_u64(group_sum + g, kPublished | __float_as_uint(s));
+    top = atomic_add_u32(ws, 1u);
   }
   top = readlane_u32(top, 63);
   if (top != n_groups - 1) return;  // wave-uniform
-  device_fence_acquire();
   float t = 0.0f;
-  for (unsigned i = lane; i < n_groups; i += 64) t += atomic_load_f32(group_sum + i);
-  t = lane_group_sum<6>(t);
-  if (lane == 63) out[0] = f16_bits(t);
+  for (unsigned base = 0; base < n_groups; base += 64) {
+    const unsigned count = n_groups - base < 64 ? n_groups - base : 64;
+    float part;
+    if (!gather_published(group_sum + base, count, lane, &part)) {
+      if (lane == 0) out[0] = failed;
+      return;
+    }
+    t += part;
+  }
+  if (lane == 0) out[0] = f16_bits(t);
 }
 
 // One partition (blockDim/64 * U tiles) per block.  workspace: ticket counter at word 0,

@@ -5,6 +5,8 @@
 //                      128-bit chunk of x and the matching chunk of each row (a wave reads
 //                      1 KiB of a row contiguously), multiplies with packed fp16 dot
 //                      products into fp32, and finishes with a DPP wave reduction.
+//   gemv_block_kernel: rows of 8 KiB and more: a block of waves shares two rows (the access
+//                      shape of the block-per-segment reduction), partials meet in LDS.
 //   gemv_mfma_kernel : the reference's formulation (GEMV as a 16-wide GEMM,
 //                      src/gemv/wmma_naive.cu:29-94): a wave owns a 16-row strip, the strip
 //                      is the A operand of v_mfma_f32_16x16x32_f16 and x, replicated over
@@ -65,7 +67,54 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__re
   }
 }
 
-// K must be a multiple of 128.  One wave per 16-row strip.
+// Long rows: a block of WPB waves shares ROWS consecutive rows; wave w takes the tiles
+// w*U .. w*U+U-1 of every step of WPB*U tiles (the x chunks it loads serve all ROWS rows),
+// partial dot products meet in LDS.  Same access shape as the block-per-segment reduction,
+// which is what moves long contiguous rows fastest.
+template <int ROWS, int U, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, float *__restrict__ y, size_t M, size_t k_chunks, float alpha,
+                                                                float beta) {
+  __shared__ float partial[ROWS][kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  const size_t row0 = (size_t)blockIdx.x * ROWS;
+  const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  float acc[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+  for (size_t c0 = (size_t)wave * U * 64; c0 < k_chunks; c0 += (size_t)WPB * U * 64) {
+    half8_t xv[U], av[ROWS][U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t c = c0 + (size_t)u * 64 + lane;
+      const bool ok = c < k_chunks;
+      xv[u] = ok ? x[c] : zero;
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        const size_t row = row0 + r < M ? row0 + r : M - 1;
+        av[r][u] = ok ? load_chunk<NT>(A + row * k_chunks + c) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) acc[r] = dot8(av[r][u], xv[u], acc[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; r++) {
+    const float s = lane_group_sum<6>(acc[r]);
+    if (lane == 63) partial[r][wave] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < ROWS && row0 + threadIdx.x < M) {
+    float s = 0.0f;
+    for (int w = 0; w < WPB; w++) s += partial[threadIdx.x][w];
+    float *p = y + row0 + threadIdx.x;
+    *p = beta == 0.0f ? alpha * s : alpha * s + beta * *p;
+  }
+}
+
+// K must be a multiple of 8.  One wave per 16-row strip.
 template <bool NT>
 __global__ __launch_bounds__(kMaxBlock) void gemv_mfma_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, float *__restrict__ y, size_t M, size_t k_chunks, float alpha,
                                                                float beta) {
@@ -77,7 +126,7 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_mfma_kernel(const half8_t *__r
   const size_t row = row0 + r < M ? row0 + r : M - 1;
   const half8_t *arow = A + row * k_chunks;
   float4_t acc = {0, 0, 0, 0};
-  // a step covers 128 k = 16 chunks; lane (r, b) takes chunks 4b .. 4b+3 of the step
+  // a step covers 256 k = 32 chunks in two halves; lane (r, b) takes chunks 4b .. 4b+3 of each half
   for (size_t c0 = 0; c0 < k_chunks; c0 += 32) {
     half8_t av[2][4], xv[2][4];
 #pragma unroll

@@ -1,0 +1,154 @@
+"""Runs the GPU kernel SOURCES (tcu_scope_amd/csrc/*.hpp) lane by lane on the CPU, through the same
+dispatch code the library uses, and compares with the oracle.  tests/emu/wave_ops_emu.hpp
+replaces the wave primitives (DPP, lane swaps, MFMA, ballot) by rendezvous between 64
+fibers per wave; it is strict about divergence around cross-lane operations.  This checks
+indexing, lane-layout arithmetic, masks and tails without a GPU; the hardware behaviour
+the emulation assumes is checked by tests/test_gpu_probe.py on the GPU."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+EMU = os.path.join(HERE, "emu")
+CLANG = "/opt/rocm/llvm/bin/clang++"
+
+V_AUTO, V_MFMA_16, V_MFMA_16N, V_MFMA_16N_BLOCK, V_MFMA_256, V_MFMA_256N, V_MFMA_256N_BLOCK, V_WAVE, V_BLOCK = range(9)
+
+
+@pytest.fixture(scope="module")
+def emu():
+    if not os.path.exists(CLANG):
+        pytest.skip("host clang++ (ROCm LLVM) not available")
+    lib = os.path.join(EMU, "libtcu_emu.so")
+    srcs = [os.path.join(EMU, f) for f in ("emu_driver.cpp", "wave_ops_emu.hpp")]
+    csrc = os.path.join(HERE, "..", "tcu_scope_amd", "csrc")
+    srcs += [os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith(".hpp")]
+    if not os.path.exists(lib) or any(os.path.getmtime(s) > os.path.getmtime(lib) for s in srcs):
+        subprocess.check_call([CLANG, "-x", "c++", "-std=c++17", "-O1", "-fPIC", "-shared", "-Wno-psabi", "-I" + EMU, "-o", lib, os.path.join(EMU, "emu_driver.cpp")])
+    L = ctypes.CDLL(lib)
+    sz, vp, ci, cf = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    L.emu_seg_reduce_f16.argtypes = [vp, vp, sz, sz, ci, ci, ci]
+    L.emu_seg_scan_f16.argtypes = [vp, vp, vp, sz, sz, ci, ci, ci]
+    L.emu_full_reduce_f16.argtypes = [vp, vp, sz, vp, ctypes.POINTER(sz), ci, sz, ci]
+    L.emu_full_scan_f16.argtypes = [vp, vp, sz, vp, ctypes.POINTER(sz), ci, sz, ci]
+    L.emu_gemv_f16_f32.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci]
+    L.emu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
+    L.emu_generate_f16.argtypes = [vp, sz, ctypes.c_uint64, ci, sz]
+    L.emu_last_error.restype = ctypes.c_char_p
+    return L
+
+
+def aligned(n, dtype, fill=None):
+    raw = np.zeros(n * np.dtype(dtype).itemsize + 256, np.uint8)
+    off = (-raw.ctypes.data) % 256
+    a = raw[off:off + n * np.dtype(dtype).itemsize].view(dtype)
+    if fill is not None:
+        a[:] = fill
+    return a
+
+
+def copy_in(x, dtype=np.uint16):
+    a = aligned(max(x.size, 1), dtype)
+    a[:x.size] = x
+    return a
+
+
+CASES = [  # (segment size, variants, (tiles per wave, waves per block) list, segment counts)
+    (16, (V_WAVE, V_MFMA_16, V_MFMA_16N, V_AUTO), ((8, 2), (1, 1)), (96, 1027)),
+    (64, (V_WAVE, V_MFMA_16N), ((4, 1),), (37,)),
+    (256, (V_WAVE, V_MFMA_256, V_MFMA_256N), ((2, 2), (8, 1)), (19,)),
+    (512, (V_WAVE, V_MFMA_16N, V_BLOCK, V_MFMA_256N_BLOCK), ((2, 1),), (9,)),
+    (2048, (V_WAVE, V_MFMA_256N, V_BLOCK, V_MFMA_16N_BLOCK, V_AUTO), ((2, 2), (8, 1)), (5,)),
+    (8192, (V_WAVE, V_MFMA_16N, V_MFMA_256N_BLOCK), ((4, 2),), (3,)),
+]
+
+
+@pytest.mark.parametrize("seg,variants,shapes,counts", CASES)
+def test_segmented_kernels_bit_exact_on_grid_inputs(emu, oracle, seg, variants, shapes, counts):
+    for nseg in counts:
+        x = oracle.generate_f16(nseg * seg, 17 + seg, oracle.DIST_GRID)  # exact partial sums: results are fixed bit for bit
+        sc = oracle.seg_scan_f64(x, nseg, seg)
+        want_scan = sc.astype(np.float16).view(np.uint16)
+        want_red = want_scan.reshape(nseg, seg)[:, -1]
+        xi = copy_in(x)
+        for v in variants:
+            for u, w in shapes:
+                red = aligned(nseg + 8, np.uint16, 0xFFFF)
+                assert emu.emu_seg_reduce_f16(xi.ctypes.data, red.ctypes.data, nseg, seg, v, u, w) == 0, emu.emu_last_error()
+                assert np.array_equal(red[:nseg], want_red) and np.all(red[nseg:] == 0xFFFF), ("reduce", seg, v, u, w, nseg)
+                out = aligned(nseg * seg + 64, np.uint16, 0xFFFF)
+                tot = aligned(nseg, np.uint16, 0xFFFF)
+                assert emu.emu_seg_scan_f16(xi.ctypes.data, out.ctypes.data, tot.ctypes.data, nseg, seg, v, u, w) == 0, emu.emu_last_error()
+                assert np.array_equal(out[:nseg * seg], want_scan) and np.all(out[nseg * seg:] == 0xFFFF), ("scan", seg, v, u, w, nseg)
+                assert np.array_equal(tot, want_red), ("scan totals", seg, v, u, w, nseg)
+
+
+def test_generic_segment_sizes_and_preconditions(emu, oracle):
+    for seg, nseg in ((1, 70), (7, 33), (100, 5)):
+        x = oracle.generate_f16(nseg * seg, 3, oracle.DIST_GRID)
+        sc = oracle.seg_scan_f64(x, nseg, seg).astype(np.float16).view(np.uint16)
+        xi = copy_in(x)
+        red = aligned(nseg, np.uint16)
+        out = aligned(nseg * seg, np.uint16)
+        assert emu.emu_seg_reduce_f16(xi.ctypes.data, red.ctypes.data, nseg, seg, V_AUTO, 0, 0) == 0
+        assert emu.emu_seg_scan_f16(xi.ctypes.data, out.ctypes.data, None, nseg, seg, V_AUTO, 0, 0) == 0
+        assert np.array_equal(out, sc) and np.array_equal(red, sc.reshape(nseg, seg)[:, -1])
+        assert emu.emu_seg_reduce_f16(xi.ctypes.data, red.ctypes.data, nseg, seg, V_WAVE, 0, 0) == 2
+    xi = copy_in(np.zeros(512, np.uint16))
+    assert emu.emu_seg_reduce_f16(xi.ctypes.data, xi.ctypes.data, 4, 32, V_MFMA_16, 0, 0) == 2 and b"must be 16" in emu.emu_last_error()
+    assert emu.emu_seg_scan_f16(xi.ctypes.data, xi.ctypes.data, None, 2, 256, V_BLOCK, 0, 0) == 2
+
+
+def test_full_array_kernels(emu, oracle):
+    sz = ctypes.c_size_t
+    for n in (8, 1003, 8192 * 3 + 1024, (1 << 16) + 56):
+        x = oracle.generate_f16(n, 5, oracle.DIST_GRID)
+        w64 = oracle.seg_scan_f64(x, 1, n)
+        xi = copy_in(x)
+        for strategy, seg, wpb in ((0, 0, 0), (1, 2048, 4), (1, 1024, 1), (2, 0, 0), (2, 256, 2)):
+            for op, fn in (("reduce", emu.emu_full_reduce_f16), ("scan", emu.emu_full_scan_f16)):
+                need = sz(0)
+                rc = fn(xi.ctypes.data, None, n, None, ctypes.byref(need), strategy, seg, wpb)
+                if rc == 2:
+                    assert strategy == 2 and n % (seg or 2048)
+                    continue
+                assert rc == 0
+                ws = aligned(need.value, np.uint8, 0xAB)  # the workspace needs no initialisation
+                out = aligned(n if op == "scan" else 1, np.uint16, 0xFFFF)
+                assert fn(xi.ctypes.data, out.ctypes.data, n, ws.ctypes.data, ctypes.byref(need), strategy, seg, wpb) == 0, emu.emu_last_error()
+                ref = w64 if op == "scan" else w64[-1:]
+                if strategy != 2:
+                    assert np.array_equal(out, ref.astype(np.float16).view(np.uint16)), (op, n, strategy, seg, wpb)
+                else:  # per-segment totals are rounded to fp16 on the way, as in the reference
+                    assert oracle.check_f16(out, ref, n)[0] == 0, (op, n, strategy, seg, wpb)
+
+
+def test_gemv_gemm_and_generator(emu, oracle):
+    for dist in (0, 1, 3):
+        out = aligned(5000, np.uint16)
+        assert emu.emu_generate_f16(out.ctypes.data, 5000, 42, dist, 77) == 0
+        assert np.array_equal(out, oracle.generate_f16(5000, 42, dist, first=77))
+    for M, K in ((64, 512), (37, 256), (5, 24), (7, 4608)):
+        A, x = oracle.generate_f16(M * K, 1, oracle.DIST_NORMAL), oracle.generate_f16(K, 2, oracle.DIST_NORMAL)
+        y0 = np.linspace(-1, 1, M).astype(np.float32)
+        Ai, xi = copy_in(A), copy_in(x)
+        for v in (V_AUTO, V_WAVE, V_MFMA_16N):
+            y = copy_in(y0, np.float32)
+            rc = emu.emu_gemv_f16_f32(Ai.ctypes.data, xi.ctypes.data, y.ctypes.data, M, K, 1.5, -0.5, v)
+            if rc == 2:
+                assert K % 8
+                continue
+            assert rc == 0 and oracle.check_f32_rel(y[:M], oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0), 1e-4, float(np.sqrt(K)))[0] == 0, (M, K, v)
+    for M, N, K in ((128, 128, 64), (64, 32, 48), (33, 17, 20)):
+        A, B = oracle.generate_f16(M * K, 5, oracle.DIST_SMALLINT), oracle.generate_f16(N * K, 6, oracle.DIST_SMALLINT)
+        C0 = (np.arange(M * N) % 7).astype(np.float32)
+        Ai, Bi, Ci = copy_in(A), copy_in(B), copy_in(C0, np.float32)
+        for v in (V_AUTO, V_BLOCK, V_MFMA_16N):
+            D = aligned(M * N, np.float32, -777)
+            rc = emu.emu_gemm_f16_f32(Ai.ctypes.data, Bi.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, K, 2.0, 3.0, v)
+            if rc == 2:
+                continue
+            assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A, B, M, N, K, 2.0, 3.0, C0)), (M, N, K, v)
