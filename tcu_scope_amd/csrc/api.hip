@@ -81,6 +81,14 @@ int tcu_set_option(const char *name, int value) {
     tcu::options().nontemporal = value != 0;
     return TCU_OK;
   }
+  if (std::strcmp(name, "gemm_big_tiles") == 0) {
+    tcu::options().gemm_big_tiles = value != 0;
+    return TCU_OK;
+  }
+  if (std::strcmp(name, "gemm_bk64") == 0) {
+    tcu::options().gemm_bk64 = value != 0;
+    return TCU_OK;
+  }
   if (std::strcmp(name, "static_order") == 0) {
     tcu::options().static_order = value != 0;
     return TCU_OK;

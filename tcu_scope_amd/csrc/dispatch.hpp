@@ -34,6 +34,8 @@ inline int fail(int code, const std::string &msg) {
 struct Options {
   bool nontemporal = true;
   bool static_order = false;
+  bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
+  bool gemm_bk64 = true;       // K step 64 where K allows
 };
 inline Options &options() {
   static Options o;
@@ -545,7 +547,14 @@ inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, s
   float *d = static_cast<float *>(D);
   if (variant == TCU_VARIANT_BLOCK_LDS && !lds_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the LDS kernel needs M, N multiples of 128 and K a multiple of 32");
   if (variant == TCU_VARIANT_MFMA_16N && !direct_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the direct kernel needs M, N multiples of 32 and K a multiple of 16");
-  if (lds_ok && variant != TCU_VARIANT_MFMA_16N) {
+  if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && options().gemm_big_tiles) {
+    const size_t grid = (M / kGemmBigBM) * (N / kGemmBigBN);
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    if (K % 64 == 0 && options().gemm_bk64)
+      launch(gemm_lds256_kernel<64>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+    else
+      launch(gemm_lds256_kernel<32>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+  } else if (lds_ok && variant != TCU_VARIANT_MFMA_16N) {
     const size_t grid = (M / kGemmBM) * (N / kGemmBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     launch(gemm_lds_kernel, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);

@@ -22,6 +22,8 @@ namespace tcu {
 constexpr int kGemmBM = 128, kGemmBN = 128, kGemmBK = 32;
 constexpr int kGemmLdsStride = 40;  // halves per LDS row (32 + 8 pad)
 
+TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_m, size_t *tile_n);
+
 TCU_DEVICE void gemm_store_tile(float *D, const float *C, size_t ldc, size_t row0, size_t col0, const float16_t &acc, int lane, float alpha, float beta) {
   const size_t col = col0 + (lane & 31);
 #pragma unroll
@@ -38,9 +40,8 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict
   __shared__ __attribute__((aligned(16))) half_t lds_b[2][kGemmBN * kGemmLdsStride];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  // block -> tile: consecutive blocks walk down a column of tiles so that they share B
-  const size_t tiles_m = M / kGemmBM;
-  const size_t tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+  size_t tile_m, tile_n;
+  gemm_tile_of_block(M / kGemmBM, N / kGemmBN, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
   // global -> LDS copy assignment: 128 rows x 4 chunks = 512 chunks per operand, 2 per thread
   const int crow = tid >> 2, cchunk = tid & 3;  // rows crow and crow + 64
@@ -102,6 +103,108 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict
   for (int i = 0; i < 2; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++) gemm_store_tile(D, C, N, tile_m * kGemmBM + wm * 64 + i * 32, tile_n * kGemmBN + wn * 64 + j * 32, acc[i][j], lane, alpha, beta);
+}
+
+// Block -> tile: the hardware deals consecutive block ids round-robin to the 8 XCDs, each
+// with its own L2.  Block ids are first regrouped so that an XCD owns a contiguous range of
+// tile ids, and tile ids walk bands of 4 tile rows column by column, so that the ~32 blocks
+// an XCD runs at a time form a 4 x 8 patch sharing A row panels and B column panels in L2.
+TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_m, size_t *tile_n) {
+  const size_t nb = tiles_m * tiles_n, b = blockIdx.x;
+  const size_t id = nb % 8 == 0 ? (b % 8) * (nb / 8) + b / 8 : b;
+  constexpr size_t GM = 4;
+  const size_t band = id / (GM * tiles_n);
+  const size_t rows = tiles_m - band * GM < GM ? tiles_m - band * GM : GM;
+  const size_t r = id - band * GM * tiles_n;
+  *tile_m = band * GM + r % rows;
+  *tile_n = r / rows;
+}
+
+// M % 256 == 0, N % 256 == 0, K % BK == 0; 256 threads.  256 x 256 x BK block tile, 2 x 2
+// waves of 128 x 128 (4 x 4 MFMA 32x32x16 accumulators = 256 registers, one wave per SIMD):
+// per 16-wide k substep a wave reads 8 fragments from LDS for 16 MFMAs, which leaves LDS
+// at half of its bandwidth.  BK = 64 makes a step long enough (about 0.85 us of MFMA) to
+// cover the latency of the next step's global loads; LDS rows are padded by 8 halves
+// (stride 72 halves: the 128-bit fragment reads of 16 lanes hit distinct banks).
+constexpr int kGemmBigBM = 256, kGemmBigBN = 256;
+template <int BK>
+__global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
+                                                          float beta) {
+  constexpr int STRIDE = BK + 8;            // halves per LDS row
+  constexpr int CPR = BK / 8;               // chunks per row
+  constexpr int RPP = 256 / CPR;            // rows copied per pass of the block
+  constexpr int PASSES = kGemmBigBM / RPP;  // passes per operand
+  __shared__ __attribute__((aligned(16))) half_t lds_a[2][kGemmBigBM * STRIDE];
+  __shared__ __attribute__((aligned(16))) half_t lds_b[2][kGemmBigBN * STRIDE];
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  size_t tile_m, tile_n;
+  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, &tile_m, &tile_n);
+  const size_t k_chunks = K / 8;
+  const int crow = tid / CPR, cchunk = tid % CPR;  // rows crow + RPP*i
+  const half8_t *ga = A + (tile_m * kGemmBigBM + crow) * k_chunks + cchunk;
+  const half8_t *gb = B + (tile_n * kGemmBigBN + crow) * k_chunks + cchunk;
+  const int so = crow * STRIDE + cchunk * 8;
+
+  float16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+  half8_t ra[PASSES], rb[PASSES];
+#pragma unroll
+  for (int i = 0; i < PASSES; i++) {
+    ra[i] = ga[(size_t)i * RPP * k_chunks];
+    rb[i] = gb[(size_t)i * RPP * k_chunks];
+  }
+#pragma unroll
+  for (int i = 0; i < PASSES; i++) {
+    *reinterpret_cast<half8_t *>(&lds_a[0][so + i * RPP * STRIDE]) = ra[i];
+    *reinterpret_cast<half8_t *>(&lds_b[0][so + i * RPP * STRIDE]) = rb[i];
+  }
+  __syncthreads();
+
+  const size_t steps = K / BK;
+  const int frow = lane & 31, fk = (lane >> 5) * 8;
+  for (size_t s = 0; s < steps; s++) {
+    const int cur = (int)(s & 1);
+    if (s + 1 < steps) {
+      const size_t o = (s + 1) * CPR;
+#pragma unroll
+      for (int i = 0; i < PASSES; i++) {
+        ra[i] = ga[(size_t)i * RPP * k_chunks + o];
+        rb[i] = gb[(size_t)i * RPP * k_chunks + o];
+      }
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; kk++) {
+      half8_t fa[4], fb[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) fa[i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][(wm * 128 + i * 32 + frow) * STRIDE + kk * 16 + fk]);
+#pragma unroll
+      for (int j = 0; j < 4; j++) fb[j] = *reinterpret_cast<const half8_t *>(&lds_b[cur][(wn * 128 + j * 32 + frow) * STRIDE + kk * 16 + fk]);
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[i], fb[j], acc[i][j]);
+    }
+    if (s + 1 < steps) {
+      const int nxt = cur ^ 1;
+#pragma unroll
+      for (int i = 0; i < PASSES; i++) {
+        *reinterpret_cast<half8_t *>(&lds_a[nxt][so + i * RPP * STRIDE]) = ra[i];
+        *reinterpret_cast<half8_t *>(&lds_b[nxt][so + i * RPP * STRIDE]) = rb[i];
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) gemm_store_tile(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 32, tile_n * kGemmBigBN + wn * 128 + j * 32, acc[i][j], lane, alpha, beta);
 }
 
 // M % 32 == 0, N % 32 == 0, K % 16 == 0; one 32 x 32 tile per wave.

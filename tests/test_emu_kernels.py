@@ -142,7 +142,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
                 assert K % 8
                 continue
             assert rc == 0 and oracle.check_f32_rel(y[:M], oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0), 1e-4, float(np.sqrt(K)))[0] == 0, (M, K, v)
-    for M, N, K in ((128, 128, 64), (64, 32, 48), (33, 17, 20)):
+    for M, N, K in ((128, 128, 64), (256, 512, 64), (64, 32, 48), (33, 17, 20)):
         A, B = oracle.generate_f16(M * K, 5, oracle.DIST_SMALLINT), oracle.generate_f16(N * K, 6, oracle.DIST_SMALLINT)
         C0 = (np.arange(M * N) % 7).astype(np.float32)
         Ai, Bi, Ci = copy_in(A), copy_in(B), copy_in(C0, np.float32)
