@@ -85,6 +85,10 @@ int tcu_set_option(const char *name, int value) {
     tcu::options().gemm_big_tiles = value != 0;
     return TCU_OK;
   }
+  if (std::strcmp(name, "gemm_depth") == 0) {
+    tcu::options().gemm_depth = value;
+    return TCU_OK;
+  }
   if (std::strcmp(name, "gemm_bk64") == 0) {
     tcu::options().gemm_bk64 = value != 0;
     return TCU_OK;

@@ -35,7 +35,8 @@ struct Options {
   bool nontemporal = true;
   bool static_order = false;
   bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
-  bool gemm_bk64 = true;       // K step 64 where K allows
+  bool gemm_bk64 = true;       // K step 64 (prefetch depth <= 2) where K allows
+  int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
 };
 inline Options &options() {
   static Options o;
@@ -550,10 +551,23 @@ inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, s
   if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && options().gemm_big_tiles) {
     const size_t grid = (M / kGemmBigBM) * (N / kGemmBigBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    if (K % 64 == 0 && options().gemm_bk64)
-      launch(gemm_lds256_kernel<64>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
-    else
-      launch(gemm_lds256_kernel<32>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+    const bool bk64 = K % 64 == 0 && options().gemm_bk64;
+    const size_t steps = K / (bk64 ? 64 : 32);
+    int depth = options().gemm_depth < 1 ? 1 : (options().gemm_depth > 4 ? 4 : options().gemm_depth);
+    if (bk64 && depth > 2) depth = 2;
+    while (steps % (size_t)depth) depth--;  // the kernels take whole groups of `depth` steps
+#define TCU_GEMM256(BK_, D_) launch(gemm_lds256_kernel<BK_, D_>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta)
+    if (bk64) {
+      if (depth == 2) TCU_GEMM256(64, 2); else TCU_GEMM256(64, 1);
+    } else {
+      switch (depth) {
+        case 4: TCU_GEMM256(32, 4); break;
+        case 3: TCU_GEMM256(32, 3); break;
+        case 2: TCU_GEMM256(32, 2); break;
+        default: TCU_GEMM256(32, 1); break;
+      }
+    }
+#undef TCU_GEMM256
   } else if (lds_ok && variant != TCU_VARIANT_MFMA_16N) {
     const size_t grid = (M / kGemmBM) * (N / kGemmBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");

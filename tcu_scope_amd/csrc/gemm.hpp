@@ -120,14 +120,17 @@ TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_
   *tile_n = r / rows;
 }
 
-// M % 256 == 0, N % 256 == 0, K % BK == 0; 256 threads.  256 x 256 x BK block tile, 2 x 2
+// M % 256 == 0, N % 256 == 0, K % (BK * DEPTH) == 0; 256 threads.  256 x 256 x BK block tile, 2 x 2
 // waves of 128 x 128 (4 x 4 MFMA 32x32x16 accumulators = 256 registers, one wave per SIMD):
 // per 16-wide k substep a wave reads 8 fragments from LDS for 16 MFMAs, which leaves LDS
-// at half of its bandwidth.  BK = 64 makes a step long enough (about 0.85 us of MFMA) to
-// cover the latency of the next step's global loads; LDS rows are padded by 8 halves
-// (stride 72 halves: the 128-bit fragment reads of 16 lanes hit distinct banks).
+// at half of its bandwidth.  With one wave per SIMD nothing else hides memory latency, so
+// the global loads of step s+DEPTH are issued at the top of step s into one of DEPTH
+// register stages (the loop is unrolled DEPTH times to keep stage indices static) and reach
+// LDS at the end of step s+DEPTH-1; fragments of substep kk+1 are read from LDS while the
+// MFMAs of substep kk run.  LDS rows are padded by 8 halves (the 128-bit fragment reads of
+// 16 lanes hit distinct banks).
 constexpr int kGemmBigBM = 256, kGemmBigBN = 256;
-template <int BK>
+template <int BK, int DEPTH>
 __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
                                                           float beta) {
   constexpr int STRIDE = BK + 8;            // halves per LDS row
@@ -145,6 +148,7 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
   const half8_t *ga = A + (tile_m * kGemmBigBM + crow) * k_chunks + cchunk;
   const half8_t *gb = B + (tile_n * kGemmBigBN + crow) * k_chunks + cchunk;
   const int so = crow * STRIDE + cchunk * 8;
+  const size_t steps = K / BK;
 
   float16_t acc[4][4];
 #pragma unroll
@@ -154,52 +158,72 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-  half8_t ra[PASSES], rb[PASSES];
+  // stage d holds the data of the steps s with s % DEPTH == d.  The loop body is free of
+  // branches (steps % DEPTH == 0 is the caller's duty; loads past the last step re-read the
+  // last step and are never used), which keeps every stage in registers.
+  half8_t ra[DEPTH][PASSES], rb[DEPTH][PASSES];
 #pragma unroll
-  for (int i = 0; i < PASSES; i++) {
-    ra[i] = ga[(size_t)i * RPP * k_chunks];
-    rb[i] = gb[(size_t)i * RPP * k_chunks];
+  for (int d = 0; d < DEPTH; d++) {
+#pragma unroll
+    for (int i = 0; i < PASSES; i++) {
+      ra[d][i] = ga[(size_t)i * RPP * k_chunks + (size_t)d * CPR];
+      rb[d][i] = gb[(size_t)i * RPP * k_chunks + (size_t)d * CPR];
+    }
   }
 #pragma unroll
   for (int i = 0; i < PASSES; i++) {
-    *reinterpret_cast<half8_t *>(&lds_a[0][so + i * RPP * STRIDE]) = ra[i];
-    *reinterpret_cast<half8_t *>(&lds_b[0][so + i * RPP * STRIDE]) = rb[i];
+    *reinterpret_cast<half8_t *>(&lds_a[0][so + i * RPP * STRIDE]) = ra[0][i];
+    *reinterpret_cast<half8_t *>(&lds_b[0][so + i * RPP * STRIDE]) = rb[0][i];
   }
   __syncthreads();
 
-  const size_t steps = K / BK;
   const int frow = lane & 31, fk = (lane >> 5) * 8;
-  for (size_t s = 0; s < steps; s++) {
-    const int cur = (int)(s & 1);
-    if (s + 1 < steps) {
-      const size_t o = (s + 1) * CPR;
+  for (size_t s0 = 0; s0 < steps; s0 += DEPTH) {
 #pragma unroll
-      for (int i = 0; i < PASSES; i++) {
-        ra[i] = ga[(size_t)i * RPP * k_chunks + o];
-        rb[i] = gb[(size_t)i * RPP * k_chunks + o];
+    for (int d = 0; d < DEPTH; d++) {
+      const size_t s = s0 + d;
+      const int cur = (DEPTH & 1) ? (int)(s & 1) : (d & 1);
+      // stage d went to LDS at the end of the previous step (or in the prologue): refill it
+      {
+        const size_t sn = s + DEPTH < steps ? s + DEPTH : steps - 1;
+        const size_t o = sn * CPR;
+#pragma unroll
+        for (int i = 0; i < PASSES; i++) {
+          ra[d][i] = ga[(size_t)i * RPP * k_chunks + o];
+          rb[d][i] = gb[(size_t)i * RPP * k_chunks + o];
+        }
       }
-    }
+      half8_t fa[2][4], fb[2][4];
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; kk++) {
-      half8_t fa[4], fb[4];
+      for (int i = 0; i < 4; i++) fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][(wm * 128 + i * 32 + frow) * STRIDE + fk]);
 #pragma unroll
-      for (int i = 0; i < 4; i++) fa[i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][(wm * 128 + i * 32 + frow) * STRIDE + kk * 16 + fk]);
+      for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t *>(&lds_b[cur][(wn * 128 + j * 32 + frow) * STRIDE + fk]);
 #pragma unroll
-      for (int j = 0; j < 4; j++) fb[j] = *reinterpret_cast<const half8_t *>(&lds_b[cur][(wn * 128 + j * 32 + frow) * STRIDE + kk * 16 + fk]);
+      for (int kk = 0; kk < BK / 16; kk++) {
+        const int p = kk & 1, q = p ^ 1;
+        if (kk + 1 < BK / 16) {
 #pragma unroll
-      for (int i = 0; i < 4; i++)
+          for (int i = 0; i < 4; i++) fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][(wm * 128 + i * 32 + frow) * STRIDE + (kk + 1) * 16 + fk]);
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[i], fb[j], acc[i][j]);
-    }
-    if (s + 1 < steps) {
-      const int nxt = cur ^ 1;
+          for (int j = 0; j < 4; j++) fb[q][j] = *reinterpret_cast<const half8_t *>(&lds_b[cur][(wn * 128 + j * 32 + frow) * STRIDE + (kk + 1) * 16 + fk]);
+        }
+        sched_fence();  // keep the reads above the MFMAs: the scheduler otherwise sinks each read to its first use
 #pragma unroll
-      for (int i = 0; i < PASSES; i++) {
-        *reinterpret_cast<half8_t *>(&lds_a[nxt][so + i * RPP * STRIDE]) = ra[i];
-        *reinterpret_cast<half8_t *>(&lds_b[nxt][so + i * RPP * STRIDE]) = rb[i];
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
       }
+      {  // the next step's data sits in stage (d + 1) % DEPTH (after the last step: unused)
+        const int nxt = cur ^ 1;
+        const int dn = (d + 1) % DEPTH;
+#pragma unroll
+        for (int i = 0; i < PASSES; i++) {
+          *reinterpret_cast<half8_t *>(&lds_a[nxt][so + i * RPP * STRIDE]) = ra[dn][i];
+          *reinterpret_cast<half8_t *>(&lds_b[nxt][so + i * RPP * STRIDE]) = rb[dn][i];
+        }
+      }
+      __syncthreads();
     }
-    __syncthreads();
   }
 #pragma unroll
   for (int i = 0; i < 4; i++)

@@ -138,6 +138,9 @@ TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
     *p = v;
 }
 
+// stops the instruction scheduler from moving anything across this point
+TCU_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+
 // orders LDS traffic between the lanes of one wave (no s_barrier: a wave runs in lockstep)
 TCU_DEVICE void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -365,6 +365,7 @@ template <bool NT>
 inline void store_chunk(uint4_t *p, uint4_t v) {
   *p = v;
 }
+inline void sched_fence() {}
 inline void wave_lds_fence() {
   emu::wave_sync();
 }
