@@ -122,13 +122,17 @@ TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_
 
 // M % 256 == 0, N % 256 == 0, K % (BK * DEPTH) == 0; 256 threads.  256 x 256 x BK block tile, 2 x 2
 // waves of 128 x 128 (4 x 4 MFMA 32x32x16 accumulators = 256 registers, one wave per SIMD):
-// per 16-wide k substep a wave reads 8 fragments from LDS for 16 MFMAs, which leaves LDS
-// at half of its bandwidth.  With one wave per SIMD nothing else hides memory latency, so
-// the global loads of step s+DEPTH are issued at the top of step s into one of DEPTH
-// register stages (the loop is unrolled DEPTH times to keep stage indices static) and reach
-// LDS at the end of step s+DEPTH-1; fragments of substep kk+1 are read from LDS while the
-// MFMAs of substep kk run.  LDS rows are padded by 8 halves (the 128-bit fragment reads of
-// 16 lanes hit distinct banks).
+// per 16-wide k substep a wave reads 8 fragments from LDS for 16 MFMAs.  With one wave per
+// SIMD nothing else hides latency, so the kernel is software-pipelined by hand:
+//   - global loads run DEPTH steps ahead in DEPTH register stages (the loop is unrolled
+//     DEPTH times to keep stage indices static);
+//   - the stage of step s+1 is written to the other LDS buffer during the second-last
+//     substep of step s, the one barrier of the step sits before the last substep, and the
+//     fragments of step s+1's first substep are read behind that barrier while the last 16
+//     MFMAs of step s run; inside a step the fragments of substep kk+1 are read while the
+//     MFMAs of substep kk run.
+// LDS rows are padded by 8 halves (the 128-bit fragment reads of 16 lanes hit distinct
+// banks).
 constexpr int kGemmBigBM = 256, kGemmBigBN = 256;
 template <int BK, int DEPTH>
 __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
@@ -158,71 +162,115 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-  // stage d holds the data of the steps s with s % DEPTH == d.  The loop body is free of
-  // branches (steps % DEPTH == 0 is the caller's duty; loads past the last step re-read the
-  // last step and are never used), which keeps every stage in registers.
+  // Step 0 goes straight to LDS; register stage d then holds the steps t with (t - 1) % DEPTH
+  // == d, i.e. during step s the stages hold the steps s+1 .. s+DEPTH.  The loop body is free
+  // of branches (steps % DEPTH == 0 is the caller's duty; loads past the last step re-read
+  // the last step and are never used), which keeps every stage in registers.
   half8_t ra[DEPTH][PASSES], rb[DEPTH][PASSES];
-#pragma unroll
-  for (int d = 0; d < DEPTH; d++) {
+  {
+    half8_t ta[PASSES], tb[PASSES];
 #pragma unroll
     for (int i = 0; i < PASSES; i++) {
-      ra[d][i] = ga[(size_t)i * RPP * k_chunks + (size_t)d * CPR];
-      rb[d][i] = gb[(size_t)i * RPP * k_chunks + (size_t)d * CPR];
+      ta[i] = ga[(size_t)i * RPP * k_chunks];
+      tb[i] = gb[(size_t)i * RPP * k_chunks];
     }
-  }
 #pragma unroll
-  for (int i = 0; i < PASSES; i++) {
-    *reinterpret_cast<half8_t *>(&lds_a[0][so + i * RPP * STRIDE]) = ra[0][i];
-    *reinterpret_cast<half8_t *>(&lds_b[0][so + i * RPP * STRIDE]) = rb[0][i];
+    for (int d = 0; d < DEPTH; d++) {
+      const size_t t = (size_t)d + 1 < steps ? (size_t)d + 1 : steps - 1;
+#pragma unroll
+      for (int i = 0; i < PASSES; i++) {
+        ra[d][i] = ga[(size_t)i * RPP * k_chunks + t * CPR];
+        rb[d][i] = gb[(size_t)i * RPP * k_chunks + t * CPR];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PASSES; i++) {
+      *reinterpret_cast<half8_t *>(&lds_a[0][so + i * RPP * STRIDE]) = ta[i];
+      *reinterpret_cast<half8_t *>(&lds_b[0][so + i * RPP * STRIDE]) = tb[i];
+    }
   }
   __syncthreads();
 
   const int frow = lane & 31, fk = (lane >> 5) * 8;
+  constexpr int SUB = BK / 16;  // 16-wide k substeps per step (even: fragment parity carries over steps)
+  const int fao = (wm * 128 + frow) * STRIDE + fk, fbo = (wn * 128 + frow) * STRIDE + fk;
+  half8_t fa[2][4], fb[2][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[0][fao + i * 32 * STRIDE]);
+    fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[0][fbo + i * 32 * STRIDE]);
+  }
   for (size_t s0 = 0; s0 < steps; s0 += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) {
       const size_t s = s0 + d;
       const int cur = (DEPTH & 1) ? (int)(s & 1) : (d & 1);
-      // stage d went to LDS at the end of the previous step (or in the prologue): refill it
-      {
-        const size_t sn = s + DEPTH < steps ? s + DEPTH : steps - 1;
-        const size_t o = sn * CPR;
+      const int nxt = cur ^ 1;
+      const size_t sn = s + 1 + DEPTH < steps ? s + 1 + DEPTH : steps - 1;
+      const size_t o = sn * CPR;
 #pragma unroll
-        for (int i = 0; i < PASSES; i++) {
-          ra[d][i] = ga[(size_t)i * RPP * k_chunks + o];
-          rb[d][i] = gb[(size_t)i * RPP * k_chunks + o];
-        }
-      }
-      half8_t fa[2][4], fb[2][4];
-#pragma unroll
-      for (int i = 0; i < 4; i++) fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][(wm * 128 + i * 32 + frow) * STRIDE + fk]);
-#pragma unroll
-      for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t *>(&lds_b[cur][(wn * 128 + j * 32 + frow) * STRIDE + fk]);
-#pragma unroll
-      for (int kk = 0; kk < BK / 16; kk++) {
+      for (int kk = 0; kk < SUB; kk++) {
         const int p = kk & 1, q = p ^ 1;
-        if (kk + 1 < BK / 16) {
+        if (kk == SUB - 1) {
+          // the LDS writes of this step are visible behind the barrier; the fragments of the
+          // next step's first substep are read while the MFMAs of this step's last one run
+          __syncthreads();
+          sched_fence();
 #pragma unroll
-          for (int i = 0; i < 4; i++) fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][(wm * 128 + i * 32 + frow) * STRIDE + (kk + 1) * 16 + fk]);
+          for (int i = 0; i < 4; i++) {
+            fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[nxt][fao + i * 32 * STRIDE]);
+            fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[nxt][fbo + i * 32 * STRIDE]);
+          }
+          // stage d went to LDS before the barrier: refill it with step s + 1 + DEPTH
 #pragma unroll
-          for (int j = 0; j < 4; j++) fb[q][j] = *reinterpret_cast<const half8_t *>(&lds_b[cur][(wn * 128 + j * 32 + frow) * STRIDE + (kk + 1) * 16 + fk]);
+          for (int i = 0; i < PASSES; i++) {
+            ra[d][i] = ga[(size_t)i * RPP * k_chunks + o];
+            rb[d][i] = gb[(size_t)i * RPP * k_chunks + o];
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][fao + i * 32 * STRIDE + (kk + 1) * 16]);
+            fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[cur][fbo + i * 32 * STRIDE + (kk + 1) * 16]);
+          }
         }
-        sched_fence();  // keep the reads above the MFMAs: the scheduler otherwise sinks each read to its first use
+        if (kk == SUB - 2) {
+          // the next step's data (stage d) goes to the other LDS buffer, whose readers all
+          // passed the barrier of the previous step
+#pragma unroll
+          for (int i = 0; i < PASSES; i++) {
+            *reinterpret_cast<half8_t *>(&lds_a[nxt][so + i * RPP * STRIDE]) = ra[d][i];
+            *reinterpret_cast<half8_t *>(&lds_b[nxt][so + i * RPP * STRIDE]) = rb[d][i];
+          }
+        }
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
           for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
-      }
-      {  // the next step's data sits in stage (d + 1) % DEPTH (after the last step: unused)
-        const int nxt = cur ^ 1;
-        const int dn = (d + 1) % DEPTH;
+        // issue order of the substep: the 8 fragment reads lead, one per MFMA, then the
+        // LDS writes or global loads of the substep spread over the remaining MFMAs
 #pragma unroll
-        for (int i = 0; i < PASSES; i++) {
-          *reinterpret_cast<half8_t *>(&lds_a[nxt][so + i * RPP * STRIDE]) = ra[dn][i];
-          *reinterpret_cast<half8_t *>(&lds_b[nxt][so + i * RPP * STRIDE]) = rb[dn][i];
+        for (int t = 0; t < 8; t++) {
+          sched_group<kSchedDsRead, 1>();
+          sched_group<kSchedMfma, 1>();
         }
+        if (kk == SUB - 2) {
+#pragma unroll
+          for (int t = 0; t < 8; t++) {
+            sched_group<kSchedDsWrite, PASSES / 4>();
+            sched_group<kSchedMfma, 1>();
+          }
+        } else if (kk == SUB - 1) {
+#pragma unroll
+          for (int t = 0; t < 8; t++) {
+            sched_group<kSchedVmemRead, PASSES / 4>();
+            sched_group<kSchedMfma, 1>();
+          }
+        } else {
+          sched_group<kSchedMfma, 8>();
+        }
+        sched_fence();
       }
-      __syncthreads();
     }
   }
 #pragma unroll

@@ -140,6 +140,12 @@ TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
 
 // stops the instruction scheduler from moving anything across this point
 TCU_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+// Instruction-mix hints for the scheduler inside one region: "next, COUNT instructions of KIND".
+enum : int { kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200 };
+template <int KIND, int COUNT>
+TCU_DEVICE void sched_group() {
+  __builtin_amdgcn_sched_group_barrier(KIND, COUNT, 0);
+}
 
 // orders LDS traffic between the lanes of one wave (no s_barrier: a wave runs in lockstep)
 TCU_DEVICE void wave_lds_fence() {

@@ -366,6 +366,9 @@ inline void store_chunk(uint4_t *p, uint4_t v) {
   *p = v;
 }
 inline void sched_fence() {}
+enum : int { kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200 };
+template <int KIND, int COUNT>
+inline void sched_group() {}
 inline void wave_lds_fence() {
   emu::wave_sync();
 }
