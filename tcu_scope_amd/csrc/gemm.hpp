@@ -234,14 +234,17 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
             fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[cur][fbo + i * 32 * STRIDE + (kk + 1) * 16]);
           }
         }
-        if (kk == SUB - 2) {
-          // the next step's data (stage d) goes to the other LDS buffer, whose readers all
-          // passed the barrier of the previous step
+        // the next step's data (stage d) goes to the other LDS buffer, whose readers all
+        // passed the barrier of the previous step: A and B in different substeps where the
+        // step has enough of them, so that LDS is not flooded just before the barrier
+        constexpr int WA = SUB >= 4 ? SUB - 3 : SUB - 2, WB = SUB - 2;
+        if (kk == WA) {
 #pragma unroll
-          for (int i = 0; i < PASSES; i++) {
-            *reinterpret_cast<half8_t *>(&lds_a[nxt][so + i * RPP * STRIDE]) = ra[d][i];
-            *reinterpret_cast<half8_t *>(&lds_b[nxt][so + i * RPP * STRIDE]) = rb[d][i];
-          }
+          for (int i = 0; i < PASSES; i++) *reinterpret_cast<half8_t *>(&lds_a[nxt][so + i * RPP * STRIDE]) = ra[d][i];
+        }
+        if (kk == WB) {
+#pragma unroll
+          for (int i = 0; i < PASSES; i++) *reinterpret_cast<half8_t *>(&lds_b[nxt][so + i * RPP * STRIDE]) = rb[d][i];
         }
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -254,10 +257,11 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
           sched_group<kSchedDsRead, 1>();
           sched_group<kSchedMfma, 1>();
         }
-        if (kk == SUB - 2) {
+        if (kk == WA || kk == WB) {
+          constexpr int W = (WA == WB ? 2 : 1) * PASSES;  // 8 writes in every case
 #pragma unroll
           for (int t = 0; t < 8; t++) {
-            sched_group<kSchedDsWrite, PASSES / 4>();
+            sched_group<kSchedDsWrite, W / 8>();
             sched_group<kSchedMfma, 1>();
           }
         } else if (kk == SUB - 1) {
