@@ -24,13 +24,20 @@ constexpr int kGemmLdsStride = 40;  // halves per LDS row (32 + 8 pad)
 
 TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_m, size_t *tile_n);
 
+// D and C are streamed once: non-temporal accesses keep them from displacing the A and B
+// panels that other tiles reuse from L2.  All of a tile's C values are read before its first
+// store, so the loads overlap and C may be the same buffer as D.
 TCU_DEVICE void gemm_store_tile(float *D, const float *C, size_t ldc, size_t row0, size_t col0, const float16_t &acc, int lane, float alpha, float beta) {
-  const size_t col = col0 + (lane & 31);
+  const size_t base = (row0 + 4 * (lane >> 5)) * ldc + col0 + (lane & 31);
+  if (beta == 0.0f) {
 #pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const size_t row = row0 + 8 * (i / 4) + 4 * (lane >> 5) + (i % 4);
-    const size_t idx = row * ldc + col;
-    D[idx] = beta == 0.0f ? alpha * acc[i] : alpha * acc[i] + beta * C[idx];
+    for (int i = 0; i < 16; i++) __builtin_nontemporal_store(alpha * acc[i], D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+  } else {
+    float c[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) c[i] = __builtin_nontemporal_load(C + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+#pragma unroll
+    for (int i = 0; i < 16; i++) __builtin_nontemporal_store(alpha * acc[i] + beta * c[i], D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
   }
 }
 

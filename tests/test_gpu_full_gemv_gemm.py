@@ -143,6 +143,37 @@ def test_gemm_small_exact_and_normal(tcu, oracle, M, N, K):
                     assert bad == 0, (v.name, alpha, beta, bad, worst, first)
 
 
+def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
+    """The 256 x 256 tile kernel in every (K step, prefetch depth) instantiation, including the
+    depths the dispatcher falls back to when the step count is not a multiple of the requested
+    one, and with C aliasing D.  Integer-valued inputs: results must be exact."""
+    import torch
+
+    M, N = 512, 256
+    try:
+        for K in (64, 96, 160, 384, 768):
+            A = oracle.generate_f16(M * K, 11, oracle.DIST_SMALLINT)
+            B = oracle.generate_f16(N * K, 12, oracle.DIST_SMALLINT)
+            C0 = (np.arange(M * N) % 5).astype(np.float32)
+            Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
+            ref0 = oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0)
+            ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
+            for bk64 in (0, 1):
+                for depth in (1, 2, 3, 4):
+                    tcu.set_option("gemm_bk64", bk64)
+                    tcu.set_option("gemm_depth", depth)
+                    D = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS)
+                    torch.cuda.synchronize()
+                    assert np.array_equal(D.cpu().numpy().astype(np.float64), ref0), (K, bk64, depth)
+                    Cd = torch.from_numpy(C0.copy()).cuda().view(M, N)
+                    D = tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd, variant=tcu.Variant.BLOCK_LDS)  # in place
+                    torch.cuda.synchronize()
+                    assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("in place", K, bk64, depth)
+    finally:
+        tcu.set_option("gemm_bk64", 1)
+        tcu.set_option("gemm_depth", 4)
+
+
 def test_gemm_8192(tcu, oracle):
     """M = N = K = 8192, N(0,1) inputs, 1e-2 relative: 64 sampled rows against the fp64 oracle."""
     import torch
