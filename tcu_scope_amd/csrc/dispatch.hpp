@@ -35,7 +35,7 @@ struct Options {
   bool nontemporal = true;
   bool static_order = false;
   bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
-  bool gemm_bk64 = true;       // K step 64 (prefetch depth <= 2) where K allows
+  bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
 };
 inline Options &options() {

@@ -155,10 +155,18 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
   size_t tile_m, tile_n;
   gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
+  // Copy assignment: CPR consecutive lanes take one row's BK halves (one or two full cache
+  // lines of global memory), 16 consecutive lanes 16 / CPR consecutive rows.  Inside LDS the
+  // rows of every aligned group of 16 are permuted (lds_row): the 16 / CPR rows that 16
+  // lanes store in one go land CPR positions apart, which puts their 128-bit stores into 16
+  // different groups of four banks (row stride = 2 * CPR + 1 such groups, odd), and 16
+  // consecutive rows read by 16 lanes still occupy 16 different positions.
   const int crow = tid / CPR, cchunk = tid % CPR;  // rows crow + RPP*i
+  constexpr int ROT = CPR == 8 ? 1 : 2;  // rotate the low 4 bits of the row index right by ROT
+  auto lds_row = [](int r) { return (r & ~15) | ((r & 15) >> ROT) | ((r << (4 - ROT)) & 15); };
   const half8_t *ga = A + (tile_m * kGemmBigBM + crow) * k_chunks + cchunk;
   const half8_t *gb = B + (tile_n * kGemmBigBN + crow) * k_chunks + cchunk;
-  const int so = crow * STRIDE + cchunk * 8;
+  const int so = lds_row(crow) * STRIDE + cchunk * 8;
   const size_t steps = K / BK;
 
   float16_t acc[4][4];
@@ -200,7 +208,7 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
 
   const int frow = lane & 31, fk = (lane >> 5) * 8;
   constexpr int SUB = BK / 16;  // 16-wide k substeps per step (even: fragment parity carries over steps)
-  const int fao = (wm * 128 + frow) * STRIDE + fk, fbo = (wn * 128 + frow) * STRIDE + fk;
+  const int fao = (wm * 128 + lds_row(frow)) * STRIDE + fk, fbo = (wn * 128 + lds_row(frow)) * STRIDE + fk;
   half8_t fa[2][4], fb[2][4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
