@@ -83,7 +83,15 @@ const char *tcu_last_error(void);
 int tcu_abi_version(void);
 /* Compute units, wavefront size, LDS bytes per CU, 1 if the device is gfx950. */
 int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int *is_gfx950);
-/* Tuning switches used by the benchmarks: "nontemporal" (0/1, default 1). */
+/* Tuning switches used by the benchmarks and tests (process-wide, not thread-safe against
+ * concurrent launches):
+ *   "nontemporal"     0/1, default 1: non-temporal loads and stores in the streaming kernels
+ *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
+ *   "gemm_big_tiles"  0/1, default 1: 256 x 256 block tiles where M and N allow
+ *   "gemm_direct_lds" 0/3/4, default 4: global -> LDS transfers with that many LDS buffers; 0 = register-staged kernel
+ *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
+ *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
+ * Unknown names return TCU_ERR_INVALID_ARG. */
 int tcu_set_option(const char *name, int value);
 
 /* ---- segmented reduction -------------------------------------------------------------- */

@@ -75,30 +75,7 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
   return TCU_OK;
 }
 
-int tcu_set_option(const char *name, int value) {
-  if (!name) return tcu::fail(TCU_ERR_INVALID_ARG, "tcu_set_option: null name");
-  if (std::strcmp(name, "nontemporal") == 0) {
-    tcu::options().nontemporal = value != 0;
-    return TCU_OK;
-  }
-  if (std::strcmp(name, "gemm_big_tiles") == 0) {
-    tcu::options().gemm_big_tiles = value != 0;
-    return TCU_OK;
-  }
-  if (std::strcmp(name, "gemm_depth") == 0) {
-    tcu::options().gemm_depth = value;
-    return TCU_OK;
-  }
-  if (std::strcmp(name, "gemm_bk64") == 0) {
-    tcu::options().gemm_bk64 = value != 0;
-    return TCU_OK;
-  }
-  if (std::strcmp(name, "static_order") == 0) {
-    tcu::options().static_order = value != 0;
-    return TCU_OK;
-  }
-  return tcu::fail(TCU_ERR_INVALID_ARG, std::string("tcu_set_option: unknown option ") + name);
-}
+int tcu_set_option(const char *name, int value) { return tcu::set_option(name, value); }
 
 int tcu_seg_reduce_f16(const void *d_in, void *d_out, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
   const unsigned long before = tcu::launch_count();

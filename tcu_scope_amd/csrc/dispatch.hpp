@@ -36,11 +36,25 @@ struct Options {
   bool static_order = false;
   bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
+  int gemm_direct_lds = 4;     // > 0: global -> LDS transfers without staging registers, that many LDS buffers (3 or 4); 0: register-staged kernel
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
 };
 inline Options &options() {
   static Options o;
   return o;
+}
+inline int set_option(const char *name, int value) {
+  if (!name) return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: null name");
+  const std::string n(name);
+  Options &o = options();
+  if (n == "nontemporal") o.nontemporal = value != 0;
+  else if (n == "static_order") o.static_order = value != 0;
+  else if (n == "gemm_big_tiles") o.gemm_big_tiles = value != 0;
+  else if (n == "gemm_direct_lds") o.gemm_direct_lds = value;
+  else if (n == "gemm_depth") o.gemm_depth = value;
+  else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
+  else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
+  return TCU_OK;
 }
 
 inline bool is_pow2(size_t x) { return x && !(x & (x - 1)); }
@@ -551,6 +565,13 @@ inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, s
   if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && options().gemm_big_tiles) {
     const size_t grid = (M / kGemmBigBM) * (N / kGemmBigBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    if (options().gemm_direct_lds > 0 && K <= ((size_t)1 << 22)) {
+      if (options().gemm_direct_lds == 3)
+        launch(gemm_dlds_kernel<3>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      else
+        launch(gemm_dlds_kernel<4>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      return TCU_OK;
+    }
     const bool bk64 = K % 64 == 0 && options().gemm_bk64;
     const size_t steps = K / (bk64 ? 64 : 32);
     int depth = options().gemm_depth < 1 ? 1 : (options().gemm_depth > 4 ? 4 : options().gemm_depth);

@@ -138,10 +138,54 @@ TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
     *p = v;
 }
 
+// Global -> LDS without a register round trip: lane l of the wave moves the 16 bytes at its
+// own global address `src` to lds_base + 16 * l (lds_base is the same for the whole wave).
+// Written as inline assembly on purpose: for the compiler's own form of this instruction the
+// wait-count pass drains every transfer in flight before the next LDS read it cannot prove
+// disjoint, which would undo a multi-stage prefetch.  The price: the compiler knows nothing
+// of these transfers, so the reader orders them by hand: wait_vector_loads<N>() for the
+// wave's own, then a barrier for everybody's.
+// An LDS location is named by its byte offset inside the block's LDS (lds_addr_t), which
+// keeps the address arithmetic of a transfer in scalar integer registers.
+using lds_addr_t = uint32_t;
+// tells the compiler that a value is the same in every lane (it then lives in a scalar register)
+TCU_DEVICE uint32_t wave_uniform(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane(x); }
+TCU_DEVICE lds_addr_t lds_address_of(const half_t *lds_pointer) {
+  using lds_ptr_t = const __attribute__((address_space(3))) half_t *;
+  return (lds_addr_t)(uintptr_t)(lds_ptr_t)lds_pointer;
+}
+// The global address is wave_base (the same for the whole wave, kept in scalar registers)
+// plus the lane's own byte offset.
+TCU_DEVICE void load_chunk_to_lds(const void *wave_base, uint32_t lane_byte_offset, lds_addr_t lds_base) {
+  const uint32_t base = wave_uniform(lds_base);
+  const uint64_t g = (uint64_t)wave_base;
+  // (the builtin returns a signed int: widen through uint32_t, or bit 31 of the low word smears over the high one)
+  const uint32_t g_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)g), g_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
+  const uint64_t gs = ((uint64_t)g_hi << 32) | (uint64_t)g_lo;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(base), "v"(lane_byte_offset), "s"(gs) : "memory", "m0");
+}
+// blocks until at most N of this wave's vector memory loads are still in flight (they
+// complete in issue order); N <= 63
+template <int N>
+TCU_DEVICE void wait_vector_loads() {
+  static_assert(N >= 0 && N <= 63, "vmcnt has 6 bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Block barrier for code that orders its own memory traffic: waits for this wave's LDS
+// operations only (not for vector memory loads in flight, which __syncthreads() would drain)
+// and keeps the compiler from moving memory accesses across it.
+TCU_DEVICE void block_barrier_lds_only() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // stops the instruction scheduler from moving anything across this point
 TCU_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 // Instruction-mix hints for the scheduler inside one region: "next, COUNT instructions of KIND".
-enum : int { kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200 };
+enum : int { kSchedMfma = 0x008, kSchedVmem = 0x010, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200 };
 template <int KIND, int COUNT>
 TCU_DEVICE void sched_group() {
   __builtin_amdgcn_sched_group_barrier(KIND, COUNT, 0);

@@ -11,6 +11,7 @@ int emu_seg_scan_f16(const void *in, void *out, void *totals, size_t nseg, size_
 }
 int emu_add_partial_sums_f16(void *out, const void *ps, size_t nseg, size_t seg) { return tcu::add_partial_sums_dispatch(out, ps, nseg, seg, nullptr); }
 const char *emu_last_error() { return tcu::last_error_string().c_str(); }
+int emu_set_option(const char *name, int value) { return tcu::set_option(name, value); }
 }
 extern "C" {
 int emu_full_reduce_f16(const void *in, void *out, size_t n, void *ws, size_t *ws_bytes, int strategy, size_t seg, int wpb) {

@@ -366,7 +366,17 @@ inline void store_chunk(uint4_t *p, uint4_t v) {
   *p = v;
 }
 inline void sched_fence() {}
-enum : int { kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200 };
+// lanes run one after another here, so the transfer is a plain copy and nothing is in flight
+using lds_addr_t = uintptr_t;
+inline uintptr_t wave_uniform(uintptr_t x) { return x; }
+inline lds_addr_t lds_address_of(const half_t *lds_pointer) { return reinterpret_cast<uintptr_t>(lds_pointer); }
+inline void load_chunk_to_lds(const void *wave_base, uint32_t lane_byte_offset, lds_addr_t lds_base) {
+  *reinterpret_cast<half8_t *>(lds_base + 16 * (uintptr_t)lane_id()) = *reinterpret_cast<const half8_t *>(static_cast<const char *>(wave_base) + lane_byte_offset);
+}
+template <int N>
+inline void wait_vector_loads() {}
+inline void block_barrier_lds_only() { emu::block_sync(); }
+enum : int { kSchedMfma = 0x008, kSchedVmem = 0x010, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200 };
 template <int KIND, int COUNT>
 inline void sched_group() {}
 inline void wave_lds_fence() {

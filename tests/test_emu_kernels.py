@@ -36,6 +36,7 @@ def emu():
     L.emu_full_scan_f16.argtypes = [vp, vp, sz, vp, ctypes.POINTER(sz), ci, sz, ci]
     L.emu_gemv_f16_f32.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci]
     L.emu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
+    L.emu_set_option.argtypes = [ctypes.c_char_p, ci]
     L.emu_generate_f16.argtypes = [vp, sz, ctypes.c_uint64, ci, sz]
     L.emu_last_error.restype = ctypes.c_char_p
     return L
@@ -152,3 +153,20 @@ def test_gemv_gemm_and_generator(emu, oracle):
             if rc == 2:
                 continue
             assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A, B, M, N, K, 2.0, 3.0, C0)), (M, N, K, v)
+    # the 256 x 256 tile kernels: register-staged (K step 32 / 64, every prefetch depth that
+    # divides the step count) and direct-to-LDS (3 and 4 buffers)
+    M, N, K = 256, 256, 192
+    A, B = oracle.generate_f16(M * K, 7, oracle.DIST_SMALLINT), oracle.generate_f16(N * K, 8, oracle.DIST_SMALLINT)
+    C0 = (np.arange(M * N) % 5).astype(np.float32)
+    Ai, Bi, Ci = copy_in(A), copy_in(B), copy_in(C0, np.float32)
+    ref = oracle.gemm_f64(A, B, M, N, K, 1.5, 2.0, C0)
+    try:
+        for direct_lds, bk64, depth in ((3, 0, 4), (4, 0, 4), (0, 0, 1), (0, 0, 2), (0, 0, 3), (0, 0, 4), (0, 1, 1), (0, 1, 2)):
+            for name, val in ((b"gemm_direct_lds", direct_lds), (b"gemm_bk64", bk64), (b"gemm_depth", depth)):
+                assert emu.emu_set_option(name, val) == 0
+            D = aligned(M * N, np.float32, -777)
+            rc = emu.emu_gemm_f16_f32(Ai.ctypes.data, Bi.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
+            assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), ref), (direct_lds, bk64, depth)
+    finally:
+        for name, val in ((b"gemm_direct_lds", 4), (b"gemm_bk64", 0), (b"gemm_depth", 4)):
+            emu.emu_set_option(name, val)

@@ -144,7 +144,7 @@ def test_gemm_small_exact_and_normal(tcu, oracle, M, N, K):
 
 
 def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
-    """The 256 x 256 tile kernel in every (K step, prefetch depth) instantiation, including the
+    """The 256 x 256 tile kernels (register-staged and direct-to-LDS) in every (K step, prefetch depth / buffer count) instantiation, including the
     depths the dispatcher falls back to when the step count is not a multiple of the requested
     one, and with C aliasing D.  Integer-valued inputs: results must be exact."""
     import torch
@@ -158,19 +158,21 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
             ref0 = oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0)
             ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
-            for bk64 in (0, 1):
-                for depth in (1, 2, 3, 4):
-                    tcu.set_option("gemm_bk64", bk64)
-                    tcu.set_option("gemm_depth", depth)
-                    D = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS)
-                    torch.cuda.synchronize()
-                    assert np.array_equal(D.cpu().numpy().astype(np.float64), ref0), (K, bk64, depth)
-                    Cd = torch.from_numpy(C0.copy()).cuda().view(M, N)
-                    D = tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd, variant=tcu.Variant.BLOCK_LDS)  # in place
-                    torch.cuda.synchronize()
-                    assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("in place", K, bk64, depth)
+            shapes = [(0, bk64, depth) for bk64 in (0, 1) for depth in (1, 2, 3, 4)] + [(3, 0, 4), (4, 0, 4)]
+            for direct_lds, bk64, depth in shapes:
+                tcu.set_option("gemm_direct_lds", direct_lds)
+                tcu.set_option("gemm_bk64", bk64)
+                tcu.set_option("gemm_depth", depth)
+                D = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS)
+                torch.cuda.synchronize()
+                assert np.array_equal(D.cpu().numpy().astype(np.float64), ref0), (K, direct_lds, bk64, depth)
+                Cd = torch.from_numpy(C0.copy()).cuda().view(M, N)
+                D = tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd, variant=tcu.Variant.BLOCK_LDS)  # in place
+                torch.cuda.synchronize()
+                assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("in place", K, direct_lds, bk64, depth)
     finally:
-        tcu.set_option("gemm_bk64", 1)
+        tcu.set_option("gemm_direct_lds", 4)
+        tcu.set_option("gemm_bk64", 0)
         tcu.set_option("gemm_depth", 4)
 
 
