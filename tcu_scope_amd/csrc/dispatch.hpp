@@ -36,7 +36,7 @@ struct Options {
   bool static_order = false;
   bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
-  int gemm_direct_lds = 4;     // > 0: global -> LDS transfers without staging registers, that many LDS buffers (3 or 4); 0: register-staged kernel
+  int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers without staging registers, that many LDS buffers; 0: register-staged kernel; -1: by K
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
 };
 inline Options &options() {
@@ -565,8 +565,11 @@ inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, s
   if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && options().gemm_big_tiles) {
     const size_t grid = (M / kGemmBigBM) * (N / kGemmBigBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    if (options().gemm_direct_lds > 0 && K <= ((size_t)1 << 22)) {
-      if (options().gemm_direct_lds == 3)
+    // measured: the transfer kernel is the faster one (1.15-1.22 vs 1.0-1.1 PFLOP/s at 8192^3)
+    // except when rows are a multiple of 32 KiB apart (K % 16384 == 0: 0.85 vs 0.98 PFLOP/s)
+    const int direct_lds = options().gemm_direct_lds >= 0 ? options().gemm_direct_lds : (K % 16384 == 0 ? 0 : 4);
+    if (direct_lds > 0 && K <= ((size_t)1 << 22)) {
+      if (direct_lds == 3)
         launch(gemm_dlds_kernel<3>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       else
         launch(gemm_dlds_kernel<4>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);

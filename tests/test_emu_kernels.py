@@ -168,5 +168,5 @@ def test_gemv_gemm_and_generator(emu, oracle):
             rc = emu.emu_gemm_f16_f32(Ai.ctypes.data, Bi.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), ref), (direct_lds, bk64, depth)
     finally:
-        for name, val in ((b"gemm_direct_lds", 4), (b"gemm_bk64", 0), (b"gemm_depth", 4)):
+        for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4)):
             emu.emu_set_option(name, val)

@@ -171,7 +171,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
                 torch.cuda.synchronize()
                 assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("in place", K, direct_lds, bk64, depth)
     finally:
-        tcu.set_option("gemm_direct_lds", 4)
+        tcu.set_option("gemm_direct_lds", -1)
         tcu.set_option("gemm_bk64", 0)
         tcu.set_option("gemm_depth", 4)
 
