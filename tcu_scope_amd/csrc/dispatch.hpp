@@ -196,6 +196,49 @@ inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned b
     }                                                                      \
   } while (0)
 
+// ----- segments far larger than one block's reach (AUTO only) ---------------------------------
+// A block-per-segment kernel leaves the machine idle when there are fewer segments than
+// compute units (measured at N = 2^28: reduce 148 us at S = 2^20, 31 ms at S = 2^28; scan
+// 353 us at S = 2^21).  From these sizes on a segment is cut into partitions of 65536 halves:
+// reduce = partition sums, then one small block per segment adds them in index order; scan =
+// the single-pass look-back scan with the look-back stopped at segment starts.  Both need a
+// few bytes per partition of temporary device memory, taken in stream order.
+constexpr size_t kHugeReduceSegment = (size_t)1 << 20, kHugeScanSegment = (size_t)1 << 21, kHugePartHalves = 65536;
+
+inline int seg_reduce_huge(const half8_t *in, uint16_t *out, size_t num_segments, size_t S, bool nt, void *stream) {
+  const char *what = "tcu_seg_reduce_f16";
+  const size_t pps = S / kHugePartHalves, parts = num_segments * pps;
+  if (parts > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+  float *partials = static_cast<float *>(stream_alloc(parts * sizeof(float), stream));
+  if (!partials) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partition sums");
+  const size_t n_chunks = num_segments * S / 8;
+  if (nt)
+    launch(partition_sums_kernel<8, true>, (unsigned)parts, 1024u, stream, in, partials, n_chunks);
+  else
+    launch(partition_sums_kernel<8, false>, (unsigned)parts, 1024u, stream, in, partials, n_chunks);
+  launch(segment_of_partials_kernel, (unsigned)num_segments, 256u, stream, static_cast<const float *>(partials), out, pps);
+  stream_free(partials, stream);
+  return TCU_OK;
+}
+
+inline int seg_scan_huge(const half8_t *in, uint4_t *out, uint16_t *totals, size_t num_segments, size_t S, bool nt, void *stream) {
+  const char *what = "tcu_seg_scan_f16";
+  const size_t pps = S / kHugePartHalves, parts = num_segments * pps;
+  if (parts > kMaxGrid || pps > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+  const size_t words = 64 + 2 * parts;  // ticket counter, then one 64-bit descriptor per partition
+  unsigned *ws = static_cast<unsigned *>(stream_alloc(words * sizeof(unsigned), stream));
+  if (!ws) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partition descriptors");
+  const size_t n_chunks = num_segments * S / 8;
+  launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
+  const int static_order = options().static_order ? 1 : 0;
+  if (nt)
+    launch(full_scan_kernel<8, false, true>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals);
+  else
+    launch(full_scan_kernel<8, false, false>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals);
+  stream_free(ws, stream);
+  return TCU_OK;
+}
+
 inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
   SegArgs a{num_segments, segment_size, variant, tiles_per_wave, waves_per_block, false};
   bool generic = false;
@@ -213,6 +256,7 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
     launch(seg_reduce_generic_kernel, (unsigned)grid, (unsigned)gw * 64u, stream, static_cast<const uint16_t *>(d_in), out, num_segments, S);
     return TCU_OK;
   }
+  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeReduceSegment) return seg_reduce_huge(in, out, num_segments, S, nt, stream);
   const size_t n_chunks = N / 8;
   const Plan plan = auto_plan_reduce(S);
   const bool use_block = variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant);
@@ -306,6 +350,7 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
     launch(seg_scan_generic_kernel, (unsigned)grid, (unsigned)gw * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), totals, num_segments, S);
     return TCU_OK;
   }
+  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeScanSegment) return seg_scan_huge(in, out, totals, num_segments, S, nt, stream);
   const size_t n_chunks = N / 8;
   const Plan plan = auto_plan_scan(S);
   const bool use_block = variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant);
@@ -394,6 +439,9 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
   const char *what = "tcu_full_reduce_f16";
   if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
   if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
+  // AUTO with the default partition: partition sums, then one small block adds them (measured
+  // 90 us at 2^28 against 96 us for the single kernel, whose workspace must be zeroed first)
+  const bool two_level = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0;
   if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {
@@ -420,6 +468,15 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
       return TCU_OK;
     }
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    if (two_level) {  // p is 16 waves of 8 tiles; the workspace (sized for the single kernel) holds one float per partition
+      float *partials = static_cast<float *>(d_ws);
+      if (nt)
+        launch(partition_sums_kernel<8, true>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks);
+      else
+        launch(partition_sums_kernel<8, false>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks);
+      launch(segment_of_partials_kernel, 1u, 256u, stream, static_cast<const float *>(partials), static_cast<uint16_t *>(d_out), grid);
+      return TCU_OK;
+    }
     unsigned *ws = static_cast<unsigned *>(d_ws);
     launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
     TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, false, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws);
@@ -476,7 +533,7 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
     unsigned *ws = static_cast<unsigned *>(d_ws);
     const size_t words = 64 + 2 * parts;
     launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
-    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, false, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0);
+    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, false, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr));
     return TCU_OK;
   }
   // the reference's three-kernel sequence: segmented scan + totals, exclusive scan of the totals, add

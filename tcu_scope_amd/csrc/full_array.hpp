@@ -134,8 +134,11 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
 
 // One partition (blockDim/64 * U tiles) per block.  workspace: ticket counter at word 0,
 // descriptors (64-bit: flag << 32 | float bits) from byte 256.
+// parts_per_segment = 0: one scan over the whole array.  Otherwise the array is a sequence of
+// segments of parts_per_segment whole partitions each, scanned independently (segments far
+// larger than what one block can walk), and `totals`, if given, receives every segment's sum.
 template <int U, bool MFMA, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order) {
+__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order, unsigned parts_per_segment, uint16_t *totals) {
   __shared__ float wave_total[kMaxWaves];
   __shared__ unsigned s_part;
   __shared__ float s_prefix;
@@ -166,15 +169,19 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
     float aggregate = 0.0f;
     for (int w = 0; w < WPB; w++) aggregate += wave_total[w];
     float prefix = 0.0f;
-    if (part == 0) {
-      if (lane == 0) atomic_store_u64(desc, kFlagPrefix | __float_as_uint(aggregate));
+    // the scan restarts at every segment: a segment's first partition has nothing to wait for,
+    // and nobody looks back past it
+    const unsigned in_segment = parts_per_segment ? part % parts_per_segment : part;
+    const long long floor = (long long)part - in_segment;
+    if (in_segment == 0) {
+      if (lane == 0) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(aggregate));
     } else {
       if (lane == 0) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
       long long base = (long long)part - 1;
       unsigned polls = 0;
       while (true) {  // every lane of wave 0 takes the same path
         const long long idx = base - lane;
-        unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : kFlagPrefix;
+        unsigned long long d = idx >= floor ? atomic_load_u64(desc + idx) : kFlagPrefix;
         const unsigned flag = (unsigned)(d >> 32);
         const unsigned long long is_prefix = ballot(flag == 2u);
         const unsigned long long is_empty = ballot(flag == 0u);
@@ -196,6 +203,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
       }
       if (lane == 0) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
     }
+    if (totals && parts_per_segment && in_segment == parts_per_segment - 1 && lane == 0) totals[part / parts_per_segment] = f16_bits(prefix + aggregate);
     if (lane == 0) s_prefix = prefix;
   }
   __syncthreads();
@@ -207,6 +215,41 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
     scan_tile<6, MFMA, NT>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
     carry += tile_total;
   }
+}
+
+// Segments far larger than one block's reach, first level: block b adds its partition
+// (blockDim/64 * U tiles) and writes the fp32 partial to partial[b].
+template <int U, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void partition_sums_kernel(const half8_t *__restrict__ in, float *__restrict__ partial_out, size_t n_chunks) {
+  __shared__ float partial[kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  half8_t v[U];
+  load_tiles<U, NT>(v, in, ((size_t)blockIdx.x * WPB + wave) * U * kTileChunks, n_chunks, lane);
+  float accs[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < U; j++) accs[j & 1] = sum8(v[j], accs[j & 1]);
+  const float total = lane_group_sum<6>(accs[0] + accs[1]);
+  if (lane == 63) partial[wave] = total;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.0f;
+    for (int w = 0; w < WPB; w++) s += partial[w];
+    partial_out[blockIdx.x] = s;
+  }
+}
+// second level: block j adds the parts_per_segment partials of segment j (fixed order: lane
+// strides, then lanes, then waves) and writes the fp16 result
+__global__ __launch_bounds__(256) void segment_of_partials_kernel(const float *__restrict__ partial_in, uint16_t *__restrict__ out, size_t parts_per_segment) {
+  __shared__ float partial[4];
+  const int lane = lane_id(), wave = wave_in_block();
+  const float *p = partial_in + (size_t)blockIdx.x * parts_per_segment;
+  float acc = 0.0f;
+  for (size_t i = threadIdx.x; i < parts_per_segment; i += 256) acc += p[i];
+  acc = lane_group_sum<6>(acc);
+  if (lane == 63) partial[wave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = f16_bits((partial[0] + partial[1]) + (partial[2] + partial[3]));
 }
 
 // out[0] = fp16(sum of n halves), one block

@@ -20,5 +20,15 @@ inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, static_cast<hipStream_t>(stream), static_cast<KArgs>(args)...);
 }
 
+// Temporary device memory in stream order (from the device's default memory pool: after the
+// first use a request is served from the pool without a driver allocation).  The block may be
+// used by work enqueued on `stream` between the two calls.
+inline void *stream_alloc(size_t bytes, void *stream) {
+  void *p = nullptr;
+  if (hipMallocAsync(&p, bytes, static_cast<hipStream_t>(stream)) != hipSuccess) return nullptr;
+  return p;
+}
+inline void stream_free(void *p, void *stream) { (void)hipFreeAsync(p, static_cast<hipStream_t>(stream)); }
+
 }  // namespace tcu
 #endif  // TCU_LAUNCH_HPP

@@ -411,5 +411,8 @@ template <typename... KArgs, typename... Args>
 inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void *, Args... args) {
   emu::launch(grid, block, [=]() { kernel(static_cast<KArgs>(args)...); });
 }
+// launches run to completion before they return here, so plain host memory is "stream ordered"
+inline void *stream_alloc(size_t bytes, void *) { return std::malloc(bytes ? bytes : 1); }
+inline void stream_free(void *p, void *) { std::free(p); }
 }  // namespace tcu
 #endif

@@ -228,3 +228,34 @@ def test_full_size_seg_scan(tcu, oracle, seg):
     if seg <= 8192:
         for v in variants_for(tcu, seg):
             assert torch.equal(tcu.seg_scan(gd, seg, variant=v), base), f"grid inputs: {v.name} differs from WAVE_SHUFFLE"
+
+
+@pytest.mark.parametrize("seg_log2", [20, 21, 24, 28])
+def test_segments_larger_than_a_block_can_walk(tcu, oracle, seg_log2):
+    """AUTO on segments of 2^20 halves and more (partition sums / look-back scan restarted at
+    segment starts), up to the whole 2^28 array as one segment: uniform inputs within the
+    tolerance, exact-grid inputs bit for bit, per-segment totals, repeated calls."""
+    import torch
+
+    seg = 1 << seg_log2
+    n = max(1 << 24, seg) if seg_log2 < 28 else seg
+    nseg = n // seg
+    x = oracle.generate_f16(n, 3, oracle.DIST_UNIFORM)
+    xd = to_dev(x)
+    ref = oracle.seg_scan_f64(x, nseg, seg)
+    for rep in range(2):  # the temporaries come from a pool: the second call reuses them
+        expect_ok(oracle, to_host(tcu.seg_reduce(xd, seg)), ref.reshape(nseg, seg)[:, -1], seg, f"reduce seg=2^{seg_log2} call {rep}")
+        tot = torch.zeros(nseg, dtype=torch.float16, device="cuda")
+        got = to_host(tcu.seg_scan(xd, seg, totals=tot))
+        expect_ok(oracle, got, ref, seg, f"scan seg=2^{seg_log2} call {rep}")
+        expect_ok(oracle, to_host(tot), ref.reshape(nseg, seg)[:, -1], seg, f"scan totals seg=2^{seg_log2} call {rep}")
+    g = oracle.generate_f16(n, 4, oracle.DIST_GRID)
+    gd = to_dev(g)
+    want64 = oracle.seg_scan_f64(g, nseg, seg)
+    if np.abs(want64).max() < 4096:  # fp32 sums of multiples of 1/2048 are exact up to 8192
+        want = want64.astype(np.float16).view(np.uint16)
+        assert np.array_equal(to_host(tcu.seg_scan(gd, seg)), want)
+        assert np.array_equal(to_host(tcu.seg_reduce(gd, seg)), want.reshape(nseg, seg)[:, -1])
+    else:
+        expect_ok(oracle, to_host(tcu.seg_scan(gd, seg)), want64, seg, f"grid scan seg=2^{seg_log2}")
+        expect_ok(oracle, to_host(tcu.seg_reduce(gd, seg)), want64.reshape(nseg, seg)[:, -1], seg, f"grid reduce seg=2^{seg_log2}")
