@@ -130,6 +130,7 @@ inline Plan auto_plan_reduce(size_t S) {
   if (S == 2048) return {false, 1, 1};
   if (S == 4096) return {true, 2, 4};
   if (S == 8192) return {true, 4, 8};
+  if (S >= 262144) return {true, 2, 8};
   return {true, 1, 8};
 }
 inline Plan auto_plan_scan(size_t S) {
@@ -138,7 +139,9 @@ inline Plan auto_plan_scan(size_t S) {
   if (S == 2048) return {true, 4, 2};
   if (S == 4096) return {true, 1, 2};
   if (S == 8192) return {true, 4, 8};
-  return {true, 2, 16};
+  if (S == 16384) return {true, 2, 16};
+  if (S == 32768) return {true, 8, 8};
+  return {true, 8, 16};
 }
 
 inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || v == TCU_VARIANT_MFMA_256N_BLOCK || v == TCU_VARIANT_BLOCK_LDS; }
