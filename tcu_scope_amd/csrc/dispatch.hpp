@@ -37,6 +37,7 @@ struct Options {
   bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers without staging registers, that many LDS buffers; 0: register-staged kernel; -1: by K
+  bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
 };
 inline Options &options() {
@@ -52,6 +53,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemm_big_tiles") o.gemm_big_tiles = value != 0;
   else if (n == "gemm_direct_lds") o.gemm_direct_lds = value;
   else if (n == "gemm_depth") o.gemm_depth = value;
+  else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
   else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
   return TCU_OK;
@@ -506,6 +508,8 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
   const char *what = "tcu_full_scan_f16";
   if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
   if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
+  // AUTO with the default partition: the kernel that parks 4 more tiles per wave in LDS
+  const bool lds_held = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && options().scan_lds_tiles;
   if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {
@@ -536,6 +540,14 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
     unsigned *ws = static_cast<unsigned *>(d_ws);
     const size_t words = 64 + 2 * parts;
     launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
+    if (lds_held) {  // partitions of 16 x 12 tiles: fewer than `parts`, same workspace layout
+      const size_t big_parts = (n_tiles + 16 * 12 - 1) / (16 * 12);
+      if (nt)
+        launch(full_scan_lds_kernel<8, 4, true>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0);
+      else
+        launch(full_scan_lds_kernel<8, 4, false>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0);
+      return TCU_OK;
+    }
     TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, false, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr));
     return TCU_OK;
   }

@@ -217,6 +217,108 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   }
 }
 
+// The look-back scan with more bytes in flight per wave slot.  A block of full_scan_kernel
+// waits about 30 % of its life for its predecessors' aggregates with its whole partition
+// parked in registers and nothing in flight; wave slots (32 per CU), not registers, cap what a
+// CU can hold.  Here every wave parks ULDS more tiles in LDS (global -> LDS transfers, no
+// registers involved): 16 waves x (8 + 4) tiles = 98304 halves per partition, 64 KiB of LDS
+// per block, still two blocks per CU.  Tiles U .. U+ULDS-1 of a wave follow its register
+// tiles in memory and in scan order.  Same workspace and descriptors as full_scan_kernel.
+template <int U, int ULDS, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order) {
+  __shared__ __attribute__((aligned(1024))) half_t held[kMaxWaves * ULDS * kTileHalves];
+  __shared__ float wave_total[kMaxWaves];
+  __shared__ unsigned s_part;
+  __shared__ float s_prefix;
+  const int lane = lane_id();
+  const int wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  unsigned long long *desc = reinterpret_cast<unsigned long long *>(ws + 64);
+  ScanOperands ops;
+
+  if (!static_order) {
+    if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
+    __syncthreads();
+  }
+  const unsigned part = static_order ? blockIdx.x : s_part;
+  const size_t t0 = ((size_t)part * WPB + wave) * (U + ULDS);
+
+  half8_t v[U];
+  load_tiles<U, NT>(v, in, t0 * kTileChunks, n_chunks, lane);
+  half_t *mine = held + (size_t)wave * ULDS * kTileHalves;
+  const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < ULDS; j++) {
+    const size_t c0 = (t0 + U + j) * kTileChunks;
+    if (c0 + lane < n_chunks)
+      load_chunk_to_lds(in + c0, (uint32_t)lane * 16u, lds_address_of(mine + j * kTileHalves));
+    else
+      *reinterpret_cast<half8_t *>(mine + j * kTileHalves + lane * 8) = zero;
+  }
+  float acc = 0.0f;
+#pragma unroll
+  for (int j = 0; j < U; j++) acc = sum8(v[j], acc);
+  wait_vector_loads<0>();
+#pragma unroll
+  for (int j = 0; j < ULDS; j++) acc = sum8(*reinterpret_cast<const half8_t *>(mine + j * kTileHalves + lane * 8), acc);
+  acc = lane_group_sum<6>(acc);
+  if (lane == 63) wave_total[wave] = acc;
+  __syncthreads();
+
+  if (wave == 0) {
+    float aggregate = 0.0f;
+    for (int w = 0; w < WPB; w++) aggregate += wave_total[w];
+    float prefix = 0.0f;
+    if (part == 0) {
+      if (lane == 0) atomic_store_u64(desc, kFlagPrefix | __float_as_uint(aggregate));
+    } else {
+      if (lane == 0) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
+      long long base = (long long)part - 1;
+      unsigned polls = 0;
+      while (true) {  // every lane of wave 0 takes the same path
+        const long long idx = base - lane;
+        unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : kFlagPrefix;
+        const unsigned flag = (unsigned)(d >> 32);
+        const unsigned long long is_prefix = ballot(flag == 2u);
+        const unsigned long long is_empty = ballot(flag == 0u);
+        const int first_prefix = is_prefix ? __builtin_ctzll(is_prefix) : 64;
+        const unsigned long long needed = first_prefix >= 63 ? ~0ull : ((2ull << first_prefix) - 1ull);
+        if (is_empty & needed) {
+          if (++polls > (1u << 20)) {  // give up: never spin without bound
+            if (lane == 0) atomic_add_u32(ws + 1, 1u);
+            break;
+          }
+          spin_pause();
+          continue;
+        }
+        float val = lane <= first_prefix ? __uint_as_float((unsigned)d) : 0.0f;
+        val = lane_group_sum<6>(val);
+        prefix += readlane(val, 63);
+        if (first_prefix < 64) break;
+        base -= 64;
+      }
+      if (lane == 0) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
+    }
+    if (lane == 0) s_prefix = prefix;
+  }
+  __syncthreads();
+  float carry = s_prefix;
+  for (int w = 0; w < wave; w++) carry += wave_total[w];
+#pragma unroll
+  for (int j = 0; j < U; j++) {
+    float tile_total;
+    scan_tile<6, false, NT>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    carry += tile_total;
+  }
+#pragma unroll
+  for (int j = 0; j < ULDS; j++) {
+    float tile_total;
+    const half8_t h = *reinterpret_cast<const half8_t *>(mine + j * kTileHalves + lane * 8);
+    scan_tile<6, false, NT>(h, carry, ops, lane, out, (t0 + U + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    carry += tile_total;
+  }
+}
+
 // Segments far larger than one block's reach, first level: block b adds its partition
 // (blockDim/64 * U tiles) and writes the fp32 partial to partial[b].
 template <int U, bool NT>

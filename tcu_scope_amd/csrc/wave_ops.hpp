@@ -170,6 +170,7 @@ template <int N>
 TCU_DEVICE void wait_vector_loads() {
   static_assert(N >= 0 && N <= 63, "vmcnt has 6 bits");
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  asm volatile("" ::: "memory");  // later reads of what the loads wrote stay behind the wait
 }
 
 // Block barrier for code that orders its own memory traffic: waits for this wave's LDS

@@ -126,7 +126,7 @@ def test_generic_segment_sizes_and_preconditions(emu, oracle):
 
 def test_full_array_kernels(emu, oracle):
     sz = ctypes.c_size_t
-    for n in (8, 1003, 8192 * 3 + 1024, (1 << 16) + 56):
+    for n in (8, 1003, 8192 * 3 + 1024, (1 << 16) + 56, 2 * 98304 + 8 * 37):
         x = oracle.generate_f16(n, 5, oracle.DIST_GRID)
         w64 = oracle.seg_scan_f64(x, 1, n)
         xi = copy_in(x)
