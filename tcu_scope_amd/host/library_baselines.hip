@@ -1,0 +1,244 @@
+// Library comparators measured beside the hand-written kernels, under the names of the
+// reference's library baselines: CUB_FULL_REDUCTION / CUB_FULL_PREFIXSUM
+// (src/reduction/cub.cu, src/prefixsum/cub.cu: cub::DeviceReduce::Sum,
+// cub::DeviceScan::InclusiveSum), CUB_DEVICE_SEGMENTED_REDUCTION and its TUNE sweep
+// (src/reduction/seg_cub_device.cu:18-63: cub::DeviceSegmentedReduce::Sum over an offsets
+// array), CUBLAS_WMMA_GEMM (src/gemm/cublas.cu:65: cublasGemmEx, fp16 in, fp32 out) and
+// CUBLAS_GEMV.  Here they run hipCUB (rocPRIM) and rocBLAS, the libraries this GPU ships with.
+// Nothing of the product calls these libraries; the file only feeds the benchmark executable.
+// Arithmetic: the reductions and the scan read fp16, accumulate in fp32 and write fp16 (the
+// reference's patched CUB adds in fp16), so they move the same bytes as the kernels they are
+// compared with.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <hipcub/hipcub.hpp>
+#include <rocblas/rocblas.h>
+
+#include <vector>
+
+#include "args.hpp"
+#include "harness.hpp"
+
+using harness::DeviceBuffer;
+using harness::EventPair;
+
+namespace {
+
+struct HalfToFloat {
+  __host__ __device__ float operator()(const __half &h) const { return __half2float(h); }
+};
+using HalfAsFloat = hipcub::TransformInputIterator<float, HalfToFloat, const __half *>;
+
+// an fp16 destination that takes fp32 values (rocPRIM assigns its accumulator type to *out)
+struct HalfOut {
+  __half *p;
+  struct Ref {
+    __half *p;
+    __host__ __device__ Ref &operator=(float v) {
+      *p = __float2half(v);
+      return *this;
+    }
+  };
+  using iterator_category = std::random_access_iterator_tag;
+  using value_type = float;
+  using difference_type = std::ptrdiff_t;
+  using pointer = void;
+  using reference = Ref;
+  __host__ __device__ Ref operator*() const { return Ref{p}; }
+  __host__ __device__ Ref operator[](difference_type i) const { return Ref{p + i}; }
+  __host__ __device__ HalfOut operator+(difference_type i) const { return HalfOut{p + i}; }
+  __host__ __device__ HalfOut &operator+=(difference_type i) {
+    p += i;
+    return *this;
+  }
+};
+
+template <class Body>
+void guarded(benchmark::State &state, Body body) {
+  try {
+    body();
+  } catch (const std::exception &e) {
+    state.SkipWithError(e.what());
+  } catch (...) {
+    state.SkipWithError("unknown exception");
+  }
+}
+
+template <class Launch>
+void timed_loop(benchmark::State &state, Launch launch) {
+  EventPair ev;
+  size_t it = 0;
+  for (auto _ : state) {
+    ev.start();
+    launch(it++);
+    const float ms = ev.stop_ms();
+    state.PauseTiming();
+    state.SetIterationTime(ms / 1000);
+    state.ResumeTiming();
+  }
+}
+
+void counters(benchmark::State &state, size_t num_segments, size_t segment_size, size_t num_elements, double bytes) {
+  state.counters.insert({{"num_segments", (double)num_segments},
+                         {"segment_size", (double)segment_size},
+                         {"num_elements", (double)num_elements},
+                         {"flops", {state.iterations() * 1.0 * num_elements, benchmark::Counter::kAvgThreadsRate}},
+                         {"bytes_per_second", {state.iterations() * bytes, benchmark::Counter::kAvgThreadsRate}},
+                         {"hbm_peak_fraction", {state.iterations() * bytes / 8e12, benchmark::Counter::kAvgThreadsRate}}});
+}
+
+}  // namespace
+
+static void CUB_FULL_REDUCTION(benchmark::State &state) {
+  guarded(state, [&] {
+    const size_t n = state.range(0);
+    const int nin = n <= ((size_t)1 << 29) ? 2 : 1;
+    DeviceBuffer in[2] = {DeviceBuffer(n * 2), DeviceBuffer(nin == 2 ? n * 2 : 16)};
+    DeviceBuffer out(16);
+    for (int i = 0; i < nin; i++) harness::fill_input(in[i].get(), n, harness::flags().seed + i);
+    size_t temp_bytes = 0;
+    HalfAsFloat src0(static_cast<const __half *>(in[0].get()), HalfToFloat());
+    PRINT_IF_ERROR(hipcub::DeviceReduce::Sum(nullptr, temp_bytes, src0, HalfOut{static_cast<__half *>(out.get())}, (int)n));
+    DeviceBuffer temp(temp_bytes ? temp_bytes : 16);
+    timed_loop(state, [&](size_t it) {
+      HalfAsFloat src(static_cast<const __half *>(in[it % nin].get()), HalfToFloat());
+      PRINT_IF_ERROR(hipcub::DeviceReduce::Sum(temp.get(), temp_bytes, src, HalfOut{static_cast<__half *>(out.get())}, (int)n));
+    });
+    counters(state, 1, n, n, 2.0 * n);
+  });
+}
+BENCHMARK(CUB_FULL_REDUCTION)->ARGS()->UseManualTime();
+
+static void CUB_FULL_PREFIXSUM(benchmark::State &state) {
+  guarded(state, [&] {
+    const size_t n = state.range(0);
+    const int nin = n <= ((size_t)1 << 29) ? 2 : 1;
+    DeviceBuffer in[2] = {DeviceBuffer(n * 2), DeviceBuffer(nin == 2 ? n * 2 : 16)};
+    DeviceBuffer out(n * 2);
+    for (int i = 0; i < nin; i++) harness::fill_input(in[i].get(), n, harness::flags().seed + i);
+    size_t temp_bytes = 0;
+    HalfAsFloat src0(static_cast<const __half *>(in[0].get()), HalfToFloat());
+    PRINT_IF_ERROR(hipcub::DeviceScan::InclusiveSum(nullptr, temp_bytes, src0, HalfOut{static_cast<__half *>(out.get())}, (int)n));
+    DeviceBuffer temp(temp_bytes ? temp_bytes : 16);
+    timed_loop(state, [&](size_t it) {
+      HalfAsFloat src(static_cast<const __half *>(in[it % nin].get()), HalfToFloat());
+      PRINT_IF_ERROR(hipcub::DeviceScan::InclusiveSum(temp.get(), temp_bytes, src, HalfOut{static_cast<__half *>(out.get())}, (int)n));
+    });
+    counters(state, 1, n, n, 4.0 * n);
+  });
+}
+BENCHMARK(CUB_FULL_PREFIXSUM)->ARGS()->UseManualTime();
+
+static void run_device_segmented_reduction(benchmark::State &state) {
+  guarded(state, [&] {
+    const size_t num_segments = state.range(0), segment_size = state.range(1), n = num_segments * segment_size;
+    if (n >= ((size_t)1 << 31) || num_segments >= ((size_t)1 << 31)) {
+      state.SkipWithError("offsets are 32-bit integers");
+      return;
+    }
+    const int nin = n <= ((size_t)1 << 29) ? 2 : 1;
+    DeviceBuffer in[2] = {DeviceBuffer(n * 2), DeviceBuffer(nin == 2 ? n * 2 : 16)};
+    DeviceBuffer out(num_segments * 2), offsets((num_segments + 1) * sizeof(int));
+    for (int i = 0; i < nin; i++) harness::fill_input(in[i].get(), n, harness::flags().seed + i);
+    {
+      std::vector<int> h(num_segments + 1);
+      for (size_t j = 0; j <= num_segments; j++) h[j] = (int)(j * segment_size);
+      PRINT_IF_ERROR(hipMemcpy(offsets.get(), h.data(), h.size() * sizeof(int), hipMemcpyHostToDevice));
+    }
+    const int *off = static_cast<const int *>(offsets.get());
+    size_t temp_bytes = 0;
+    HalfAsFloat src0(static_cast<const __half *>(in[0].get()), HalfToFloat());
+    PRINT_IF_ERROR(hipcub::DeviceSegmentedReduce::Sum(nullptr, temp_bytes, src0, HalfOut{static_cast<__half *>(out.get())}, (int)num_segments, off, off + 1));
+    DeviceBuffer temp(temp_bytes ? temp_bytes : 16);
+    timed_loop(state, [&](size_t it) {
+      HalfAsFloat src(static_cast<const __half *>(in[it % nin].get()), HalfToFloat());
+      PRINT_IF_ERROR(hipcub::DeviceSegmentedReduce::Sum(temp.get(), temp_bytes, src, HalfOut{static_cast<__half *>(out.get())}, (int)num_segments, off, off + 1));
+    });
+    counters(state, num_segments, segment_size, n, 2.0 * n + 2.0 * num_segments + 4.0 * num_segments);
+  });
+}
+static void CUB_DEVICE_SEGMENTED_REDUCTION(benchmark::State &state) { run_device_segmented_reduction(state); }
+static void CUB_DEVICE_TUNE_SEGMENTED_REDUCTION(benchmark::State &state) { run_device_segmented_reduction(state); }
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_16_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_32_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_64_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_128_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_256_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_512_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_1024_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_2048_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_4096_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_8192_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_16384_ARGS()->UseManualTime();
+BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
+
+// ---- rocBLAS ------------------------------------------------------------------------------------
+namespace {
+rocblas_handle blas() {
+  static rocblas_handle h = [] {
+    rocblas_handle x = nullptr;
+    if (rocblas_create_handle(&x) != rocblas_status_success) throw std::runtime_error("rocblas_create_handle failed");
+    return x;
+  }();
+  return h;
+}
+void check_blas(rocblas_status s, const char *what) {
+  if (s != rocblas_status_success) throw std::runtime_error(std::string(what) + ": rocBLAS status " + std::to_string((int)s));
+}
+}  // namespace
+
+// D (M x N row-major) = alpha * A (M x K row-major) * B (K x N column-major) + beta * C, the
+// layouts of tcu_gemm_f16_f32.  In rocBLAS's column-major terms: D^T (N x M) = op(B) * A'.
+static void CUBLAS_WMMA_GEMM(benchmark::State &state) {
+  guarded(state, [&] {
+    const size_t M = state.range(0), N = state.range(1), K = state.range(2);
+    const float alpha = 1.1f, beta = 1.2f;
+    DeviceBuffer A(M * K * 2), B(N * K * 2), C(M * N * 4), D(M * N * 4);
+    TCU_CHECK(tcu_generate_f16(A.get(), M * K, harness::flags().seed, TCU_DIST_NORMAL, 0, nullptr));
+    TCU_CHECK(tcu_generate_f16(B.get(), N * K, harness::flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
+    PRINT_IF_ERROR(hipMemset(C.get(), 0, M * N * 4));
+    auto run = [&] {
+      check_blas(rocblas_gemm_ex(blas(), rocblas_operation_transpose, rocblas_operation_none, (rocblas_int)N, (rocblas_int)M, (rocblas_int)K, &alpha, B.get(), rocblas_datatype_f16_r, (rocblas_int)K, A.get(),
+                                 rocblas_datatype_f16_r, (rocblas_int)K, &beta, C.get(), rocblas_datatype_f32_r, (rocblas_int)N, D.get(), rocblas_datatype_f32_r, (rocblas_int)N, rocblas_datatype_f32_r,
+                                 rocblas_gemm_algo_standard, 0, 0),
+                 "rocblas_gemm_ex");
+    };
+    run();
+    PRINT_IF_ERROR(hipDeviceSynchronize());
+    timed_loop(state, [&](size_t) { run(); });
+    state.counters.insert({{"M", (double)M},
+                           {"N", (double)N},
+                           {"K", (double)K},
+                           {"flops", {state.iterations() * 2.0 * M * N * K, benchmark::Counter::kAvgThreadsRate}},
+                           {"mfma_peak_fraction", {state.iterations() * 2.0 * M * N * K / 2.5e15, benchmark::Counter::kAvgThreadsRate}}});
+  });
+}
+BENCHMARK(CUBLAS_WMMA_GEMM)->Apply(GemmArgs)->UseManualTime();
+
+// y (M) = alpha * A (M x K row-major) x + beta * y as a one-column GEMM (fp16 in, fp32 out)
+static void CUBLAS_GEMV(benchmark::State &state) {
+  guarded(state, [&] {
+    const size_t M = state.range(0), K = state.range(1);
+    const float alpha = 1.0f, beta = 0.0f;
+    DeviceBuffer A(M * K * 2), x(K * 2), y(M * 4);
+    TCU_CHECK(tcu_generate_f16(A.get(), M * K, harness::flags().seed, TCU_DIST_NORMAL, 0, nullptr));
+    TCU_CHECK(tcu_generate_f16(x.get(), K, harness::flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
+    PRINT_IF_ERROR(hipMemset(y.get(), 0, M * 4));
+    auto run = [&] {
+      check_blas(rocblas_gemm_ex(blas(), rocblas_operation_transpose, rocblas_operation_none, (rocblas_int)M, 1, (rocblas_int)K, &alpha, A.get(), rocblas_datatype_f16_r, (rocblas_int)K, x.get(),
+                                 rocblas_datatype_f16_r, (rocblas_int)K, &beta, y.get(), rocblas_datatype_f32_r, (rocblas_int)M, y.get(), rocblas_datatype_f32_r, (rocblas_int)M, rocblas_datatype_f32_r,
+                                 rocblas_gemm_algo_standard, 0, 0),
+                 "rocblas_gemm_ex");
+    };
+    run();
+    PRINT_IF_ERROR(hipDeviceSynchronize());
+    timed_loop(state, [&](size_t) { run(); });
+    const double bytes = 2.0 * M * K + 2.0 * K + 4.0 * M;
+    state.counters.insert({{"M", (double)M},
+                           {"N", (double)K},
+                           {"flops", {state.iterations() * 2.0 * M * K, benchmark::Counter::kAvgThreadsRate}},
+                           {"bytes_per_second", {state.iterations() * bytes, benchmark::Counter::kAvgThreadsRate}},
+                           {"hbm_peak_fraction", {state.iterations() * bytes / 8e12, benchmark::Counter::kAvgThreadsRate}}});
+  });
+}
+BENCHMARK(CUBLAS_GEMV)->Apply(GemvArgs)->UseManualTime();
