@@ -107,6 +107,16 @@ int tcu_set_option(const char *name, int value);
  * — the reference's WARPS_PER_BLOCK. */
 int tcu_seg_reduce_f16(const void *d_in, void *d_out, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
 
+/* Segments given by offsets: d_out[j] = fp16( sum of d_in[begin[j] .. end[j]) ), an empty
+ * segment (end[j] <= begin[j]) gives 0.  Segments may start at any element, overlap or
+ * leave gaps.  Replaces cub::DeviceSegmentedReduce::Sum(d_temp, bytes, d_in, d_out,
+ * num_segments, d_offsets, d_offsets + 1) as the reference calls it
+ * (src/reduction/seg_cub_device.cu:46-48, 61-63); no temporary storage is needed.
+ * offset_bits: 32 or 64 (signed integers, device memory).  expected_segment_size: the
+ * typical segment length, used to choose how many lanes share a segment (0 = unknown: a
+ * whole wave per segment). */
+int tcu_seg_reduce_offsets_f16(const void *d_in, void *d_out, size_t num_segments, const void *d_begin_offsets, const void *d_end_offsets, int offset_bits, size_t expected_segment_size, void *stream);
+
 /* ---- segmented inclusive prefix sum ------------------------------------------------------ */
 
 /* d_out[j*S + i] = fp16( d_in[j*S] + ... + d_in[j*S + i] ).  d_totals (may be NULL)

@@ -54,6 +54,9 @@ def lib():
         L.tcu_oracle_full_scan_ref.argtypes = [u16p, u16p, sz]
         L.tcu_oracle_add_partial_sums_ref.argtypes = [u16p, u16p, sz, sz]
         L.tcu_oracle_seg_reduce_f64.argtypes = [u16p, f64p, sz, sz]
+        i64p = c.POINTER(c.c_int64)
+        L.tcu_oracle_seg_reduce_offsets_ref.argtypes = [u16p, u16p, sz, i64p, i64p]
+        L.tcu_oracle_seg_reduce_offsets_f64.argtypes = [u16p, f64p, sz, i64p, i64p]
         L.tcu_oracle_seg_scan_f64.argtypes = [u16p, f64p, sz, sz]
         L.tcu_oracle_gemv_f64.argtypes = [u16p, u16p, f32p, f64p, sz, sz, c.c_double, c.c_double]
         L.tcu_oracle_gemm_f64.argtypes = [u16p, u16p, f32p, f64p, sz, sz, sz, c.c_double, c.c_double, sz, sz]
@@ -181,6 +184,32 @@ def seg_reduce_f64(x, num_segments, segment_size):
         _split(num_segments, lambda lo, hi: L.tcu_oracle_seg_reduce_f64(_p(x[lo * S:], ctypes.c_uint16), _p(out[lo:], ctypes.c_double), hi - lo, S))
     else:
         L.tcu_oracle_seg_reduce_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), num_segments, S)
+    return out
+
+
+def _offsets(x, begin, end):
+    begin = np.ascontiguousarray(begin, dtype=np.int64)
+    end = np.ascontiguousarray(end, dtype=np.int64)
+    assert begin.shape == end.shape and begin.ndim == 1
+    live = end > begin
+    assert not live.any() or (begin[live].min() >= 0 and end[live].max() <= x.size)
+    return begin, end
+
+
+def seg_reduce_offsets_ref(x, begin, end):
+    """fp32 sequential sum of x[begin[j]:end[j]] per segment, fp16 bits out."""
+    x = _u16(x)
+    begin, end = _offsets(x, begin, end)
+    out = np.empty(begin.size, dtype=np.uint16)
+    lib().tcu_oracle_seg_reduce_offsets_ref(_p(x, ctypes.c_uint16), _p(out, ctypes.c_uint16), begin.size, _p(begin, ctypes.c_int64), _p(end, ctypes.c_int64))
+    return out
+
+
+def seg_reduce_offsets_f64(x, begin, end):
+    x = _u16(x)
+    begin, end = _offsets(x, begin, end)
+    out = np.empty(begin.size, dtype=np.float64)
+    lib().tcu_oracle_seg_reduce_offsets_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), begin.size, _p(begin, ctypes.c_int64), _p(end, ctypes.c_int64))
     return out
 
 

@@ -84,7 +84,14 @@ void tcu_oracle_full_scan_ref(const uint16_t *in, uint16_t *out, size_t n);
  * one fp16 addition per element. */
 void tcu_oracle_add_partial_sums_ref(uint16_t *out, const uint16_t *partial_sums, size_t num_segments, size_t segment_size);
 
+/* Segments given by offsets: segment j covers in[begin[j], end[j]) and is empty when
+ * end[j] <= begin[j]: the argument convention of cub::DeviceSegmentedReduce::Sum as the
+ * reference calls it (src/reduction/seg_cub_device.cu:46-48: d_offsets, d_offsets + 1).
+ * fp32 sequential sum, fp16 result, like the fixed-size loop above. */
+void tcu_oracle_seg_reduce_offsets_ref(const uint16_t *in, uint16_t *out, size_t num_segments, const int64_t *begin, const int64_t *end);
+
 /* ---- definition (fp64) -------------------------------------------------------------- */
+void tcu_oracle_seg_reduce_offsets_f64(const uint16_t *in, double *out, size_t num_segments, const int64_t *begin, const int64_t *end);
 void tcu_oracle_seg_reduce_f64(const uint16_t *in, double *out, size_t num_segments, size_t segment_size);
 void tcu_oracle_seg_scan_f64(const uint16_t *in, double *out, size_t num_segments, size_t segment_size);
 /* y = alpha*A*x + beta*y0; A is M x K row-major fp16, x fp16, y0 may be NULL when beta==0 */

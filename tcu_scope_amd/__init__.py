@@ -27,6 +27,7 @@ from .binding import (  # noqa: F401
     lib,
     library_path,
     seg_reduce,
+    seg_reduce_offsets,
     seg_scan,
     set_option,
     stream_probe,

@@ -305,6 +305,71 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
   return TCU_OK;
 }
 
+// ----- segmented reduction over an offsets array ------------------------------------------------
+
+template <typename OFF>
+inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_segments, const OFF *begin, const OFF *end, size_t expected, void *stream) {
+  const int vector = aligned16(in) ? 1 : 0;
+  const bool nt = options().nontemporal;
+  // expected length of 2^17 halves and more: several 1024-thread blocks per segment (about
+  // 65536 halves each), fp32 partials in stream-ordered temporary memory, then one small
+  // block per segment adds them.  (A wave per segment: 158 us at 2^19, 57 ms for one 2^28 segment.)
+  if (expected >= ((size_t)1 << 17)) {
+    size_t slices = (expected + 65535) / 65536;
+    if (slices > 4096) slices = 4096;
+    const size_t blocks = num_segments * slices;
+    if (blocks > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_offsets_f16: grid exceeds the launch limit");
+    float *partials = static_cast<float *>(stream_alloc(blocks * sizeof(float), stream));
+    if (!partials) return fail(TCU_ERR_RUNTIME, "tcu_seg_reduce_offsets_f16: no temporary device memory for the partial sums");
+    if (nt)
+      launch(seg_reduce_offsets_sliced_kernel<OFF, true>, (unsigned)blocks, 1024u, stream, in, partials, begin, end, (unsigned)slices, vector);
+    else
+      launch(seg_reduce_offsets_sliced_kernel<OFF, false>, (unsigned)blocks, 1024u, stream, in, partials, begin, end, (unsigned)slices, vector);
+    launch(segment_of_partials_kernel, (unsigned)num_segments, 256u, stream, static_cast<const float *>(partials), out, slices);
+    stream_free(partials, stream);
+    return TCU_OK;
+  }
+  // lanes per segment: about one 128-bit chunk per lane for the expected length, a whole wave when unknown
+  int g_log2 = 6;
+  if (expected) {
+    g_log2 = 1;
+    while (g_log2 < 6 && ((size_t)8 << g_log2) < expected) g_log2++;
+  }
+  const size_t threads = num_segments << g_log2;
+  const size_t grid = (threads + 255) / 256;
+  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_offsets_f16: grid exceeds the launch limit");
+#define TCU_OFFSETS_CASE(GL)                                                                                                              \
+  case GL:                                                                                                                               \
+    if (nt)                                                                                                                              \
+      launch(seg_reduce_offsets_kernel<OFF, GL, true>, (unsigned)grid, 256u, stream, in, out, num_segments, begin, end, vector);          \
+    else                                                                                                                                 \
+      launch(seg_reduce_offsets_kernel<OFF, GL, false>, (unsigned)grid, 256u, stream, in, out, num_segments, begin, end, vector);         \
+    break
+  switch (g_log2) {
+    TCU_OFFSETS_CASE(1);
+    TCU_OFFSETS_CASE(2);
+    TCU_OFFSETS_CASE(3);
+    TCU_OFFSETS_CASE(4);
+    TCU_OFFSETS_CASE(5);
+    default:
+      TCU_OFFSETS_CASE(6);
+  }
+#undef TCU_OFFSETS_CASE
+  return TCU_OK;
+}
+
+inline int seg_reduce_offsets_dispatch(const void *d_in, void *d_out, size_t num_segments, const void *d_begin, const void *d_end, int offset_bits, size_t expected, void *stream) {
+  const char *what = "tcu_seg_reduce_offsets_f16";
+  if (offset_bits != 32 && offset_bits != 64) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": offset_bits must be 32 or 64");
+  if (num_segments == 0) return TCU_OK;
+  if (!d_in || !d_out || !d_begin || !d_end) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  if (num_segments > ((size_t)1 << 56)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": too many segments");
+  const uint16_t *in = static_cast<const uint16_t *>(d_in);
+  uint16_t *out = static_cast<uint16_t *>(d_out);
+  if (offset_bits == 32) return seg_reduce_offsets_typed(in, out, num_segments, static_cast<const int32_t *>(d_begin), static_cast<const int32_t *>(d_end), expected, stream);
+  return seg_reduce_offsets_typed(in, out, num_segments, static_cast<const int64_t *>(d_begin), static_cast<const int64_t *>(d_end), expected, stream);
+}
+
 // ----- segmented inclusive prefix sum -------------------------------------------------------
 
 template <int LPS_LOG2, bool MFMA>

@@ -258,4 +258,86 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_generic_kernel(const uin
   if (lane == 63) out[seg] = f16_bits(acc);
 }
 
+// Segments given by offsets: segment j = in[begin[j], end[j]) in halves, empty when
+// end[j] <= begin[j]; segments may start anywhere, overlap or leave gaps (the interface of
+// cub::DeviceSegmentedReduce::Sum as the reference calls it, src/reduction/seg_cub_device.cu:46-48).
+// G = 2^G_LOG2 adjacent lanes share a segment: the part between the first and the last
+// 16-byte boundary inside the segment goes through 128-bit loads (lane `sub` takes chunks
+// sub, sub + G, ..., four in flight), the ragged head and tail (< 8 halves each) through
+// 2-byte loads, and a DPP butterfly adds the G partial sums.  With `vector` false (input not
+// 16-byte aligned) everything takes the 2-byte path.
+// this lane's share of the sum over in[b, e): lane `sub` of `g` lanes that split the range
+template <bool NT>
+TCU_DEVICE float offsets_range_sum(const uint16_t *__restrict__ in, size_t b, size_t e, size_t sub, size_t g, int vector) {
+  size_t body_b = (b + 7) & ~(size_t)7, body_e = e & ~(size_t)7;  // aligned part [body_b, body_e)
+  if (!vector || body_b >= body_e) body_b = body_e = e;            // none: the head is the whole range
+  float acc = 0.0f, acc1 = 0.0f;
+  for (size_t i = b + sub; i < body_b; i += g) acc += (float)__builtin_bit_cast(half_t, in[i]);
+  for (size_t i = body_e + sub; i < e; i += g) acc += (float)__builtin_bit_cast(half_t, in[i]);
+  const half8_t *chunks = reinterpret_cast<const half8_t *>(in);
+  size_t c = body_b / 8 + sub;
+  const size_t ce = body_e / 8;
+  for (; c + 3 * g < ce; c += 4 * g) {
+    const half8_t v0 = load_chunk<NT>(chunks + c), v1 = load_chunk<NT>(chunks + c + g), v2 = load_chunk<NT>(chunks + c + 2 * g), v3 = load_chunk<NT>(chunks + c + 3 * g);
+    acc = sum8(v0, acc);
+    acc1 = sum8(v1, acc1);
+    acc = sum8(v2, acc);
+    acc1 = sum8(v3, acc1);
+  }
+  for (; c < ce; c += g) acc = sum8(load_chunk<NT>(chunks + c), acc);
+  return acc + acc1;
+}
+
+template <typename OFF, int G_LOG2, bool NT>
+__global__ __launch_bounds__(256) void seg_reduce_offsets_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, size_t num_segments, const OFF *__restrict__ begin,
+                                                                 const OFF *__restrict__ end, int vector) {
+  constexpr int G = 1 << G_LOG2;
+  const int lane = lane_id();
+  const int sub = lane & (G - 1);
+  const size_t seg = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> G_LOG2;
+  const bool live = seg < num_segments;
+  size_t b = 0, e = 0;
+  if (live) {
+    const OFF ob = begin[seg], oe = end[seg];
+    if (oe > ob) {
+      b = (size_t)ob;
+      e = (size_t)oe;
+    }
+  }
+  const float total = lane_group_sum<G_LOG2>(offsets_range_sum<NT>(in, b, e, (size_t)sub, (size_t)G, vector));
+  const bool holder = G_LOG2 <= 4 ? sub == 0 : sub == G - 1;
+  if (live && holder) out[seg] = f16_bits(total);
+}
+
+// Long segments: `slices` blocks share a segment.  Block (segment j, slice p) adds the p-th of
+// `slices` equal parts of the segment (part length rounded up to whole 128-bit chunks) and
+// writes an fp32 partial to partial[j * slices + p]; a second kernel adds the partials.
+template <typename OFF, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void seg_reduce_offsets_sliced_kernel(const uint16_t *__restrict__ in, float *__restrict__ partial_out, const OFF *__restrict__ begin,
+                                                                              const OFF *__restrict__ end, unsigned slices, int vector) {
+  __shared__ float partial[kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const size_t seg = blockIdx.x / slices, p = blockIdx.x % slices;
+  size_t b = 0, e = 0;
+  {
+    const OFF ob = begin[seg], oe = end[seg];
+    if (oe > ob) {
+      b = (size_t)ob;
+      e = (size_t)oe;
+    }
+  }
+  const size_t part = (((e - b) + slices - 1) / slices + 7) & ~(size_t)7;
+  size_t sb = b + p * part, se = sb + part;
+  if (sb > e) sb = e;
+  if (se > e) se = e;
+  const float total = lane_group_sum<6>(offsets_range_sum<NT>(in, sb, se, (size_t)threadIdx.x, (size_t)blockDim.x, vector));
+  if (lane == 63) partial[wave] = total;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.0f;
+    for (unsigned w = 0; w < (blockDim.x >> 6); w++) s += partial[w];
+    partial_out[blockIdx.x] = s;
+  }
+}
+
 }  // namespace tcu

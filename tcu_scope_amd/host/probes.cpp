@@ -104,3 +104,14 @@ SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_MFMA_16N);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_MFMA_16N_BLOCK);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_WAVE_SHUFFLE);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_BLOCK_LDS);
+
+// ---- segmented reduction through an offsets array (the hand-written counterpart of the
+// CUB_DEVICE_SEGMENTED_REDUCTION library baseline; same offsets, same argument tuples) ------------
+static void TCU_OFFSETS_SEGMENTED_REDUCTION(benchmark::State &state) { harness::run_seg_reduce_offsets(state, true, "TCU_OFFSETS_SEGMENTED_REDUCTION"); }
+// without the length hint: a whole wave per segment
+static void TCU_OFFSETS_NOHINT_SEGMENTED_REDUCTION(benchmark::State &state) { harness::run_seg_reduce_offsets(state, false, "TCU_OFFSETS_NOHINT_SEGMENTED_REDUCTION"); }
+BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
+BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_16_ARGS()->UseManualTime();
+BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_256_ARGS()->UseManualTime();
+BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_4096_ARGS()->UseManualTime();
+BENCHMARK(TCU_OFFSETS_NOHINT_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();

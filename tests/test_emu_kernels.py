@@ -37,6 +37,7 @@ def emu():
     L.emu_gemv_f16_f32.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci]
     L.emu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
     L.emu_set_option.argtypes = [ctypes.c_char_p, ci]
+    L.emu_seg_reduce_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz]
     L.emu_generate_f16.argtypes = [vp, sz, ctypes.c_uint64, ci, sz]
     L.emu_last_error.restype = ctypes.c_char_p
     return L
@@ -106,6 +107,47 @@ def test_segments_larger_than_a_block_can_walk(emu, oracle):
     assert emu.emu_seg_scan_f16(xi.ctypes.data, out.ctypes.data, tot.ctypes.data, nseg, seg, V_AUTO, 0, 0) == 0, emu.emu_last_error()
     assert np.array_equal(out[:nseg * seg], want) and np.all(out[nseg * seg:] == 0xFFFF)
     assert np.array_equal(tot[:nseg], want.reshape(nseg, seg)[:, -1]) and np.all(tot[nseg:] == 0xFFFF)
+
+
+def ragged_offsets(rng, n, nseg, max_len):
+    """begin/end of nseg segments inside [0, n): arbitrary starts, lengths 0..max_len, some inverted (= empty)."""
+    begin = rng.integers(0, n, nseg)
+    length = rng.integers(0, max_len + 1, nseg)
+    end = np.minimum(begin + length, n)
+    inverted = rng.random(nseg) < 0.05
+    end[inverted] = begin[inverted] - rng.integers(0, 3, inverted.sum())
+    return begin.astype(np.int64), end.astype(np.int64)
+
+
+def test_segmented_reduction_over_offsets(emu, oracle):
+    rng = np.random.default_rng(7)
+    n = 50000
+    x = oracle.generate_f16(n, 9, oracle.DIST_GRID)  # exact partial sums: any order gives the same bits
+    xi = copy_in(x)
+    for max_len, expected, bits in ((20, 16, 32), (20, 0, 64), (300, 128, 64), (3000, 0, 32), (3000, 2048, 32), (40, 64, 32), (40000, 1 << 17, 64), (3000, 3 << 17, 32)):
+        nseg = 12 if expected >= (1 << 17) else 200 if max_len > 1000 else 600
+        begin, end = ragged_offsets(rng, n, nseg, max_len)
+        want = oracle.seg_reduce_offsets_f64(x, begin, end).astype(np.float16).view(np.uint16)
+        assert np.array_equal(want, oracle.seg_reduce_offsets_ref(x, begin, end))
+        dt = np.int32 if bits == 32 else np.int64
+        bi, ei = copy_in(begin.astype(dt), dt), copy_in(end.astype(dt), dt)
+        out = aligned(nseg + 8, np.uint16, 0xFFFF)
+        assert emu.emu_seg_reduce_offsets_f16(xi.ctypes.data, out.ctypes.data, nseg, bi.ctypes.data, ei.ctypes.data, bits, expected) == 0, emu.emu_last_error()
+        assert np.array_equal(out[:nseg], want) and np.all(out[nseg:] == 0xFFFF), (max_len, expected, bits)
+    # the offsets array of the reference's harness: one array, begin = offsets, end = offsets + 1
+    seg, nseg = 48, 500
+    off = copy_in((np.arange(nseg + 1) * seg).astype(np.int32), np.int32)
+    out = aligned(nseg, np.uint16)
+    assert emu.emu_seg_reduce_offsets_f16(xi.ctypes.data, out.ctypes.data, nseg, off.ctypes.data, off.ctypes.data + 4, 32, seg) == 0
+    assert np.array_equal(out, oracle.seg_scan_f64(x, nseg, seg).astype(np.float16).view(np.uint16).reshape(nseg, seg)[:, -1])
+    # input that is not 16-byte aligned: everything through the 2-byte path
+    begin, end = ragged_offsets(rng, n - 1, 300, 100)
+    want = oracle.seg_reduce_offsets_f64(x[1:], begin, end).astype(np.float16).view(np.uint16)
+    bi, ei = copy_in(begin, np.int64), copy_in(end, np.int64)
+    out = aligned(300, np.uint16)
+    assert emu.emu_seg_reduce_offsets_f16(xi.ctypes.data + 2, out.ctypes.data, 300, bi.ctypes.data, ei.ctypes.data, 64, 64) == 0
+    assert np.array_equal(out, want)
+    assert emu.emu_seg_reduce_offsets_f16(xi.ctypes.data, out.ctypes.data, 300, bi.ctypes.data, ei.ctypes.data, 16, 0) == 1
 
 
 def test_generic_segment_sizes_and_preconditions(emu, oracle):

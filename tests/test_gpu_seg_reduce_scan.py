@@ -259,3 +259,42 @@ def test_segments_larger_than_a_block_can_walk(tcu, oracle, seg_log2):
     else:
         expect_ok(oracle, to_host(tcu.seg_scan(gd, seg)), want64, seg, f"grid scan seg=2^{seg_log2}")
         expect_ok(oracle, to_host(tcu.seg_reduce(gd, seg)), want64.reshape(nseg, seg)[:, -1], seg, f"grid reduce seg=2^{seg_log2}")
+
+
+def test_segmented_reduction_over_offsets(tcu, oracle):
+    """tcu_seg_reduce_offsets_f16: ragged, empty, inverted and overlapping segments with 32- and 64-bit offsets and
+    every lanes-per-segment choice, against the fp64 oracle with the per-segment tolerance 2 ulp + 1e-3*sqrt(length);
+    exact-grid inputs bit for bit; uniform offsets must equal tcu_seg_reduce_f16 exactly on such inputs."""
+    import torch
+
+    rng = np.random.default_rng(11)
+    n = 1 << 22
+    x = oracle.generate_f16(n, 8, oracle.DIST_UNIFORM)
+    g = oracle.generate_f16(n, 9, oracle.DIST_GRID)
+    xd, gd = to_dev(x), to_dev(g)
+    for max_len, nseg in ((24, 200000), (700, 50000), (20000, 3000), (1 << 20, 40)):
+        begin = rng.integers(0, n, nseg)
+        end = np.minimum(begin + rng.integers(0, max_len + 1, nseg), n)
+        inv = rng.random(nseg) < 0.03
+        end[inv] = begin[inv] - 1
+        length = np.maximum(end - begin, 0)
+        ref = oracle.seg_reduce_offsets_f64(x, begin, end)
+        want_grid = oracle.seg_reduce_offsets_f64(g, begin, end)
+        exact = np.abs(want_grid).max() < 4096 and max_len <= 20000
+        for dtype in (torch.int32, torch.int64):
+            bd, ed = torch.from_numpy(begin).to(dtype).cuda(), torch.from_numpy(end).to(dtype).cuda()
+            for expected in (0, 16, 100, 512, 1 << 16, 1 << 17, 1 << 20):
+                got = to_host(tcu.seg_reduce_offsets(xd, bd, ed, expected_segment_size=expected)).view(np.float16).astype(np.float64)
+                allow = 2 * np.maximum(np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64), 2.0 ** -24) + 1e-3 * np.sqrt(length)
+                bad = np.abs(got - ref) > allow
+                assert not bad.any(), (max_len, str(dtype), expected, int(bad.sum()), int(np.argmax(bad)))
+                if exact:
+                    gg = to_host(tcu.seg_reduce_offsets(gd, bd, ed, expected_segment_size=expected))
+                    assert np.array_equal(gg, want_grid.astype(np.float16).view(np.uint16)), (max_len, str(dtype), expected)
+    for seg in (16, 48, 256, 4096):
+        nseg = (1 << 20) // seg
+        off = (torch.arange(nseg + 1, dtype=torch.int64) * seg).to(torch.int32).cuda()
+        got = tcu.seg_reduce_offsets(gd, off[:-1], off[1:], expected_segment_size=seg)
+        want = oracle.seg_scan_f64(g, nseg, seg).astype(np.float16).view(np.uint16).reshape(nseg, seg)[:, -1]
+        assert np.array_equal(to_host(got), want), seg
+    assert tcu.seg_reduce_offsets(xd, off[:0], off[:0]).numel() == 0

@@ -38,6 +38,17 @@ def test_benchmark_names_follow_the_reference_grammar():
         "CUDA_WMMA_GEMM_NAIVE/M:8192/N:8192/K:8192/manual_time",
         "CUDA_WMMA_GEMV_NAIVE/M:16384/N:16384/manual_time",
         "CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/segment_size:16/num_elements:1048576/manual_time",
+        # the "unsafe" twins and the library baselines that the reference's plot specs select
+        "CUDA_UNSAFE_WMMA_SEGMENTED_REDUCTION_16N<8>/num_segments:16777216/segment_size:16/num_elements:268435456/manual_time",
+        "CUDA_UNSAFE_WMMA_SEGMENTED_REDUCTION_16N_OPT<2>/num_segments:16777216/segment_size:16/num_elements:268435456/manual_time",
+        "CUDA_UNSAFE_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK<4>/num_segments:16384/segment_size:16384/num_elements:268435456/manual_time",
+        "CUDA_UNSAFE_WMMA_TUNE_SEGMENTED_REDUCTION_256N<4>/num_segments:4194304/segment_size:256/base_segment_size:256/max_elements_log2:30/manual_time",
+        "CUDA_UNSAFE_WMMAFULL_REDUCTION_ATOMIC_W_ATOMIC_BALLOT<2 * 256, 4>/num_elements:1073741824/manual_time",
+        "CUDA_WMMA_FULL_REDUCTION_2KERS_BLOCK_BASE_256<8 * 256, 16>/num_elements:1073741824/manual_time",
+        "CUB_DEVICE_SEGMENTED_REDUCTION/num_segments:16777216/segment_size:16/num_elements:268435456/manual_time",
+        "CUB_FULL_REDUCTION/num_elements:1073741824/manual_time",
+        "CUB_FULL_PREFIXSUM/num_elements:1073741824/manual_time",
+        "CUBLAS_WMMA_GEMM/M:8192/N:8192/K:8192/manual_time",
     ]:
         assert n in have, n
     # the filter is a regular expression over those names
@@ -51,7 +62,9 @@ def test_harness_runs_verifies_and_reports(tmp_path):
     filt = ("(CUDA_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16<1, 4>|256<1, 4>|16N<4>|256N<4>|256N_BLOCK<4>)|CUB_(WARP|BLOCK)_SEGMENTED_(REDUCTION|PREFIXSUM)<(256, 16|512, 32, BLOCK_(SCAN|REDUCE)_RAKING)>"
             "|TCU_AUTO_SEGMENTED_(REDUCTION|PREFIXSUM))/.*num_elements:4194304/"
             "|CUDA_WMMA_FULL_(REDUCTION_(2KERS_BASE_16|ATOMIC_W_BLOCK_SYNC)|PREFIXSUM_(3KERS|CG))<8 \\* 256, 4>/num_elements:4194304/"
-            "|CUDA_WMMA_GEM[MV](_NAIVE)?/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/")
+            "|CUDA_WMMA_GEM[MV](_NAIVE)?/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/"
+            "|CUDA_UNSAFE_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16N<4>|256N_BLOCK<4>)/.*num_elements:4194304/"
+            "|CUB_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/|CUB_DEVICE_SEGMENTED_REDUCTION/.*segment_size:256/num_elements:4194304/|CUBLAS_(WMMA_GEMM|GEMV)/M:512/")
     p = subprocess.run([BENCH, f"--benchmark_filter={filt}", "--benchmark_min_time=0.02", f"--benchmark_out={out}", "--benchmark_out_format=json", "--tcu_verify=all", "--v=1"],
                        capture_output=True, text=True, timeout=300)
     assert p.returncode == 0, p.stdout + p.stderr

@@ -164,3 +164,31 @@ def test_gemv_gemm_f64_against_numpy(oracle):
     want = as_f(Ai, np.int64).reshape(M, K) @ as_f(Bi, np.int64).reshape(N, K).T
     assert np.array_equal(oracle.gemm_f64(Ai, Bi, M, N, K), want.astype(np.float64))
     # a transposed B operand would fail this: B is not symmetric in shape (N != K)
+
+
+def test_offsets_reduction_against_numpy_and_the_fixed_size_oracle(oracle):
+    """Segments given by begin/end offsets: numpy slices summed in float64 / sequentially in float32,
+    the fixed-size functions on uniform offsets, empty and inverted segments, overlapping segments."""
+    rng = np.random.default_rng(3)
+    n = 20000
+    x = oracle.generate_f16(n, 4, oracle.DIST_UNIFORM)
+    xf = x.view(np.float16)
+    begin = rng.integers(0, n, 400)
+    end = np.minimum(begin + rng.integers(0, 700, 400), n)
+    end[::17] = begin[::17] - 1  # inverted = empty
+    got64 = oracle.seg_reduce_offsets_f64(x, begin, end)
+    got16 = oracle.seg_reduce_offsets_ref(x, begin, end)
+    for j in range(400):
+        sl = xf[begin[j]:max(end[j], begin[j])]
+        assert abs(got64[j] - math.fsum(float(v) for v in sl)) <= 1e-9
+        acc = np.float32(0)
+        for v in sl:
+            acc = np.float32(acc + np.float32(v))
+        assert got16[j] == np.float16(acc).view(np.uint16)
+    seg, nseg = 125, 160
+    b = np.arange(nseg) * seg
+    assert np.array_equal(oracle.seg_reduce_offsets_f64(x, b, b + seg), oracle.seg_reduce_f64(x, nseg, seg))
+    assert np.array_equal(oracle.seg_reduce_offsets_ref(x, b, b + seg), oracle.seg_reduce_ref(x, nseg, seg))
+    # overlapping segments are independent: [0, 100) and [50, 150) share elements
+    o = oracle.seg_reduce_offsets_f64(x, np.array([0, 50, 0]), np.array([100, 150, 150]))
+    assert abs(o[2] - (o[0] + o[1] - oracle.seg_reduce_offsets_f64(x, np.array([50]), np.array([100]))[0])) <= 1e-9
