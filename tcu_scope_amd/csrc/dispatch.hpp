@@ -141,7 +141,7 @@ inline Plan auto_plan_scan(size_t S) {
   if (S == 2048) return {true, 4, 2};
   if (S == 4096) return {true, 1, 2};
   if (S == 8192) return {true, 4, 8};
-  if (S == 16384) return {true, 2, 16};
+  if (S == 16384) return {true, 8, 4};
   if (S == 32768) return {true, 8, 8};
   return {true, 8, 16};
 }
