@@ -89,8 +89,8 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
  *   "scan_lds_tiles"  0/1, default 1: full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves)
  *   "gemm_big_tiles"  0/1, default 1: 256 x 256 block tiles where M and N allow
- *   "gemm_direct_lds" -1/0/3/4, default -1: 3 or 4 = global -> LDS transfers with that many LDS buffers,
- *                     0 = register-staged kernel, -1 = chosen by K
+ *   "gemm_direct_lds" -1/0/3/4/64, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
+ *                     buffers; 64 = K step 64, two buffers; 0 = register-staged kernel; -1 = chosen by shape
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
  * Unknown names return TCU_ERR_INVALID_ARG. */

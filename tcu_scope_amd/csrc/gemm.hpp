@@ -298,27 +298,32 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
     for (int j = 0; j < 4; j++) gemm_store_tile(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 32, tile_n * kGemmBigBN + wn * 128 + j * 32, acc[i][j], lane, alpha, beta);
 }
 
-// M % 256 == 0, N % 256 == 0, K % 32 == 0, K <= 2^22 (lane offsets are 32-bit); 256 threads.  Same tiling as gemm_lds256_kernel
-// (256 x 256 x 32 block tile, 2 x 2 waves of 128 x 128), but the operands travel from global
-// memory straight into LDS (load_chunk_to_lds), NBUF K steps deep: no staging registers, no
-// LDS store instructions, and the prefetch distance is NBUF - 1 steps.
-// LDS rows are dense (32 halves = 64 bytes = 4 chunks).  A transfer instruction fills 1 KiB =
-// 16 rows in lane order, so the swizzle that keeps the fragment reads free of bank conflicts
-// is applied on the global side: LDS slot c of row r holds the row's chunk c ^ ((r >> 2) & 3);
-// the 16 rows that 16 lanes read for one k chunk then fall into 16 different groups of four
-// banks.
-// Step s (buffer s % NBUF): substep 0 reads the fragments of substep 1 and issues the
-// transfers of step s + NBUF - 1 into the buffer of step s - 1 (free since that step's
-// barrier); before substep 1 a wave waits for its own transfers of step s + 1, the barrier
+// M % 256 == 0, N % 256 == 0, K % BK == 0, K <= 2^22 (lane offsets are 32-bit); 256 threads.
+// Same tiling as gemm_lds256_kernel (256 x 256 x BK block tile, 2 x 2 waves of 128 x 128), but
+// the operands travel from global memory straight into LDS (load_chunk_to_lds), NBUF K steps
+// deep: no staging registers, no LDS store instructions, prefetch distance NBUF - 1 steps.
+// LDS rows are dense (BK halves = CPR chunks of 16 bytes).  A transfer instruction fills
+// 1 KiB = 64 / CPR rows in lane order, so the swizzle that keeps the fragment reads free of
+// bank conflicts is applied on the global side: LDS slot c of row r holds the row's chunk
+// c ^ f(r), f(r) = (r / rows per 256 bytes) % CPR; the 16 rows that 16 lanes read for one k
+// chunk then fall into 16 different groups of four banks.
+// Step s (buffer s % NBUF): in every substep but the last, the fragments of the next substep
+// are read under the first 8 MFMAs and up to 8 transfers of step s + NBUF - 1 (into the
+// buffer of step s - 1, free since that step's barrier) are issued under the other 8;
+// before the last substep a wave waits for its own transfers of step s + 1, the barrier
 // publishes everybody's, and the fragments of step s + 1, substep 0, are read while the
 // last 16 MFMAs of step s run.
-template <int NBUF>
+template <int BK, int NBUF>
 __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha, float beta) {
-  constexpr int BK = 32, ROWH = BK;                  // halves per LDS row
+  constexpr int ROWH = BK;                           // halves per LDS row
+  constexpr int CPR = BK / 8;                        // chunks per row
+  constexpr int RPT = 64 / CPR;                      // rows per transfer instruction
+  constexpr int RS = CPR == 4 ? 2 : 1;               // f(r) = (r >> RS) & (CPR - 1)
+  constexpr int SUB = BK / 16;                       // 16-wide k substeps per step
   constexpr int OPH = kGemmBigBM * ROWH;             // halves per operand per stage
   constexpr int P = NBUF - 1;                        // prefetch distance in steps
-  constexpr int TPW = kGemmBigBM / 16 / 4;           // transfer instructions per wave, operand and step (4)
-  static_assert(TPW == 4 && 2 * TPW * (P - 1) <= 63, "outstanding transfers must fit the counter");
+  constexpr int TPW = kGemmBigBM / RPT / 4;          // transfer instructions per wave, operand and step
+  static_assert((BK == 32 || BK == 64) && 2 * TPW <= 8 * (SUB - 1) && 2 * TPW * (P - 1) <= 63, "transfers must fit the substeps and the counter");
   __shared__ __attribute__((aligned(1024))) half_t lds_a[NBUF][OPH];
   __shared__ __attribute__((aligned(1024))) half_t lds_b[NBUF][OPH];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -327,26 +332,29 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
   gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
   const size_t steps = K / BK;
-  // transfer t of this wave (t = 0 .. TPW-1) fills rows 16 * (wave * TPW + t) .. + 15; the lane
-  // supplies row +lane/4, LDS slot lane%4, i.e. global chunk (lane%4) ^ ((lane/16) & 3)
+  // transfer t of this wave (t = 0 .. TPW-1) fills rows RPT * (wave * TPW + t) .. + RPT-1; the
+  // lane supplies row +lane/CPR, LDS slot lane%CPR, i.e. global chunk (lane%CPR) ^ f(row)
   // (the same lane offsets serve A and B: both have K columns).  Global addresses are a scalar
   // base per operand and step plus one of TPW 32-bit lane offsets.
-  const int trow = wave * TPW * 16 + (lane >> 2), tchunk = (lane & 3) ^ ((lane >> 4) & 3);
   uint32_t goff[TPW];
 #pragma unroll
-  for (int t = 0; t < TPW; t++) goff[t] = (uint32_t)((((size_t)trow + 16 * t) * k_chunks + tchunk) * 16);
+  for (int t = 0; t < TPW; t++) {
+    const int row = (wave * TPW + t) * RPT + lane / CPR;
+    const int chunk = (lane % CPR) ^ ((row >> RS) & (CPR - 1));
+    goff[t] = (uint32_t)(((size_t)row * k_chunks + chunk) * 16);
+  }
   const char *ga = reinterpret_cast<const char *>(A + tile_m * kGemmBigBM * k_chunks);
   const char *gb = reinterpret_cast<const char *>(B + tile_n * kGemmBigBN * k_chunks);
-  constexpr lds_addr_t STAGE = OPH * 2, TBYTES = 16 * ROWH * 2;  // bytes per stage and operand, per transfer
+  constexpr lds_addr_t STAGE = OPH * 2, TBYTES = 1024, STEPB = BK * 2;  // bytes per stage and operand, per transfer, per step and row
   const lds_addr_t ta = wave_uniform(lds_address_of(&lds_a[0][0]) + wave * TPW * TBYTES);
   const lds_addr_t tb = wave_uniform(lds_address_of(&lds_b[0][0]) + wave * TPW * TBYTES);
-  auto issue_step = [&](size_t step, int buf) {
+  // transfer x (0 .. 2*TPW-1) of a step: operand x % 2, rows of transfer x / 2
+  auto issue = [&](size_t step, int buf, int x) {
     const size_t st = step < steps ? step : steps - 1;  // past the end: a harmless re-read into a free buffer
-#pragma unroll
-    for (int t = 0; t < TPW; t++) {
-      load_chunk_to_lds(ga + st * 64, goff[t], ta + buf * STAGE + t * TBYTES);
-      load_chunk_to_lds(gb + st * 64, goff[t], tb + buf * STAGE + t * TBYTES);
-    }
+    if (x % 2 == 0)
+      load_chunk_to_lds(ga + st * STEPB, goff[x / 2], ta + buf * STAGE + (x / 2) * TBYTES);
+    else
+      load_chunk_to_lds(gb + st * STEPB, goff[x / 2], tb + buf * STAGE + (x / 2) * TBYTES);
   };
 
   float16_t acc[4][4];
@@ -358,14 +366,18 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
 #pragma unroll
-  for (int d = 0; d < P; d++) issue_step((size_t)d, d);
+  for (int d = 0; d < P; d++)
+#pragma unroll
+    for (int x = 0; x < 2 * TPW; x++) issue((size_t)d, d, x);
   wait_vector_loads<2 * TPW * (P - 1)>();
   block_barrier_lds_only();
 
-  // fragment of row r, k chunk kc: slot kc ^ ((r >> 2) & 3); rows of a lane differ by multiples of 32
-  const int frow = lane & 31, khalf = lane >> 5, fsw = (frow >> 2) & 3;
+  // fragment of row r, k chunk kc: slot kc ^ f(r); rows of a lane differ by multiples of 32
+  const int frow = lane & 31, khalf = lane >> 5, fsw = (frow >> RS) & (CPR - 1);
   const int fa0 = (wm * 128 + frow) * ROWH, fb0 = (wn * 128 + frow) * ROWH;
-  const int ko[2] = {((0 + khalf) ^ fsw) * 8, ((2 + khalf) ^ fsw) * 8};
+  int ko[SUB];
+#pragma unroll
+  for (int kk = 0; kk < SUB; kk++) ko[kk] = ((2 * kk + khalf) ^ fsw) * 8;
   half8_t fa[2][4], fb[2][4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
@@ -376,58 +388,58 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
   for (size_t s = 0; s < steps; s++) {
     const int nxt = cur + 1 == NBUF ? 0 : cur + 1;
     const int fill = cur == 0 ? NBUF - 1 : cur - 1;  // buffer of step s - 1 = buffer of step s + P
-    // ---- substep 0
-    sched_fence();
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      fa[1][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][fa0 + i * 32 * ROWH + ko[1]]);
-      fb[1][i] = *reinterpret_cast<const half8_t *>(&lds_b[cur][fb0 + i * 32 * ROWH + ko[1]]);
-    }
-    // first half of the MFMAs with the fragment reads, second half with one transfer each
-    // (the transfers are opaque to the scheduler, so fences pin them in place)
+    for (int kk = 0; kk < SUB; kk++) {
+      const int p = kk & 1, q = p ^ 1;
+      if (kk < SUB - 1) {
+        sched_fence();
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+        for (int i = 0; i < 4; i++) {
+          fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][fa0 + i * 32 * ROWH + ko[kk + 1]]);
+          fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[cur][fb0 + i * 32 * ROWH + ko[kk + 1]]);
+        }
+        // first half of the MFMAs with the fragment reads, second half with one transfer each
+        // (the transfers are opaque to the scheduler, so fences pin them in place)
 #pragma unroll
-      for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[0][i], fb[0][j], acc[i][j]);
+        for (int i = 0; i < 2; i++)
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
-      sched_group<kSchedDsRead, 1>();
-      sched_group<kSchedMfma, 1>();
-    }
-    sched_fence();
-    {
-      const size_t st = s + P < steps ? s + P : steps - 1;  // past the end: a harmless re-read into a free buffer
+          for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
 #pragma unroll
-      for (int t = 0; t < 8; t++) {
-        const int i = 2 + t / 4, j = t % 4;
-        if (t % 2 == 0)
-          load_chunk_to_lds(ga + st * 64, goff[t / 2], ta + fill * STAGE + (t / 2) * TBYTES);
-        else
-          load_chunk_to_lds(gb + st * 64, goff[t / 2], tb + fill * STAGE + (t / 2) * TBYTES);
-        acc[i][j] = mfma_32x32x16(fa[0][i], fb[0][j], acc[i][j]);
+        for (int t = 0; t < 8; t++) {
+          sched_group<kSchedDsRead, 1>();
+          sched_group<kSchedMfma, 1>();
+        }
+        sched_fence();
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const int i = 2 + t / 4, j = t % 4, x = kk * 8 + t;
+          if (x < 2 * TPW) issue(s + P, fill, x);
+          acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+          sched_fence();
+        }
+      } else {
+        // own transfers of step s + 1 done, barrier, fragments of step s + 1
+        wait_vector_loads<2 * TPW * (P - 1)>();
+        block_barrier_lds_only();
+        sched_fence();
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[nxt][fa0 + i * 32 * ROWH + ko[0]]);
+          fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[nxt][fb0 + i * 32 * ROWH + ko[0]]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          sched_group<kSchedDsRead, 1>();
+          sched_group<kSchedMfma, 1>();
+        }
+        sched_group<kSchedMfma, 8>();
         sched_fence();
       }
     }
-    // ---- substep 1: own transfers of step s + 1 done, barrier, fragments of step s + 1
-    wait_vector_loads<2 * TPW * (P - 1)>();
-    block_barrier_lds_only();
-    sched_fence();
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[nxt][fa0 + i * 32 * ROWH + ko[0]]);
-      fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[nxt][fb0 + i * 32 * ROWH + ko[0]]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[1][i], fb[1][j], acc[i][j]);
-#pragma unroll
-    for (int t = 0; t < 8; t++) {
-      sched_group<kSchedDsRead, 1>();
-      sched_group<kSchedMfma, 1>();
-    }
-    sched_group<kSchedMfma, 8>();
-    sched_fence();
     cur = nxt;
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
