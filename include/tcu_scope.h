@@ -88,6 +88,8 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *   "nontemporal"     0/1, default 1: non-temporal loads and stores in the streaming kernels
  *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
  *   "scan_lds_tiles"  0/1, default 1: full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves)
+ *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step
+ *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more)
  *   "gemm_big_tiles"  0/1, default 1: 256 x 256 block tiles where M and N allow
  *   "gemm_direct_lds" -1/0/3/4/64, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
  *                     buffers; 64 = K step 64, two buffers; 0 = register-staged kernel; -1 = chosen by shape

@@ -38,6 +38,7 @@ struct Options {
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
+  int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
 };
 inline Options &options() {
@@ -53,6 +54,9 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemm_big_tiles") o.gemm_big_tiles = value != 0;
   else if (n == "gemm_direct_lds") o.gemm_direct_lds = value;
   else if (n == "gemm_depth") o.gemm_depth = value;
+  else if (n == "gemv_rows") o.gemv_rows = value;
+  else if (n == "gemv_tiles") o.gemv_tiles = value;
+  else if (n == "gemv_waves") o.gemv_waves = value;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
   else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
@@ -664,16 +668,28 @@ inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t
     return TCU_OK;
   }
   const size_t k_tiles = (K / 8 + 63) / 64;
-  if (k_tiles >= 8) {  // rows of 8 KiB and more: block per pair of rows
-    constexpr int BROWS = 2, BU = 4;
-    const unsigned bw = k_tiles >= 32 ? 8u : k_tiles >= 16 ? 4u : 2u;
-    const size_t bgrid = (M + BROWS - 1) / BROWS;
+  if (k_tiles >= 8) {  // rows of 8 KiB and more: a block per group of rows
+    // measured at 16384^2 (48 shapes, randomised order): 2 rows x 2 tiles x 16 waves 81.5 us, 2 x 1 x 16 81.6,
+    // 2 x 1 x 8 81.7 ... 2 x 4 x 8 89.7, 4 rows 84.7+, 1 row 88+: as many waves as the row has tiles
+    const int rows = options().gemv_rows ? options().gemv_rows : 2, bu = options().gemv_tiles ? options().gemv_tiles : (k_tiles >= 32 ? 2 : 1);
+    const size_t fit = k_tiles / (size_t)bu;
+    const unsigned bw = options().gemv_waves ? (unsigned)options().gemv_waves : (fit >= 16 ? 16u : fit >= 8 ? 8u : 4u);
+    const size_t bgrid = (M + rows - 1) / rows;
     if (bgrid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    if (nt)
-      launch(gemv_block_kernel<BROWS, BU, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
-    else
-      launch(gemv_block_kernel<BROWS, BU, false>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
-    return TCU_OK;
+#define TCU_GEMV_BLOCK(R_, U_)                                                                                              \
+  if (rows == R_ && bu == U_) {                                                                                            \
+    if (nt)                                                                                                                \
+      launch(gemv_block_kernel<R_, U_, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);         \
+    else                                                                                                                   \
+      launch(gemv_block_kernel<R_, U_, false>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);        \
+    return TCU_OK;                                                                                                         \
+  }
+    TCU_GEMV_BLOCK(1, 1) TCU_GEMV_BLOCK(1, 2) TCU_GEMV_BLOCK(1, 4) TCU_GEMV_BLOCK(1, 8)
+    TCU_GEMV_BLOCK(2, 1) TCU_GEMV_BLOCK(2, 2) TCU_GEMV_BLOCK(2, 4)
+    TCU_GEMV_BLOCK(4, 1) TCU_GEMV_BLOCK(4, 2) TCU_GEMV_BLOCK(4, 4)
+    TCU_GEMV_BLOCK(8, 1) TCU_GEMV_BLOCK(8, 2)
+#undef TCU_GEMV_BLOCK
+    return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unsupported gemv_rows / gemv_tiles option");
   }
   constexpr int ROWS = 2, UK = 4;
   const size_t waves = (M + ROWS - 1) / ROWS;
