@@ -225,7 +225,7 @@ inline int seg_reduce_huge(const half8_t *in, uint16_t *out, size_t num_segments
     launch(partition_sums_kernel<8, true>, (unsigned)parts, 1024u, stream, in, partials, n_chunks);
   else
     launch(partition_sums_kernel<8, false>, (unsigned)parts, 1024u, stream, in, partials, n_chunks);
-  launch(segment_of_partials_kernel, (unsigned)num_segments, 256u, stream, static_cast<const float *>(partials), out, pps);
+  launch(segment_of_partials_kernel, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(partials), out, pps);
   stream_free(partials, stream);
   return TCU_OK;
 }
@@ -329,7 +329,7 @@ inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t nu
       launch(seg_reduce_offsets_sliced_kernel<OFF, true>, (unsigned)blocks, 1024u, stream, in, partials, begin, end, (unsigned)slices, vector);
     else
       launch(seg_reduce_offsets_sliced_kernel<OFF, false>, (unsigned)blocks, 1024u, stream, in, partials, begin, end, (unsigned)slices, vector);
-    launch(segment_of_partials_kernel, (unsigned)num_segments, 256u, stream, static_cast<const float *>(partials), out, slices);
+    launch(segment_of_partials_kernel, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(partials), out, slices);
     stream_free(partials, stream);
     return TCU_OK;
   }
@@ -548,7 +548,7 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
         launch(partition_sums_kernel<8, true>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks);
       else
         launch(partition_sums_kernel<8, false>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks);
-      launch(segment_of_partials_kernel, 1u, 256u, stream, static_cast<const float *>(partials), static_cast<uint16_t *>(d_out), grid);
+      launch(segment_of_partials_kernel, 1u, 1024u, stream, static_cast<const float *>(partials), static_cast<uint16_t *>(d_out), grid);
       return TCU_OK;
     }
     unsigned *ws = static_cast<unsigned *>(d_ws);

@@ -340,18 +340,30 @@ __global__ __launch_bounds__(kMaxBlock) void partition_sums_kernel(const half8_t
     partial_out[blockIdx.x] = s;
   }
 }
-// second level: block j adds the parts_per_segment partials of segment j (fixed order: lane
-// strides, then lanes, then waves) and writes the fp16 result
-__global__ __launch_bounds__(256) void segment_of_partials_kernel(const float *__restrict__ partial_in, uint16_t *__restrict__ out, size_t parts_per_segment) {
-  __shared__ float partial[4];
+// second level: block j (1024 threads) adds the parts_per_segment partials of segment j in a
+// fixed order (four independent strided streams per thread, then lanes, then waves) and writes
+// the fp16 result
+__global__ __launch_bounds__(1024) void segment_of_partials_kernel(const float *__restrict__ partial_in, uint16_t *__restrict__ out, size_t parts_per_segment) {
+  __shared__ float partial[16];
   const int lane = lane_id(), wave = wave_in_block();
   const float *p = partial_in + (size_t)blockIdx.x * parts_per_segment;
-  float acc = 0.0f;
-  for (size_t i = threadIdx.x; i < parts_per_segment; i += 256) acc += p[i];
-  acc = lane_group_sum<6>(acc);
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  size_t i = threadIdx.x;
+  for (; i + 3 * 1024 < parts_per_segment; i += 4 * 1024) {
+    a0 += p[i];
+    a1 += p[i + 1024];
+    a2 += p[i + 2048];
+    a3 += p[i + 3072];
+  }
+  for (; i < parts_per_segment; i += 1024) a0 += p[i];
+  const float acc = lane_group_sum<6>((a0 + a1) + (a2 + a3));
   if (lane == 63) partial[wave] = acc;
   __syncthreads();
-  if (threadIdx.x == 0) out[blockIdx.x] = f16_bits((partial[0] + partial[1]) + (partial[2] + partial[3]));
+  if (threadIdx.x == 0) {
+    float s = 0.0f;
+    for (int w = 0; w < 16; w++) s += partial[w];
+    out[blockIdx.x] = f16_bits(s);
+  }
 }
 
 // out[0] = fp16(sum of n halves), one block
