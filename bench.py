@@ -31,8 +31,8 @@ SCAN_SEGS = [16, 256, 2048, 16384]
 # WRITE_SIZE runs of this script, each counter scaled by what it reads for the plain copy
 # kernel of known size (profiles/seg_reduce_scan_2p28_hbm_traffic.md).
 MEASURED_TRAFFIC_2P28_AUTO = {
-    ("reduce", 16): 570418104, ("reduce", 256): 538967188, ("reduce", 1024): 537931321, ("reduce", 4096): 537926153, ("reduce", 16384): 537138026,
-    ("scan", 16): 1073751645, ("scan", 256): 1073705869, ("scan", 2048): 1073579459, ("scan", 16384): 1073566659,
+    ("reduce", 16): 570417963, ("reduce", 256): 538966187, ("reduce", 1024): 537931269, ("reduce", 4096): 537925093, ("reduce", 16384): 537136897,
+    ("scan", 16): 1073728548, ("scan", 256): 1073787570, ("scan", 2048): 1073609230, ("scan", 16384): 1073637069,
 }
 
 
