@@ -5,8 +5,8 @@ N = 2^28 elements, segment sizes 16..16384, on one MI355X.
 A step is one pass over the whole sweep: 5 segmented reductions (seg 16, 256, 1024, 4096,
 16384) and 4 segmented scans (seg 16, 256, 2048, 16384), each over 2^28 synthetic
 elements already resident in HBM.  `value` = elements processed per second over the
-timed steps (wall clock, synchronised on both sides).  Every launch is also bracketed by
-HIP events on the launch stream; from those come the per-kernel bandwidths and the
+timed steps (wall clock, synchronised on both sides).  Every launch also sits between two
+HIP events on the launch stream (one event per launch boundary); from those come the per-kernel bandwidths and the
 `roofline` object (algorithmic bytes / average launch time / 8 TB/s).
 Two input buffers alternate between launches so that no launch finds its input in the
 256 MB Infinity Cache.
@@ -124,15 +124,15 @@ def main():
             counter += 1
     torch.cuda.synchronize()
 
-    events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in configs] for _ in range(args.steps)]
+    # one event per launch boundary: event c precedes launch c and closes launch c - 1
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(len(configs) + 1)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
+        events[k][0].record(stream)
         for c, (kind, seg) in enumerate(configs):
-            a, b = events[k][c]
-            a.record(stream)
             launch(counter, kind, seg)
-            b.record(stream)
+            events[k][c + 1].record(stream)
             counter += 1
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -144,7 +144,7 @@ def main():
     measured_shapes = args.n_log2 == 28 and variant == tcu.Variant.AUTO and args.tiles_per_wave == 0 and args.waves_per_block == 0
     per_config = []
     for c, (kind, seg) in enumerate(configs):
-        ms = sorted(events[k][c][0].elapsed_time(events[k][c][1]) for k in range(args.steps))
+        ms = sorted(events[k][c].elapsed_time(events[k][c + 1]) for k in range(args.steps))
         avg = sum(ms) / len(ms)
         by = algorithmic_bytes(kind, n, seg)
         per_config.append({
