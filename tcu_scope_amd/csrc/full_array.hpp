@@ -1,19 +1,23 @@
 // Full-array (unsegmented) sum and inclusive prefix sum over fp16, fp32 carries.
 //
 // Single-pass kernels:
-//   full_reduce_kernel : persistent blocks stride over the array; every block leaves one
-//     fp32 partial in the workspace and takes an atomic ticket; the block that draws the
-//     last ticket adds the partials in index order (deterministic) and writes the fp16
-//     result.  Replaces the reference's atomic / cooperative-groups full reductions
-//     (src/reduction/kernel.cuh:564-786), whose combine step is an atomicAdd on one
-//     half (or a serial loop in global thread 0).
-//   full_scan_kernel   : decoupled look-back.  Partitions are handed out by an atomic
-//     ticket (so a partition's predecessors are always running or done); each block
-//     publishes {flag, fp32 aggregate} as one 64-bit word, wave 0 looks back 64
-//     descriptors at a time, then the block scans its tiles from registers.  Replaces
-//     the reference's grid-sync / spin-barrier full scans (src/prefixsum/kernel.cuh:779-972;
-//     both disabled upstream: the first needs more shared memory than exists, the second
-//     deadlocks) and its 3-kernel sequence, which moves 8+ bytes per element.
+//   full_reduce_kernel : one partition per block; every block publishes {1, fp32 partial} as
+//     one 64-bit word and takes a ticket from its group's counter; the last block of a group
+//     adds the group's words, the last group adds the group sums (index order, so the result
+//     does not depend on timing) and writes the fp16 result.  Replaces the reference's
+//     atomic / cooperative-groups full reductions (src/reduction/kernel.cuh:564-786), whose
+//     combine step is an atomicAdd on one half (or a serial loop in global thread 0).
+//   full_scan_kernel, full_scan_lds_kernel : decoupled look-back.  Partitions are handed out
+//     by an atomic ticket (so a partition's predecessors are always running or done); each
+//     block publishes {flag, fp32 aggregate} as one 64-bit word, wave 0 looks back 64
+//     descriptors at a time, then the block scans its tiles from registers (and, in the
+//     second kernel, from LDS).  Replaces the reference's grid-sync / spin-barrier full scans
+//     (src/prefixsum/kernel.cuh:779-972; both disabled upstream: the first needs more shared
+//     memory than exists, the second deadlocks) and its 3-kernel sequence, which moves 8+
+//     bytes per element.
+// Two-launch reduction (the fastest; also what segments of 2^20 halves and more take):
+//   partition_sums_kernel writes one fp32 partial per partition, segment_of_partials_kernel
+//   adds the partials of every segment.
 // Multi-kernel helpers (the reference's "2 kernels" / "3 kernels" sequences):
 //   sum_f16_kernel, exclusive_scan_f16_kernel over the per-segment totals.
 #pragma once

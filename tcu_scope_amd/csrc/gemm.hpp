@@ -10,6 +10,10 @@
 //                        two LDS buffers (one barrier per step).  Counterpart of the
 //                        reference's shared-memory kernels (src/gemm/wmma.cu:171-365,
 //                        wmma_sharedmem.cu:43-123).
+//   gemm_lds256_kernel, gemm_dlds_kernel : 256 x 256 block tile, 4 waves of 128 x 128 (all 256
+//                        accumulation registers), hand-pipelined; operands staged through
+//                        registers or moved global -> LDS directly (described at the kernels).
+//                        These run whenever M and N are multiples of 256.
 //   gemm_direct_kernel : one 32 x 32 tile per wave, fragments loaded straight from global
 //                        memory (reference compute_gemm_naive, src/gemm/wmma_naive.cu:33-88).
 //   gemm_generic_kernel: any M, N, K; one thread per output element.
