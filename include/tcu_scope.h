@@ -129,6 +129,14 @@ int tcu_seg_reduce_offsets_f16(const void *d_in, void *d_out, size_t num_segment
  * seg_cub_block.cu:13-51).  In-place (d_out == d_in) is allowed. */
 int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
 
+/* Segments given by offsets (conventions of tcu_seg_reduce_offsets_f16; segments must not
+ * overlap): d_out[i] = fp16( d_in[begin[j]] + ... + d_in[i] ) for i in [begin[j], end[j]);
+ * elements of d_out outside every segment are not written.  In-place is allowed.
+ * Hand-written counterpart of the reference's key-based library scan
+ * (thrust::inclusive_scan_by_key, src/prefixsum/seg_thrust.cu:46-47) for segments
+ * described by an offsets array (src/reduction/seg_cub_device.cu:18-22). */
+int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments, const void *d_begin_offsets, const void *d_end_offsets, int offset_bits, size_t expected_segment_size, void *stream);
+
 /* d_out[s*S + i] += d_partial_sums[s]  (one fp16 addition per element).
  * Replaces add_partial_sums (reference src/prefixsum/kernel.cuh:31-43). */
 int tcu_add_partial_sums_f16(void *d_out, const void *d_partial_sums, size_t num_segments, size_t segment_size, void *stream);

@@ -57,6 +57,8 @@ def lib():
         i64p = c.POINTER(c.c_int64)
         L.tcu_oracle_seg_reduce_offsets_ref.argtypes = [u16p, u16p, sz, i64p, i64p]
         L.tcu_oracle_seg_reduce_offsets_f64.argtypes = [u16p, f64p, sz, i64p, i64p]
+        L.tcu_oracle_seg_scan_offsets_ref.argtypes = [u16p, u16p, sz, i64p, i64p]
+        L.tcu_oracle_seg_scan_offsets_f64.argtypes = [u16p, f64p, sz, i64p, i64p]
         L.tcu_oracle_seg_scan_f64.argtypes = [u16p, f64p, sz, sz]
         L.tcu_oracle_gemv_f64.argtypes = [u16p, u16p, f32p, f64p, sz, sz, c.c_double, c.c_double]
         L.tcu_oracle_gemm_f64.argtypes = [u16p, u16p, f32p, f64p, sz, sz, sz, c.c_double, c.c_double, sz, sz]
@@ -210,6 +212,24 @@ def seg_reduce_offsets_f64(x, begin, end):
     begin, end = _offsets(x, begin, end)
     out = np.empty(begin.size, dtype=np.float64)
     lib().tcu_oracle_seg_reduce_offsets_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), begin.size, _p(begin, ctypes.c_int64), _p(end, ctypes.c_int64))
+    return out
+
+
+def seg_scan_offsets_ref(x, begin, end, fill=0xFFFF):
+    """fp32 running sums inside x[begin[j]:end[j]], fp16 bits; positions outside every segment hold `fill`."""
+    x = _u16(x)
+    begin, end = _offsets(x, begin, end)
+    out = np.full(x.size, fill, dtype=np.uint16)
+    lib().tcu_oracle_seg_scan_offsets_ref(_p(x, ctypes.c_uint16), _p(out, ctypes.c_uint16), begin.size, _p(begin, ctypes.c_int64), _p(end, ctypes.c_int64))
+    return out
+
+
+def seg_scan_offsets_f64(x, begin, end):
+    """fp64 running sums inside every segment; NaN outside every segment."""
+    x = _u16(x)
+    begin, end = _offsets(x, begin, end)
+    out = np.full(x.size, np.nan, dtype=np.float64)
+    lib().tcu_oracle_seg_scan_offsets_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), begin.size, _p(begin, ctypes.c_int64), _p(end, ctypes.c_int64))
     return out
 
 

@@ -279,6 +279,26 @@ void tcu_oracle_seg_reduce_offsets_ref(const uint16_t *in, uint16_t *out, size_t
   }
 }
 
+void tcu_oracle_seg_scan_offsets_ref(const uint16_t *in, uint16_t *out, size_t num_segments, const int64_t *begin, const int64_t *end) {
+  for (size_t j = 0; j < num_segments; j++) {
+    float s = 0.0f;
+    for (int64_t i = begin[j]; i < end[j]; i++) {
+      s += tcu_oracle_f16_to_f32(in[i]);
+      out[i] = tcu_oracle_f32_to_f16(s);
+    }
+  }
+}
+
+void tcu_oracle_seg_scan_offsets_f64(const uint16_t *in, double *out, size_t num_segments, const int64_t *begin, const int64_t *end) {
+  for (size_t j = 0; j < num_segments; j++) {
+    double s = 0;
+    for (int64_t i = begin[j]; i < end[j]; i++) {
+      s += (double)tcu_oracle_f16_to_f32(in[i]);
+      out[i] = s;
+    }
+  }
+}
+
 void tcu_oracle_seg_reduce_offsets_f64(const uint16_t *in, double *out, size_t num_segments, const int64_t *begin, const int64_t *end) {
   for (size_t j = 0; j < num_segments; j++) {
     double s = 0;

@@ -90,7 +90,13 @@ void tcu_oracle_add_partial_sums_ref(uint16_t *out, const uint16_t *partial_sums
  * fp32 sequential sum, fp16 result, like the fixed-size loop above. */
 void tcu_oracle_seg_reduce_offsets_ref(const uint16_t *in, uint16_t *out, size_t num_segments, const int64_t *begin, const int64_t *end);
 
+/* Inclusive prefix sums inside every segment of an offsets array: out[i] for i in
+ * [begin[j], end[j]) is the fp32 running sum of in[begin[j] .. i] rounded to fp16; elements
+ * of `out` outside every segment are left as they are.  Offsets convention as above. */
+void tcu_oracle_seg_scan_offsets_ref(const uint16_t *in, uint16_t *out, size_t num_segments, const int64_t *begin, const int64_t *end);
+
 /* ---- definition (fp64) -------------------------------------------------------------- */
+void tcu_oracle_seg_scan_offsets_f64(const uint16_t *in, double *out, size_t num_segments, const int64_t *begin, const int64_t *end);
 void tcu_oracle_seg_reduce_offsets_f64(const uint16_t *in, double *out, size_t num_segments, const int64_t *begin, const int64_t *end);
 void tcu_oracle_seg_reduce_f64(const uint16_t *in, double *out, size_t num_segments, size_t segment_size);
 void tcu_oracle_seg_scan_f64(const uint16_t *in, double *out, size_t num_segments, size_t segment_size);

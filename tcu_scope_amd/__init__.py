@@ -28,6 +28,7 @@ from .binding import (  # noqa: F401
     library_path,
     seg_reduce,
     seg_reduce_offsets,
+    seg_scan_offsets,
     seg_scan,
     set_option,
     stream_probe,

@@ -11,7 +11,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 
 EXPORTS = [
     "tcu_abi_version", "tcu_last_error", "tcu_init", "tcu_device_info", "tcu_set_option",
-    "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_add_partial_sums_f16",
+    "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_offsets_f16", "tcu_add_partial_sums_f16",
     "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32",
     "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_lane_probe",
 ]
@@ -84,6 +84,7 @@ def lib():
         L.tcu_seg_reduce_f16.argtypes = [vp, vp, sz, sz, ci, ci, ci, vp]
         L.tcu_seg_reduce_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz, vp]
         L.tcu_seg_scan_f16.argtypes = [vp, vp, vp, sz, sz, ci, ci, ci, vp]
+        L.tcu_seg_scan_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz, vp]
         L.tcu_add_partial_sums_f16.argtypes = [vp, vp, sz, sz, vp]
         L.tcu_full_reduce_f16.argtypes = [vp, vp, sz, vp, c.POINTER(sz), ci, sz, ci, vp]
         L.tcu_full_scan_f16.argtypes = [vp, vp, sz, vp, c.POINTER(sz), ci, sz, ci, vp]
@@ -179,6 +180,21 @@ def seg_scan(x, segment_size, variant=Variant.AUTO, tiles_per_wave=0, waves_per_
     if out is None:
         out = torch.empty(nseg * max(segment_size, 0), dtype=torch.float16, device=x.device)
     _check(lib().tcu_seg_scan_f16(_ptr(x), _ptr(out), _ptr(totals), nseg, segment_size, int(variant), tiles_per_wave, waves_per_block, _stream(stream)))
+    return out
+
+
+def seg_scan_offsets(x, begin, end, expected_segment_size=0, out=None, stream=None):
+    """Inclusive prefix sums inside every x[begin[j]:end[j]] (non-overlapping); the rest of `out` is not written."""
+    torch = _torch()
+    _need_f16(x, "x")
+    if begin.dtype != end.dtype or begin.dtype not in (torch.int32, torch.int64) or begin.numel() != end.numel():
+        raise ValueError("begin and end must be int32 or int64 tensors of the same length")
+    if not (begin.is_contiguous() and end.is_contiguous()):
+        raise ValueError("begin and end must be contiguous")
+    if out is None:
+        out = torch.zeros_like(x)
+    bits = 32 if begin.dtype == torch.int32 else 64
+    _check(lib().tcu_seg_scan_offsets_f16(_ptr(x), _ptr(out), begin.numel(), _ptr(begin), _ptr(end), bits, expected_segment_size, _stream(stream)))
     return out
 
 

@@ -92,6 +92,11 @@ int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_s
   return after_launch("tcu_seg_scan_f16", before, tcu::seg_scan_dispatch(d_in, d_out, d_totals, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, stream));
 }
 
+int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments, const void *d_begin_offsets, const void *d_end_offsets, int offset_bits, size_t expected_segment_size, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_seg_scan_offsets_f16", before, tcu::seg_scan_offsets_dispatch(d_in, d_out, num_segments, d_begin_offsets, d_end_offsets, offset_bits, expected_segment_size, stream));
+}
+
 int tcu_add_partial_sums_f16(void *d_out, const void *d_partial_sums, size_t num_segments, size_t segment_size, void *stream) {
   const unsigned long before = tcu::launch_count();
   return after_launch("tcu_add_partial_sums_f16", before, tcu::add_partial_sums_dispatch(d_out, d_partial_sums, num_segments, segment_size, stream));

@@ -464,6 +464,51 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   return TCU_OK;
 }
 
+// ----- segmented inclusive prefix sum over an offsets array -----------------------------------
+
+template <typename OFF>
+inline int seg_scan_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_segments, const OFF *begin, const OFF *end, size_t expected, void *stream) {
+  // lanes per segment: about one 128-bit chunk per lane and round for the expected length, at most 16
+  int g_log2 = 4;
+  if (expected) {
+    g_log2 = 1;
+    while (g_log2 < 4 && ((size_t)8 << g_log2) < expected) g_log2++;
+  }
+  const size_t threads = num_segments << g_log2;
+  const size_t grid = (threads + 255) / 256;
+  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_offsets_f16: grid exceeds the launch limit");
+  const int vector = aligned16(in) && aligned16(out) ? 1 : 0;
+  const bool nt = options().nontemporal;
+#define TCU_OFFSETS_CASE(GL)                                                                                                          \
+  case GL:                                                                                                                           \
+    if (nt)                                                                                                                          \
+      launch(seg_scan_offsets_kernel<OFF, GL, true>, (unsigned)grid, 256u, stream, in, out, num_segments, begin, end, vector);        \
+    else                                                                                                                             \
+      launch(seg_scan_offsets_kernel<OFF, GL, false>, (unsigned)grid, 256u, stream, in, out, num_segments, begin, end, vector);       \
+    break
+  switch (g_log2) {
+    TCU_OFFSETS_CASE(1);
+    TCU_OFFSETS_CASE(2);
+    TCU_OFFSETS_CASE(3);
+    default:
+      TCU_OFFSETS_CASE(4);
+  }
+#undef TCU_OFFSETS_CASE
+  return TCU_OK;
+}
+
+inline int seg_scan_offsets_dispatch(const void *d_in, void *d_out, size_t num_segments, const void *d_begin, const void *d_end, int offset_bits, size_t expected, void *stream) {
+  const char *what = "tcu_seg_scan_offsets_f16";
+  if (offset_bits != 32 && offset_bits != 64) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": offset_bits must be 32 or 64");
+  if (num_segments == 0) return TCU_OK;
+  if (!d_in || !d_out || !d_begin || !d_end) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  if (num_segments > ((size_t)1 << 56)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": too many segments");
+  const uint16_t *in = static_cast<const uint16_t *>(d_in);
+  uint16_t *out = static_cast<uint16_t *>(d_out);
+  if (offset_bits == 32) return seg_scan_offsets_typed(in, out, num_segments, static_cast<const int32_t *>(d_begin), static_cast<const int32_t *>(d_end), expected, stream);
+  return seg_scan_offsets_typed(in, out, num_segments, static_cast<const int64_t *>(d_begin), static_cast<const int64_t *>(d_end), expected, stream);
+}
+
 inline int add_partial_sums_dispatch(void *d_out, const void *d_ps, size_t num_segments, size_t segment_size, void *stream) {
   if (segment_size == 0) return fail(TCU_ERR_INVALID_ARG, "tcu_add_partial_sums_f16: segment_size must be positive");
   if (num_segments == 0) return TCU_OK;

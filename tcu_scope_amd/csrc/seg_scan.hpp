@@ -323,4 +323,66 @@ __global__ __launch_bounds__(256) void add_partial_sums_generic_kernel(uint16_t 
   out[i] = f16_bits((float)__builtin_bit_cast(half_t, out[i]) + ps);
 }
 
+// ---------------------------------------------------------------------------------------
+// Segments given by offsets (segment j = [begin[j], end[j]) in halves, any start, any
+// length, empty when end <= begin; segments must not overlap): inclusive prefix sums inside
+// every segment, elements outside every segment are not written.  The counterpart of the
+// reference's key-based library scan (thrust::inclusive_scan_by_key,
+// src/prefixsum/seg_thrust.cu:46-47) for segments described the way its
+// cub::DeviceSegmentedReduce baseline describes them (src/reduction/seg_cub_device.cu:18-22).
+// G = 2^G_LOG2 (2..16) adjacent lanes share a segment and walk it in rounds of G aligned
+// 8-half chunks: a chunk that lies wholly inside the segment is one 128-bit load and one
+// 128-bit store, the ragged first / last chunk goes through 2-byte accesses; chunk totals
+// are scanned across the G lanes with DPP and the round total is carried to the next round.
+// With `vector` false (input or output not 16-byte aligned) every chunk takes the 2-byte path.
+// ---------------------------------------------------------------------------------------
+template <typename OFF, int G_LOG2, bool NT>
+__global__ __launch_bounds__(256) void seg_scan_offsets_kernel(const uint16_t *in, uint16_t *out, size_t num_segments, const OFF *__restrict__ begin, const OFF *__restrict__ end, int vector) {
+  constexpr int G = 1 << G_LOG2;
+  static_assert(G_LOG2 >= 1 && G_LOG2 <= 4, "the round total must reach every lane of the group");
+  const int lane = lane_id();
+  const int sub = lane & (G - 1);
+  const size_t seg = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> G_LOG2;
+  size_t b = 0, e = 0;
+  if (seg < num_segments) {
+    const OFF ob = begin[seg], oe = end[seg];
+    if (oe > ob) {
+      b = (size_t)ob;
+      e = (size_t)oe;
+    }
+  }
+  const size_t c_first = b / 8, c_end = (e + 7) / 8;  // aligned chunks touched by the segment
+  const size_t rounds = (c_end - c_first + G - 1) / G;
+  float carry = 0.0f;
+  const half8_t *in8 = reinterpret_cast<const half8_t *>(in);
+  uint4_t *out8 = reinterpret_cast<uint4_t *>(out);
+  // every lane of the wave runs as many rounds as the longest segment of the wave needs (the
+  // DPP scans involve all lanes)
+  for (size_t r = 0; ballot(r < rounds) != 0ull; r++) {
+    const size_t c = c_first + r * G + sub;
+    const size_t lo = c * 8, hi = lo + 8;
+    const bool any = r < rounds && c < c_end;
+    const bool full = any && vector && lo >= b && hi <= e;
+    half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (full) {
+      v = load_chunk<NT>(in8 + c);
+    } else if (any) {
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        if (lo + i >= b && lo + i < e) v[i] = __builtin_bit_cast(half_t, in[lo + i]);
+    }
+    const float t = sum8(v, 0.0f);
+    const float start = lane_group_exclusive_scan<G_LOG2>(t, lane) + carry;
+    carry += lane_group_sum<G_LOG2>(t);
+    const uint4_t packed = chunk_scan_packed(v, start);
+    if (full) {
+      store_chunk<NT>(out8 + c, packed);
+    } else if (any) {
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        if (lo + i >= b && lo + i < e) out[lo + i] = (uint16_t)(packed[i / 2] >> (16 * (i & 1)));
+    }
+  }
+}
+
 }  // namespace tcu

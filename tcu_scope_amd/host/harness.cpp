@@ -324,6 +324,41 @@ void run_seg_reduce_offsets(benchmark::State &state, bool pass_expected_size, co
   });
 }
 
+void run_seg_scan_offsets(benchmark::State &state, const char *name) {
+  guarded(state, [&] {
+    const size_t num_segments = state.range(0), segment_size = state.range(1);
+    const size_t num_elements = num_segments * segment_size;
+    if (num_elements >= ((size_t)1 << 31)) {
+      state.SkipWithError("offsets are 32-bit integers");
+      return;
+    }
+    const int nin = num_elements <= ((size_t)1 << 29) ? 2 : 1;
+    DeviceBuffer in[2] = {DeviceBuffer(num_elements * 2), DeviceBuffer(nin == 2 ? num_elements * 2 : 16)};
+    DeviceBuffer out(num_elements * 2), offsets((num_segments + 1) * sizeof(int));
+    for (int i = 0; i < nin; i++) fill_input(in[i].get(), num_elements, flags().seed + i);
+    {
+      std::vector<int> h(num_segments + 1);
+      for (size_t j = 0; j <= num_segments; j++) h[j] = (int)(j * segment_size);
+      PRINT_IF_ERROR(hipMemcpy(offsets.get(), h.data(), h.size() * sizeof(int), hipMemcpyHostToDevice));
+    }
+    const int *off = static_cast<const int *>(offsets.get());
+    TCU_CHECK(tcu_seg_scan_offsets_f16(in[0].get(), out.get(), num_segments, off, off + 1, 32, segment_size, nullptr));
+    PRINT_IF_ERROR(hipDeviceSynchronize());
+    if (should_verify(num_elements)) verify_seg_scan(in[0].get(), out.get(), num_segments, segment_size, name);
+    EventPair ev;
+    size_t it = 0;
+    for (auto _ : state) {
+      ev.start();
+      TCU_CHECK(tcu_seg_scan_offsets_f16(in[it++ % nin].get(), out.get(), num_segments, off, off + 1, 32, segment_size, nullptr));
+      const float ms = ev.stop_ms();
+      state.PauseTiming();
+      state.SetIterationTime(ms / 1000);
+      state.ResumeTiming();
+    }
+    set_common_counters(state, num_segments, segment_size, num_elements, 0, 4.0 * num_elements + 4.0 * num_segments);
+  });
+}
+
 void run_seg_scan(benchmark::State &state, int variant, int tiles_per_wave, int waves_per_block, bool with_totals, const char *name) {
   guarded(state, [&] {
     const size_t num_segments = state.range(0), segment_size = state.range(1);

@@ -88,6 +88,7 @@ void run_seg_reduce(benchmark::State &state, int variant, int tiles_per_wave, in
 // segmented reduction through an offsets array (offsets[j] = j * segment_size: the array the
 // reference's CUB_DEVICE_SEGMENTED_REDUCTION harness builds, src/reduction/seg_cub_device.cu:18-22)
 void run_seg_reduce_offsets(benchmark::State &state, bool pass_expected_size, const char *name);
+void run_seg_scan_offsets(benchmark::State &state, const char *name);
 void run_seg_scan(benchmark::State &state, int variant, int tiles_per_wave, int waves_per_block, bool with_totals, const char *name);
 void run_full_reduce(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
 void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);

@@ -115,3 +115,9 @@ BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_16_ARGS()->UseManualTime();
 BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_256_ARGS()->UseManualTime();
 BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_4096_ARGS()->UseManualTime();
 BENCHMARK(TCU_OFFSETS_NOHINT_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
+// inclusive prefix sums inside the segments of the same offsets array
+static void TCU_OFFSETS_SEGMENTED_PREFIXSUM(benchmark::State &state) { harness::run_seg_scan_offsets(state, "TCU_OFFSETS_SEGMENTED_PREFIXSUM"); }
+BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->Apply(Tuning16_x_28)->UseManualTime();
+BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->SEG_16_ARGS()->UseManualTime();
+BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->SEG_256_ARGS()->UseManualTime();
+BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->SEG_2048_ARGS()->UseManualTime();

@@ -10,6 +10,7 @@ int emu_seg_scan_f16(const void *in, void *out, void *totals, size_t nseg, size_
   return tcu::seg_scan_dispatch(in, out, totals, nseg, seg, variant, u, wpb, nullptr);
 }
 int emu_seg_reduce_offsets_f16(const void *in, void *out, size_t nseg, const void *begin, const void *end, int bits, size_t expected) { return tcu::seg_reduce_offsets_dispatch(in, out, nseg, begin, end, bits, expected, nullptr); }
+int emu_seg_scan_offsets_f16(const void *in, void *out, size_t nseg, const void *begin, const void *end, int bits, size_t expected) { return tcu::seg_scan_offsets_dispatch(in, out, nseg, begin, end, bits, expected, nullptr); }
 int emu_add_partial_sums_f16(void *out, const void *ps, size_t nseg, size_t seg) { return tcu::add_partial_sums_dispatch(out, ps, nseg, seg, nullptr); }
 const char *emu_last_error() { return tcu::last_error_string().c_str(); }
 int emu_set_option(const char *name, int value) { return tcu::set_option(name, value); }

@@ -38,6 +38,7 @@ def emu():
     L.emu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
     L.emu_set_option.argtypes = [ctypes.c_char_p, ci]
     L.emu_seg_reduce_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz]
+    L.emu_seg_scan_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz]
     L.emu_generate_f16.argtypes = [vp, sz, ctypes.c_uint64, ci, sz]
     L.emu_last_error.restype = ctypes.c_char_p
     return L
@@ -148,6 +149,48 @@ def test_segmented_reduction_over_offsets(emu, oracle):
     assert emu.emu_seg_reduce_offsets_f16(xi.ctypes.data + 2, out.ctypes.data, 300, bi.ctypes.data, ei.ctypes.data, 64, 64) == 0
     assert np.array_equal(out, want)
     assert emu.emu_seg_reduce_offsets_f16(xi.ctypes.data, out.ctypes.data, 300, bi.ctypes.data, ei.ctypes.data, 16, 0) == 1
+
+
+def disjoint_offsets(rng, n, nseg, empty_every=11):
+    """nseg disjoint ragged segments of [0, n) in increasing order with gaps between them, some empty."""
+    cuts = np.sort(rng.choice(n, 2 * nseg, replace=False))
+    begin, end = cuts[0::2].astype(np.int64), cuts[1::2].astype(np.int64)
+    end[::empty_every] = begin[::empty_every]
+    return begin, end
+
+
+def test_segmented_scan_over_offsets(emu, oracle):
+    rng = np.random.default_rng(12)
+    n = 40000
+    x = oracle.generate_f16(n, 10, oracle.DIST_GRID)  # exact partial sums: results are fixed bit for bit
+    xi = copy_in(x)
+    for nseg, expected, bits in ((1500, 16, 32), (1500, 0, 64), (300, 64, 32), (40, 1000, 64), (7, 0, 32)):
+        begin, end = disjoint_offsets(rng, n, nseg)
+        w64 = oracle.seg_scan_offsets_f64(x, begin, end)
+        inside = ~np.isnan(w64)
+        want = np.full(n, 0xFFFF, np.uint16)
+        want[inside] = w64[inside].astype(np.float16).view(np.uint16)
+        assert np.array_equal(want, oracle.seg_scan_offsets_ref(x, begin, end, fill=0xFFFF))
+        dt = np.int32 if bits == 32 else np.int64
+        bi, ei = copy_in(begin.astype(dt), dt), copy_in(end.astype(dt), dt)
+        out = aligned(n + 64, np.uint16, 0xFFFF)
+        assert emu.emu_seg_scan_offsets_f16(xi.ctypes.data, out.ctypes.data, nseg, bi.ctypes.data, ei.ctypes.data, bits, expected) == 0, emu.emu_last_error()
+        assert np.array_equal(out[:n], want) and np.all(out[n:] == 0xFFFF), (nseg, expected, bits)
+    # uniform offsets from one array (begin = offsets, end = offsets + 1) == the fixed-size scan; in place
+    seg, nseg = 200, 150
+    off = copy_in((np.arange(nseg + 1) * seg).astype(np.int32), np.int32)
+    buf = copy_in(x)
+    assert emu.emu_seg_scan_offsets_f16(buf.ctypes.data, buf.ctypes.data, nseg, off.ctypes.data, off.ctypes.data + 4, 32, seg) == 0
+    assert np.array_equal(buf[:nseg * seg], oracle.seg_scan_f64(x, nseg, seg).astype(np.float16).view(np.uint16)) and np.array_equal(buf[nseg * seg:n], x[nseg * seg:])
+    # buffers that are not 16-byte aligned: the 2-byte path everywhere
+    begin, end = disjoint_offsets(rng, n - 1, 200)
+    w64 = oracle.seg_scan_offsets_f64(x[1:], begin, end)
+    inside = ~np.isnan(w64)
+    bi, ei = copy_in(begin, np.int64), copy_in(end, np.int64)
+    out = aligned(n + 8, np.uint16, 0xFFFF)
+    assert emu.emu_seg_scan_offsets_f16(xi.ctypes.data + 2, out.ctypes.data + 2, 200, bi.ctypes.data, ei.ctypes.data, 64, 32) == 0
+    got = out[1:n]
+    assert np.array_equal(got[inside], w64[inside].astype(np.float16).view(np.uint16)) and np.all(got[~inside] == 0xFFFF)
 
 
 def test_generic_segment_sizes_and_preconditions(emu, oracle):

@@ -298,3 +298,47 @@ def test_segmented_reduction_over_offsets(tcu, oracle):
         want = oracle.seg_scan_f64(g, nseg, seg).astype(np.float16).view(np.uint16).reshape(nseg, seg)[:, -1]
         assert np.array_equal(to_host(got), want), seg
     assert tcu.seg_reduce_offsets(xd, off[:0], off[:0]).numel() == 0
+
+
+def test_segmented_scan_over_offsets(tcu, oracle):
+    """tcu_seg_scan_offsets_f16: disjoint ragged segments with gaps and empty segments, 32- and 64-bit offsets, every
+    lanes-per-segment choice, against the fp64 oracle (2 ulp + 1e-3*sqrt(segment length)); positions outside every
+    segment keep their sentinel; exact-grid inputs bit for bit; uniform offsets equal the fixed-size scan; in place."""
+    import torch
+
+    rng = np.random.default_rng(21)
+    n = 1 << 22
+    x = oracle.generate_f16(n, 12, oracle.DIST_UNIFORM)
+    g = oracle.generate_f16(n, 13, oracle.DIST_GRID)
+    xd, gd = to_dev(x), to_dev(g)
+    for nseg in (150000, 20000, 500, 3):
+        cuts = np.sort(rng.choice(n, 2 * nseg, replace=False))
+        begin, end = cuts[0::2].astype(np.int64), cuts[1::2].astype(np.int64)
+        end[::9] = begin[::9]
+        ref = oracle.seg_scan_offsets_f64(x, begin, end)
+        inside = ~np.isnan(ref)
+        seglen = np.zeros(n)
+        for b, e in zip(begin, end):  # tolerance term: sqrt of the length of the segment an element belongs to
+            seglen[b:e] = e - b
+        wg = oracle.seg_scan_offsets_f64(g, begin, end)
+        exact = np.nanmax(np.abs(wg)) < 4096
+        for dtype in (torch.int32, torch.int64):
+            bd, ed = torch.from_numpy(begin).to(dtype).cuda(), torch.from_numpy(end).to(dtype).cuda()
+            for expected in (0, 16, 40, 100, 5000):
+                out = torch.full((n,), -7.0, dtype=torch.float16, device="cuda")
+                tcu.seg_scan_offsets(xd, bd, ed, expected_segment_size=expected, out=out)
+                got = to_host(out)
+                assert np.all(got[~inside] == np.float16(-7.0).view(np.uint16)), "wrote outside the segments"
+                gv = got[inside].view(np.float16).astype(np.float64)
+                allow = 2 * np.maximum(np.spacing(np.abs(ref[inside]).astype(np.float16)).astype(np.float64), 2.0 ** -24) + 1e-3 * np.sqrt(seglen[inside])
+                bad = np.abs(gv - ref[inside]) > allow
+                assert not bad.any(), (nseg, str(dtype), expected, int(bad.sum()))
+                if exact:
+                    og = to_host(tcu.seg_scan_offsets(gd, bd, ed, expected_segment_size=expected))
+                    assert np.array_equal(og[inside], wg[inside].astype(np.float16).view(np.uint16)), (nseg, str(dtype), expected)
+    for seg in (16, 48, 2048):
+        nseg = (1 << 20) // seg
+        off = (torch.arange(nseg + 1, dtype=torch.int64) * seg).to(torch.int32).cuda()
+        buf = gd[: nseg * seg].clone()
+        tcu.seg_scan_offsets(buf, off[:-1], off[1:], expected_segment_size=seg, out=buf)  # in place
+        assert np.array_equal(to_host(buf), oracle.seg_scan_f64(g, nseg, seg).astype(np.float16).view(np.uint16)), seg

@@ -192,3 +192,37 @@ def test_offsets_reduction_against_numpy_and_the_fixed_size_oracle(oracle):
     # overlapping segments are independent: [0, 100) and [50, 150) share elements
     o = oracle.seg_reduce_offsets_f64(x, np.array([0, 50, 0]), np.array([100, 150, 150]))
     assert abs(o[2] - (o[0] + o[1] - oracle.seg_reduce_offsets_f64(x, np.array([50]), np.array([100]))[0])) <= 1e-9
+
+
+def test_offsets_scan_against_numpy_and_the_fixed_size_oracle(oracle):
+    """Prefix sums inside segments given by offsets: numpy cumsum of every slice (float64, and sequential float32
+    rounded to fp16), the fixed-size functions on uniform offsets, untouched positions outside every segment,
+    last prefix of a segment == its reduction."""
+    rng = np.random.default_rng(5)
+    n = 30000
+    x = oracle.generate_f16(n, 6, oracle.DIST_UNIFORM)
+    xf = x.view(np.float16)
+    # disjoint ragged segments with gaps, some empty
+    cuts = np.sort(rng.choice(n, 600, replace=False))
+    begin, end = cuts[0::2].copy(), cuts[1::2].copy()
+    end[::13] = begin[::13]
+    got64 = oracle.seg_scan_offsets_f64(x, begin, end)
+    got16 = oracle.seg_scan_offsets_ref(x, begin, end, fill=0xFFFF)
+    covered = np.zeros(n, bool)
+    for b, e in zip(begin, end):
+        if e <= b:
+            continue
+        covered[b:e] = True
+        assert np.allclose(got64[b:e], np.cumsum(xf[b:e].astype(np.float64)), rtol=0, atol=1e-9)
+        acc, want = np.float32(0), []
+        for v in xf[b:e]:
+            acc = np.float32(acc + np.float32(v))
+            want.append(np.float16(acc))
+        assert np.array_equal(got16[b:e], np.array(want, np.float16).view(np.uint16))
+    assert np.all(np.isnan(got64[~covered])) and np.all(got16[~covered] == 0xFFFF)
+    live = end > begin
+    assert np.allclose(got64[end[live] - 1], oracle.seg_reduce_offsets_f64(x, begin, end)[live], rtol=0, atol=1e-9)
+    seg, nseg = 75, 400
+    b = np.arange(nseg) * seg
+    assert np.array_equal(oracle.seg_scan_offsets_f64(x, b, b + seg)[:nseg * seg], oracle.seg_scan_f64(x, nseg, seg))
+    assert np.array_equal(oracle.seg_scan_offsets_ref(x, b, b + seg)[:nseg * seg], oracle.seg_scan_ref(x, nseg, seg))
