@@ -180,6 +180,17 @@ int tcu_gemv_f16_f32(const void *d_A, const void *d_x, void *d_y, size_t M, size
  * (reference compute_gemm_naive, src/gemm/wmma_naive.cu:33-88). */
 int tcu_gemm_f16_f32(const void *d_A, const void *d_B, const void *d_C, void *d_D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream);
 
+/* The fp16-output twins: y (GEMV) and C, D (GEMM) hold fp16, alpha and beta are applied in
+ * fp32 and the result is rounded once (to nearest even).  They replace
+ * compute_wmma_hgemv_naive (reference src/gemv/wmma_naive.cu:96-160), compute_hgemm
+ * (src/gemm/wmma.cu:367-560) and compute_hgemm_naive (src/gemm/wmma_naive.cu:90-145).  The
+ * reference accumulates those in fp16 inside the WMMA unit; the MFMA unit accumulates in fp32
+ * only, so products are summed in fp32 here as in the fp32-output entry points.  Layouts,
+ * variants and the C == D allowance are the same; D and C must be 4-byte aligned for the
+ * tiled GEMM kernels (any alignment falls back to the scalar kernel under AUTO). */
+int tcu_gemv_f16_f16(const void *d_A, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, int variant, void *stream);
+int tcu_gemm_f16_f16(const void *d_A, const void *d_B, const void *d_C, void *d_D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream);
+
 /* ---- fills, conversions, inputs ---------------------------------------------------------------- */
 
 /* d[i] = (half) value.  Replaces cuda_memory_set / setFP16 (reference

@@ -12,7 +12,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 EXPORTS = [
     "tcu_abi_version", "tcu_last_error", "tcu_init", "tcu_device_info", "tcu_set_option",
     "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_offsets_f16", "tcu_add_partial_sums_f16",
-    "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32",
+    "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32", "tcu_gemv_f16_f16", "tcu_gemm_f16_f16",
     "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_lane_probe",
 ]
 
@@ -90,6 +90,8 @@ def lib():
         L.tcu_full_scan_f16.argtypes = [vp, vp, sz, vp, c.POINTER(sz), ci, sz, ci, vp]
         L.tcu_gemv_f16_f32.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci, vp]
         L.tcu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci, vp]
+        L.tcu_gemv_f16_f16.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci, vp]
+        L.tcu_gemm_f16_f16.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci, vp]
         L.tcu_fill_f16.argtypes = [vp, cf, sz, vp]
         L.tcu_convert_f32_to_f16.argtypes = [vp, vp, sz, vp]
         L.tcu_generate_f16.argtypes = [vp, sz, c.c_uint64, ci, sz, vp]
@@ -241,20 +243,36 @@ def full_workspace_bytes(kind, n, strategy=FullStrategy.AUTO, segment_size=0, wa
     return need.value
 
 
-def gemv(A, x, alpha=1.0, beta=0.0, y=None, variant=Variant.AUTO, stream=None):
-    """y = alpha*A@x + beta*y; A (M,K) row-major fp16, x (K,) fp16, y (M,) fp32."""
+def _out_entry(t, what, f32_entry, f16_entry):
+    torch = _torch()
+    if t.dtype == torch.float32:
+        return f32_entry
+    if t.dtype == torch.float16:
+        return f16_entry
+    raise TypeError(f"{what} must be a float32 or float16 tensor")
+
+
+def gemv(A, x, alpha=1.0, beta=0.0, y=None, variant=Variant.AUTO, stream=None, out_dtype=None):
+    """y = alpha*A@x + beta*y; A (M,K) row-major fp16, x (K,) fp16, y (M,) fp32 or fp16.
+
+    The dtype of `y` (or `out_dtype` when y is None; default float32) selects
+    tcu_gemv_f16_f32 or tcu_gemv_f16_f16."""
     torch = _torch()
     _need_f16(A, "A")
     _need_f16(x, "x")
     M, K = A.shape
     if y is None:
-        y = torch.zeros(M, dtype=torch.float32, device=A.device)
-    _check(lib().tcu_gemv_f16_f32(_ptr(A), _ptr(x), _ptr(y), M, K, alpha, beta, int(variant), _stream(stream)))
+        y = torch.zeros(M, dtype=out_dtype or torch.float32, device=A.device)
+    entry = _out_entry(y, "y", lib().tcu_gemv_f16_f32, lib().tcu_gemv_f16_f16)
+    _check(entry(_ptr(A), _ptr(x), _ptr(y), M, K, alpha, beta, int(variant), _stream(stream)))
     return y
 
 
-def gemm(A, Bt, alpha=1.0, beta=0.0, C=None, out=None, variant=Variant.AUTO, stream=None):
-    """D = alpha*A@B + beta*C with A (M,K) fp16 and B given column-major, i.e. as Bt (N,K) fp16."""
+def gemm(A, Bt, alpha=1.0, beta=0.0, C=None, out=None, variant=Variant.AUTO, stream=None, out_dtype=None):
+    """D = alpha*A@B + beta*C with A (M,K) fp16 and B given column-major, i.e. as Bt (N,K) fp16.
+
+    C and D are float32 (tcu_gemm_f16_f32) or float16 (tcu_gemm_f16_f16): the dtype of `out`,
+    else of `C`, else `out_dtype` (default float32)."""
     torch = _torch()
     _need_f16(A, "A")
     _need_f16(Bt, "Bt")
@@ -263,8 +281,11 @@ def gemm(A, Bt, alpha=1.0, beta=0.0, C=None, out=None, variant=Variant.AUTO, str
     if K != K2:
         raise ValueError("A and Bt disagree on K")
     if out is None:
-        out = torch.empty(M, N, dtype=torch.float32, device=A.device)
-    _check(lib().tcu_gemm_f16_f32(_ptr(A), _ptr(Bt), _ptr(C), _ptr(out), M, N, K, alpha, beta, int(variant), _stream(stream)))
+        out = torch.empty(M, N, dtype=C.dtype if C is not None else (out_dtype or torch.float32), device=A.device)
+    if C is not None and C.dtype != out.dtype:
+        raise TypeError("C and out must have the same dtype")
+    entry = _out_entry(out, "out", lib().tcu_gemm_f16_f32, lib().tcu_gemm_f16_f16)
+    _check(entry(_ptr(A), _ptr(Bt), _ptr(C), _ptr(out), M, N, K, alpha, beta, int(variant), _stream(stream)))
     return out
 
 

@@ -685,8 +685,9 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
 
 // ----- GEMV / GEMM -----------------------------------------------------------------------------
 
-inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
-  const char *what = "tcu_gemv_f16_f32";
+// OUT = float: tcu_gemv_f16_f32; OUT = half_t: tcu_gemv_f16_f16 (y in fp16)
+template <typename OUT>
+inline int gemv_dispatch_typed(const char *what, const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
   if (!(variant == TCU_VARIANT_AUTO || variant == TCU_VARIANT_WAVE_SHUFFLE || variant == TCU_VARIANT_MFMA_16N)) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": variant must be AUTO, WAVE_SHUFFLE or MFMA_16N");
   if (M == 0) return TCU_OK;
   if (!y || (K && (!A || !x))) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
@@ -697,19 +698,19 @@ inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t
     if (variant != TCU_VARIANT_AUTO) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": K must be a positive multiple of 8 and A, x 16-byte aligned");
     const size_t grid = (M + 3) / 4;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    launch(gemv_generic_kernel, (unsigned)grid, block, stream, static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(x), static_cast<float *>(y), M, K, alpha, beta);
+    launch(gemv_generic_kernel<OUT>, (unsigned)grid, block, stream, static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(x), static_cast<OUT *>(y), M, K, alpha, beta);
     return TCU_OK;
   }
   const half8_t *a = static_cast<const half8_t *>(A), *xv = static_cast<const half8_t *>(x);
-  float *yy = static_cast<float *>(y);
+  OUT *yy = static_cast<OUT *>(y);
   if (variant == TCU_VARIANT_MFMA_16N) {
     const size_t strips = (M + 15) / 16;
     const size_t grid = (strips + 3) / 4;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     if (nt)
-      launch(gemv_mfma_kernel<true>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+      launch(gemv_mfma_kernel<true, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
     else
-      launch(gemv_mfma_kernel<false>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+      launch(gemv_mfma_kernel<false, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
     return TCU_OK;
   }
   const size_t k_tiles = (K / 8 + 63) / 64;
@@ -724,9 +725,9 @@ inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t
 #define TCU_GEMV_BLOCK(R_, U_)                                                                                              \
   if (rows == R_ && bu == U_) {                                                                                            \
     if (nt)                                                                                                                \
-      launch(gemv_block_kernel<R_, U_, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);         \
+      launch(gemv_block_kernel<R_, U_, true, OUT>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);         \
     else                                                                                                                   \
-      launch(gemv_block_kernel<R_, U_, false>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);        \
+      launch(gemv_block_kernel<R_, U_, false, OUT>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);        \
     return TCU_OK;                                                                                                         \
   }
     TCU_GEMV_BLOCK(1, 1) TCU_GEMV_BLOCK(1, 2) TCU_GEMV_BLOCK(1, 4) TCU_GEMV_BLOCK(1, 8)
@@ -741,23 +742,31 @@ inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t
   const size_t grid = (waves + 3) / 4;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
   if (nt)
-    launch(gemv_dot_kernel<ROWS, UK, true>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+    launch(gemv_dot_kernel<ROWS, UK, true, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
   else
-    launch(gemv_dot_kernel<ROWS, UK, false>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+    launch(gemv_dot_kernel<ROWS, UK, false, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
   return TCU_OK;
 }
+inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
+  return gemv_dispatch_typed<float>("tcu_gemv_f16_f32", A, x, y, M, K, alpha, beta, variant, stream);
+}
+inline int hgemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
+  return gemv_dispatch_typed<half_t>("tcu_gemv_f16_f16", A, x, y, M, K, alpha, beta, variant, stream);
+}
 
-inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream) {
-  const char *what = "tcu_gemm_f16_f32";
+// OUT = float: tcu_gemm_f16_f32; OUT = half_t: tcu_gemm_f16_f16 (C and D in fp16)
+template <typename OUT>
+inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, const void *C, void *D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream) {
   if (!(variant == TCU_VARIANT_AUTO || variant == TCU_VARIANT_BLOCK_LDS || variant == TCU_VARIANT_MFMA_16N)) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": variant must be AUTO, BLOCK_LDS or MFMA_16N");
   if (M == 0 || N == 0) return TCU_OK;
   if (!D || (K && (!A || !B)) || (beta != 0.0f && !C)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
-  const bool al = aligned16(A) && aligned16(B);
+  // the tiled kernels move fp16 outputs as 32-bit pairs
+  const bool al = aligned16(A) && aligned16(B) && (sizeof(OUT) == 4 || ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & 3u) == 0);
   const bool lds_ok = al && M % kGemmBM == 0 && N % kGemmBN == 0 && K % kGemmBK == 0 && K > 0;
   const bool direct_ok = al && M % 32 == 0 && N % 32 == 0 && K % 16 == 0 && K > 0;
   const half8_t *a = static_cast<const half8_t *>(A), *b = static_cast<const half8_t *>(B);
-  const float *c = static_cast<const float *>(C);
-  float *d = static_cast<float *>(D);
+  const OUT *c = static_cast<const OUT *>(C);
+  OUT *d = static_cast<OUT *>(D);
   if (variant == TCU_VARIANT_BLOCK_LDS && !lds_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the LDS kernel needs M, N multiples of 128 and K a multiple of 32");
   if (variant == TCU_VARIANT_MFMA_16N && !direct_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the direct kernel needs M, N multiples of 32 and K a multiple of 16");
   if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && options().gemm_big_tiles) {
@@ -771,11 +780,11 @@ inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, s
     const int direct_lds = options().gemm_direct_lds >= 0 ? options().gemm_direct_lds : (K % 16384 == 0 ? 0 : (K % 64 == 0 && M * N <= (size_t)8192 * 8192 ? 64 : 4));
     if (direct_lds > 0 && K <= ((size_t)1 << 22)) {
       if (direct_lds == 64 && K % 64 == 0)
-        launch(gemm_dlds_kernel<64, 2>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+        launch(gemm_dlds_kernel<64, 2, OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       else if (direct_lds == 3)
-        launch(gemm_dlds_kernel<32, 3>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+        launch(gemm_dlds_kernel<32, 3, OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       else
-        launch(gemm_dlds_kernel<32, 4>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+        launch(gemm_dlds_kernel<32, 4, OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       return TCU_OK;
     }
     const bool bk64 = K % 64 == 0 && options().gemm_bk64;
@@ -783,7 +792,7 @@ inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, s
     int depth = options().gemm_depth < 1 ? 1 : (options().gemm_depth > 4 ? 4 : options().gemm_depth);
     if (bk64 && depth > 2) depth = 2;
     while (steps % (size_t)depth) depth--;  // the kernels take whole groups of `depth` steps
-#define TCU_GEMM256(BK_, D_) launch(gemm_lds256_kernel<BK_, D_>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta)
+#define TCU_GEMM256(BK_, D_) launch(gemm_lds256_kernel<BK_, D_, OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta)
     if (bk64) {
       if (depth == 2) TCU_GEMM256(64, 2); else TCU_GEMM256(64, 1);
     } else {
@@ -798,18 +807,24 @@ inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, s
   } else if (lds_ok && variant != TCU_VARIANT_MFMA_16N) {
     const size_t grid = (M / kGemmBM) * (N / kGemmBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    launch(gemm_lds_kernel, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+    launch(gemm_lds_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
   } else if (direct_ok) {
     const size_t tiles = (M / 32) * (N / 32);
     const size_t grid = (tiles + 3) / 4;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    launch(gemm_direct_kernel, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+    launch(gemm_direct_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
   } else {
     const size_t grid = (M * N + 255) / 256;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    launch(gemm_generic_kernel, (unsigned)grid, 256u, stream, static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B), c, d, M, N, K, alpha, beta);
+    launch(gemm_generic_kernel<OUT>, (unsigned)grid, 256u, stream, static_cast<const uint16_t *>(A), static_cast<const uint16_t *>(B), c, d, M, N, K, alpha, beta);
   }
   return TCU_OK;
+}
+inline int gemm_dispatch(const void *A, const void *B, const void *C, void *D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream) {
+  return gemm_dispatch_typed<float>("tcu_gemm_f16_f32", A, B, C, D, M, N, K, alpha, beta, variant, stream);
+}
+inline int hgemm_dispatch(const void *A, const void *B, const void *C, void *D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream) {
+  return gemm_dispatch_typed<half_t>("tcu_gemm_f16_f16", A, B, C, D, M, N, K, alpha, beta, variant, stream);
 }
 
 // ----- fills, conversions, inputs, probes --------------------------------------------------------

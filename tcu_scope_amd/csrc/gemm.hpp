@@ -31,22 +31,60 @@ TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_
 // D and C are streamed once: non-temporal accesses keep them from displacing the A and B
 // panels that other tiles reuse from L2.  All of a tile's C values are read before its first
 // store, so the loads overlap and C may be the same buffer as D.
-TCU_DEVICE void gemm_store_tile(float *D, const float *C, size_t ldc, size_t row0, size_t col0, const float16_t &acc, int lane, float alpha, float beta) {
-  const size_t base = (row0 + 4 * (lane >> 5)) * ldc + col0 + (lane & 31);
-  if (beta == 0.0f) {
+// OUT = float: a lane owns column (lane & 31) of rows 8*(i/4) + 4*(lane >> 5) + i%4.
+// OUT = half_t (C and D in fp16, the layout of the reference's compute_hgemm,
+// src/gemm/wmma.cu:367-560; products still accumulate in fp32, the only accumulator width the
+// MFMA unit has): neighbouring lanes trade one value of each pair of rows, so that an even lane
+// owns two adjacent columns of the even row and the odd lane the same columns of the odd row,
+// and every access moves a 32-bit pair.
+template <typename OUT>
+TCU_DEVICE void gemm_store_tile(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float16_t &acc, int lane, float alpha, float beta) {
+  if constexpr (sizeof(OUT) == 4) {
+    const size_t base = (row0 + 4 * (lane >> 5)) * ldc + col0 + (lane & 31);
+    if (beta == 0.0f) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) __builtin_nontemporal_store(alpha * acc[i], D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+      for (int i = 0; i < 16; i++) __builtin_nontemporal_store(alpha * acc[i], D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+    } else {
+      float c[16];
+#pragma unroll
+      for (int i = 0; i < 16; i++) c[i] = __builtin_nontemporal_load(C + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+#pragma unroll
+      for (int i = 0; i < 16; i++) __builtin_nontemporal_store(alpha * acc[i] + beta * c[i], D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+    }
   } else {
-    float c[16];
+    const bool odd = (lane & 1) != 0;
+    // 32-bit word index of this lane's pair in row (row0 + 4*(lane >> 5) + (lane & 1)); ldc and col0 are even
+    const size_t base = ((row0 + 4 * (lane >> 5) + (lane & 1)) * ldc + col0 + (lane & 30)) >> 1;
+    const size_t ldw = ldc >> 1;
+    uint32_t *d32 = reinterpret_cast<uint32_t *>(D);
+    const uint32_t *c32 = reinterpret_cast<const uint32_t *>(C);
+    float lo[8], hi[8];
 #pragma unroll
-    for (int i = 0; i < 16; i++) c[i] = __builtin_nontemporal_load(C + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+    for (int p = 0; p < 8; p++) {  // rows 8*(p/2) + 2*(p%2) + {0, 1} of the lane's group of four
+      const float send = odd ? acc[2 * p] : acc[2 * p + 1];
+      const float recv = dpp<DPP_QUAD_XOR1>(send, send);
+      lo[p] = odd ? recv : acc[2 * p];
+      hi[p] = odd ? acc[2 * p + 1] : recv;
+    }
+    if (beta == 0.0f) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) __builtin_nontemporal_store(alpha * acc[i] + beta * c[i], D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+      for (int p = 0; p < 8; p++) __builtin_nontemporal_store(pack_f16x2(alpha * lo[p], alpha * hi[p]), d32 + base + (size_t)(8 * (p / 2) + 2 * (p % 2)) * ldw);
+    } else {
+      uint32_t c[8];
+#pragma unroll
+      for (int p = 0; p < 8; p++) c[p] = __builtin_nontemporal_load(c32 + base + (size_t)(8 * (p / 2) + 2 * (p % 2)) * ldw);
+#pragma unroll
+      for (int p = 0; p < 8; p++) {
+        const half2_t cv = __builtin_bit_cast(half2_t, c[p]);
+        __builtin_nontemporal_store(pack_f16x2(alpha * lo[p] + beta * (float)cv[0], alpha * hi[p] + beta * (float)cv[1]), d32 + base + (size_t)(8 * (p / 2) + 2 * (p % 2)) * ldw);
+      }
+    }
   }
 }
 
 // M % 128 == 0, N % 128 == 0, K % 32 == 0; 256 threads.
-__global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
   __shared__ __attribute__((aligned(16))) half_t lds_a[2][kGemmBM * kGemmLdsStride];
   __shared__ __attribute__((aligned(16))) half_t lds_b[2][kGemmBN * kGemmLdsStride];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -145,8 +183,8 @@ TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_
 // LDS rows are padded by 8 halves (the 128-bit fragment reads of 16 lanes hit distinct
 // banks).
 constexpr int kGemmBigBM = 256, kGemmBigBN = 256;
-template <int BK, int DEPTH>
-__global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
+template <int BK, int DEPTH, typename OUT>
+__global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha,
                                                           float beta) {
   constexpr int STRIDE = BK + 8;            // halves per LDS row
   constexpr int CPR = BK / 8;               // chunks per row
@@ -317,8 +355,8 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
 // before the last substep a wave waits for its own transfers of step s + 1, the barrier
 // publishes everybody's, and the fragments of step s + 1, substep 0, are read while the
 // last 16 MFMAs of step s run.
-template <int BK, int NBUF>
-__global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+template <int BK, int NBUF, typename OUT>
+__global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
   constexpr int ROWH = BK;                           // halves per LDS row
   constexpr int CPR = BK / 8;                        // chunks per row
   constexpr int RPT = 64 / CPR;                      // rows per transfer instruction
@@ -454,7 +492,8 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
 }
 
 // M % 32 == 0, N % 32 == 0, K % 16 == 0; one 32 x 32 tile per wave.
-__global__ __launch_bounds__(kWave * 4) void gemm_direct_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
+template <typename OUT>
+__global__ __launch_bounds__(kWave * 4) void gemm_direct_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha,
                                                                  float beta) {
   const int lane = lane_id();
   const size_t tiles_m = M / 32, tiles_n = N / 32;
@@ -471,14 +510,15 @@ __global__ __launch_bounds__(kWave * 4) void gemm_direct_kernel(const half8_t *_
   gemm_store_tile(D, C, N, tile_m * 32, tile_n * 32, acc, lane, alpha, beta);
 }
 
-__global__ __launch_bounds__(256) void gemm_generic_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, const float *C, float *D, size_t M, size_t N, size_t K, float alpha,
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha,
                                                             float beta) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= M * N) return;
   const size_t m = idx / N, n = idx % N;
   float acc = 0.0f;
   for (size_t k = 0; k < K; k++) acc += (float)__builtin_bit_cast(half_t, A[m * K + k]) * (float)__builtin_bit_cast(half_t, B[n * K + k]);
-  D[idx] = beta == 0.0f ? alpha * acc : alpha * acc + beta * C[idx];
+  D[idx] = (OUT)(beta == 0.0f ? alpha * acc : alpha * acc + beta * (float)C[idx]);
 }
 
 }  // namespace tcu

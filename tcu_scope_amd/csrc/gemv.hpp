@@ -1,4 +1,6 @@
-// y = alpha * A x + beta * y;  A: M x K row-major fp16, x: K fp16, y: M fp32.
+// y = alpha * A x + beta * y;  A: M x K row-major fp16, x: K fp16, y: M values of OUT = float
+// or half_t (the reference's compute_wmma_hgemv_naive keeps y in fp16,
+// src/gemv/wmma_naive.cu:96-160); products accumulate in fp32 either way.
 //
 // The operation streams A once (2*M*K bytes) and is bound by HBM bandwidth.
 //   gemv_dot_kernel  : each wave owns ROWS consecutive rows; per step every lane loads one
@@ -20,6 +22,11 @@
 
 namespace tcu {
 
+template <typename OUT>
+TCU_DEVICE void gemv_update(OUT *p, float s, float alpha, float beta) {
+  *p = (OUT)(beta == 0.0f ? alpha * s : alpha * s + beta * (float)*p);
+}
+
 TCU_DEVICE float dot8(half8_t a, half8_t x, float acc) {
   acc = fdot2(__builtin_shufflevector(a, a, 0, 1), __builtin_shufflevector(x, x, 0, 1), acc);
   acc = fdot2(__builtin_shufflevector(a, a, 2, 3), __builtin_shufflevector(x, x, 2, 3), acc);
@@ -29,8 +36,8 @@ TCU_DEVICE float dot8(half8_t a, half8_t x, float acc) {
 }
 
 // K must be a multiple of 8; rows are 16-byte aligned.
-template <int ROWS, int UK, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, float *__restrict__ y, size_t M, size_t k_chunks, float alpha,
+template <int ROWS, int UK, bool NT, typename OUT>
+__global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t k_chunks, float alpha,
                                                               float beta) {
   const int lane = lane_id();
   const size_t row0 = ((size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block()) * ROWS;
@@ -60,10 +67,7 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__re
 #pragma unroll
   for (int r = 0; r < ROWS; r++) {
     const float s = lane_group_sum<6>(acc[r]);
-    if (lane == 63 && row0 + r < M) {
-      float *p = y + row0 + r;
-      *p = beta == 0.0f ? alpha * s : alpha * s + beta * *p;
-    }
+    if (lane == 63 && row0 + r < M) gemv_update(y + row0 + r, s, alpha, beta);
   }
 }
 
@@ -71,8 +75,8 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__re
 // w*U .. w*U+U-1 of every step of WPB*U tiles (the x chunks it loads serve all ROWS rows),
 // partial dot products meet in LDS.  Same access shape as the block-per-segment reduction,
 // which is what moves long contiguous rows fastest.
-template <int ROWS, int U, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, float *__restrict__ y, size_t M, size_t k_chunks, float alpha,
+template <int ROWS, int U, bool NT, typename OUT>
+__global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t k_chunks, float alpha,
                                                                 float beta) {
   __shared__ float partial[ROWS][kMaxWaves];
   const int lane = lane_id(), wave = wave_in_block();
@@ -109,14 +113,13 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__
   if (threadIdx.x < ROWS && row0 + threadIdx.x < M) {
     float s = 0.0f;
     for (int w = 0; w < WPB; w++) s += partial[threadIdx.x][w];
-    float *p = y + row0 + threadIdx.x;
-    *p = beta == 0.0f ? alpha * s : alpha * s + beta * *p;
+    gemv_update(y + row0 + threadIdx.x, s, alpha, beta);
   }
 }
 
 // K must be a multiple of 8.  One wave per 16-row strip.
-template <bool NT>
-__global__ __launch_bounds__(kMaxBlock) void gemv_mfma_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, float *__restrict__ y, size_t M, size_t k_chunks, float alpha,
+template <bool NT, typename OUT>
+__global__ __launch_bounds__(kMaxBlock) void gemv_mfma_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t k_chunks, float alpha,
                                                                float beta) {
   const int lane = lane_id();
   const int r = lane & 15, b = lane >> 4;
@@ -149,19 +152,20 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_mfma_kernel(const half8_t *__r
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const size_t m = row0 + 4 * b + i;
-      if (m < M) y[m] = beta == 0.0f ? alpha * acc[i] : alpha * acc[i] + beta * y[m];
+      if (m < M) gemv_update(y + m, acc[i], alpha, beta);
     }
   }
 }
 
-__global__ __launch_bounds__(kMaxBlock) void gemv_generic_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ x, float *__restrict__ y, size_t M, size_t K, float alpha, float beta) {
+template <typename OUT>
+__global__ __launch_bounds__(kMaxBlock) void gemv_generic_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t K, float alpha, float beta) {
   const int lane = lane_id();
   const size_t row = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
   if (row >= M) return;
   float acc = 0.0f;
   for (size_t k = lane; k < K; k += 64) acc += (float)__builtin_bit_cast(half_t, A[row * K + k]) * (float)__builtin_bit_cast(half_t, x[k]);
   acc = lane_group_sum<6>(acc);
-  if (lane == 63) y[row] = beta == 0.0f ? alpha * acc : alpha * acc + beta * y[row];
+  if (lane == 63) gemv_update(y + row, acc, alpha, beta);
 }
 
 }  // namespace tcu

@@ -1,19 +1,33 @@
-// GEMM / GEMV benchmarks under the reference's names (src/gemm/wmma.cu:776, wmma_naive.cu:339,
-// wmma_sharedmem.cu, src/gemv/wmma_naive.cu:357, wmma_sharedmem.cu) and the timed CPU path.
+// GEMM / GEMV benchmarks under the reference's names (src/gemm/wmma.cu:776-777,
+// wmma_naive.cu:339-340, wmma_sharedmem.cu, src/gemv/wmma_naive.cu:357-358, wmma_sharedmem.cu;
+// the H* names keep C, D or y in fp16), the accuracy comparisons (src/gemm/accuracy.cu:277,
+// src/gemv/accuracy.cu:332) and the timed CPU path.
 #include "args.hpp"
 #include "harness.hpp"
 
 static void CUDA_WMMA_GEMM(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_BLOCK_LDS, "CUDA_WMMA_GEMM"); }
 static void CUDA_WMMA_GEMM_SHAREDMEM(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_BLOCK_LDS, "CUDA_WMMA_GEMM_SHAREDMEM"); }
 static void CUDA_WMMA_GEMM_NAIVE(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMM_NAIVE"); }
+static void CUDA_WMMA_HGEMM(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_BLOCK_LDS, "CUDA_WMMA_HGEMM", true); }
+static void CUDA_WMMA_HGEMM_NAIVE(benchmark::State &state) { harness::run_gemm(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_HGEMM_NAIVE", true); }
+static void CUDA_WMMA_GEMM_ACCURACY(benchmark::State &state) { harness::run_gemm_accuracy(state, "CUDA_WMMA_GEMM_ACCURACY"); }
 BENCHMARK(CUDA_WMMA_GEMM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_HGEMM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_HGEMM_NAIVE)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_GEMM_ACCURACY)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUDA_WMMA_GEMM_SHAREDMEM)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUDA_WMMA_GEMM_NAIVE)->Apply(GemmArgs)->UseManualTime();
 
 static void CUDA_WMMA_GEMV_NAIVE(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMV_NAIVE"); }
 static void CUDA_WMMA_GEMV_SHAREDMEM(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMV_SHAREDMEM"); }
 static void TCU_WAVE_GEMV(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_WAVE_SHUFFLE, "TCU_WAVE_GEMV"); }
+static void CUDA_WMMA_HGEMV_NAIVE(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_HGEMV_NAIVE", true); }
+static void TCU_WAVE_HGEMV(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_WAVE_SHUFFLE, "TCU_WAVE_HGEMV", true); }
+static void CUDA_WMMA_GEMV_ACCURACY(benchmark::State &state) { harness::run_gemv_accuracy(state, "CUDA_WMMA_GEMV_ACCURACY"); }
 BENCHMARK(CUDA_WMMA_GEMV_NAIVE)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_HGEMV_NAIVE)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(TCU_WAVE_HGEMV)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_GEMV_ACCURACY)->Apply(GemvArgs)->UseManualTime();
 BENCHMARK(CUDA_WMMA_GEMV_SHAREDMEM)->Apply(GemvArgs)->UseManualTime();
 BENCHMARK(TCU_WAVE_GEMV)->Apply(GemvArgs)->UseManualTime();
 

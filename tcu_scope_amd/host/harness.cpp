@@ -442,22 +442,30 @@ void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, i
   });
 }
 
-void run_gemv(benchmark::State &state, int variant, const char *name) {
+void run_gemv(benchmark::State &state, int variant, const char *name, bool half_out) {
   guarded(state, [&] {
     const size_t M = state.range(0), K = state.range(1);
     const float alpha = 1.0f, beta = 0.0f;
-    DeviceBuffer A(M * K * 2), x(K * 2), y(M * 4);
+    const size_t out_size = half_out ? 2 : 4;  // bytes per element of y
+    const auto gemv = half_out ? tcu_gemv_f16_f16 : tcu_gemv_f16_f32;
+    DeviceBuffer A(M * K * 2), x(K * 2), y(M * out_size);
     TCU_CHECK(tcu_generate_f16(A.get(), M * K, flags().seed, TCU_DIST_NORMAL, 0, nullptr));
     TCU_CHECK(tcu_generate_f16(x.get(), K, flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
-    PRINT_IF_ERROR(hipMemset(y.get(), 0, M * 4));
-    TCU_CHECK(tcu_gemv_f16_f32(A.get(), x.get(), y.get(), M, K, alpha, beta, variant, nullptr));
+    PRINT_IF_ERROR(hipMemset(y.get(), 0, M * out_size));
+    TCU_CHECK(gemv(A.get(), x.get(), y.get(), M, K, alpha, beta, variant, nullptr));
     PRINT_IF_ERROR(hipDeviceSynchronize());
     if (should_verify(M * K)) {
       std::vector<uint16_t> hA(M * K), hx(K);
       std::vector<float> hy(M);
       PRINT_IF_ERROR(hipMemcpy(hA.data(), A.get(), M * K * 2, hipMemcpyDeviceToHost));
       PRINT_IF_ERROR(hipMemcpy(hx.data(), x.get(), K * 2, hipMemcpyDeviceToHost));
-      PRINT_IF_ERROR(hipMemcpy(hy.data(), y.get(), M * 4, hipMemcpyDeviceToHost));
+      if (half_out) {
+        std::vector<uint16_t> raw(M);
+        PRINT_IF_ERROR(hipMemcpy(raw.data(), y.get(), M * 2, hipMemcpyDeviceToHost));
+        for (size_t m = 0; m < M; m++) hy[m] = half_to_float(raw[m]);
+      } else {
+        PRINT_IF_ERROR(hipMemcpy(hy.data(), y.get(), M * 4, hipMemcpyDeviceToHost));
+      }
       for (size_t m = 0; m < M; m++) {
         double s = 0;
         for (size_t k = 0; k < K; k++) s += (double)half_to_float(hA[m * K + k]) * half_to_float(hx[k]);
@@ -467,13 +475,13 @@ void run_gemv(benchmark::State &state, int variant, const char *name) {
     EventPair ev;
     for (auto _ : state) {
       ev.start();
-      TCU_CHECK(tcu_gemv_f16_f32(A.get(), x.get(), y.get(), M, K, alpha, beta, variant, nullptr));
+      TCU_CHECK(gemv(A.get(), x.get(), y.get(), M, K, alpha, beta, variant, nullptr));
       const float ms = ev.stop_ms();
       state.PauseTiming();
       state.SetIterationTime(ms / 1000);
       state.ResumeTiming();
     }
-    const double bytes = 2.0 * M * K + 2.0 * K + 4.0 * M;
+    const double bytes = 2.0 * M * K + 2.0 * K + (double)out_size * M;
     state.counters.insert({{"M", (double)M},
                            {"N", (double)K},
                            {"flops", {state.iterations() * 2.0 * M * K, benchmark::Counter::kAvgThreadsRate}},
@@ -482,22 +490,32 @@ void run_gemv(benchmark::State &state, int variant, const char *name) {
   });
 }
 
-void run_gemm(benchmark::State &state, int variant, const char *name) {
+void run_gemm(benchmark::State &state, int variant, const char *name, bool half_out) {
   guarded(state, [&] {
     const size_t M = state.range(0), N = state.range(1), K = state.range(2);
-    const float alpha = 1.1f, beta = 1.2f;  // the reference's values (src/gemm/wmma.cu:575-576)
-    DeviceBuffer A(M * K * 2), B(N * K * 2), C(M * N * 4), D(M * N * 4);
+    // the reference's values (src/gemm/wmma.cu:575-576), rounded to fp16 for the fp16-output
+    // benchmark as there (src/gemm/wmma.cu:679-680)
+    const float alpha = half_out ? half_to_float(float_to_half(1.1f)) : 1.1f, beta = half_out ? half_to_float(float_to_half(1.2f)) : 1.2f;
+    const size_t out_size = half_out ? 2 : 4;  // bytes per element of C and D
+    const auto gemm = half_out ? tcu_gemm_f16_f16 : tcu_gemm_f16_f32;
+    DeviceBuffer A(M * K * 2), B(N * K * 2), C(M * N * out_size), D(M * N * out_size);
     TCU_CHECK(tcu_generate_f16(A.get(), M * K, flags().seed, TCU_DIST_NORMAL, 0, nullptr));
     TCU_CHECK(tcu_generate_f16(B.get(), N * K, flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
-    PRINT_IF_ERROR(hipMemset(C.get(), 0, M * N * 4));
-    TCU_CHECK(tcu_gemm_f16_f32(A.get(), B.get(), C.get(), D.get(), M, N, K, alpha, beta, variant, nullptr));
+    PRINT_IF_ERROR(hipMemset(C.get(), 0, M * N * out_size));
+    TCU_CHECK(gemm(A.get(), B.get(), C.get(), D.get(), M, N, K, alpha, beta, variant, nullptr));
     PRINT_IF_ERROR(hipDeviceSynchronize());
     if (should_verify(M * K) && M * N * K <= ((size_t)1 << 31)) {
       std::vector<uint16_t> hA(M * K), hB(N * K);
       std::vector<float> hD(M * N);
       PRINT_IF_ERROR(hipMemcpy(hA.data(), A.get(), M * K * 2, hipMemcpyDeviceToHost));
       PRINT_IF_ERROR(hipMemcpy(hB.data(), B.get(), N * K * 2, hipMemcpyDeviceToHost));
-      PRINT_IF_ERROR(hipMemcpy(hD.data(), D.get(), M * N * 4, hipMemcpyDeviceToHost));
+      if (half_out) {
+        std::vector<uint16_t> raw(M * N);
+        PRINT_IF_ERROR(hipMemcpy(raw.data(), D.get(), M * N * 2, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < M * N; i++) hD[i] = half_to_float(raw[i]);
+      } else {
+        PRINT_IF_ERROR(hipMemcpy(hD.data(), D.get(), M * N * 4, hipMemcpyDeviceToHost));
+      }
       for (size_t m = 0; m < M; m++)
         for (size_t n = 0; n < N; n++) {
           double s = 0;
@@ -509,7 +527,7 @@ void run_gemm(benchmark::State &state, int variant, const char *name) {
     EventPair ev;
     for (auto _ : state) {
       ev.start();
-      TCU_CHECK(tcu_gemm_f16_f32(A.get(), B.get(), C.get(), D.get(), M, N, K, alpha, beta, variant, nullptr));
+      TCU_CHECK(gemm(A.get(), B.get(), C.get(), D.get(), M, N, K, alpha, beta, variant, nullptr));
       const float ms = ev.stop_ms();
       state.PauseTiming();
       state.SetIterationTime(ms / 1000);
@@ -520,6 +538,107 @@ void run_gemm(benchmark::State &state, int variant, const char *name) {
                            {"K", (double)K},
                            {"flops", {state.iterations() * 2.0 * M * N * K, benchmark::Counter::kAvgThreadsRate}},
                            {"mfma_peak_fraction", {state.iterations() * 2.0 * M * N * K / 2.5e15, benchmark::Counter::kAvgThreadsRate}}});
+  });
+}
+
+// ---------------------------------------------------------------------------------------
+// accuracy comparisons (reference src/gemm/accuracy.cu:178-275, src/gemv/accuracy.cu:215-330):
+// fp32 values uniform in [0, 1) are narrowed to fp16 on the device, two computations of the
+// same product are compared element by element under the reference's rule (ratio within
+// 1.0001 and difference within 1e-5), and the number of violations is reported as a counter.
+// ---------------------------------------------------------------------------------------
+static void fill_uniform01_f32(std::vector<float> &v, uint64_t seed) {
+  for (size_t i = 0; i < v.size(); i++) {
+    uint64_t z = seed + (i + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    v[i] = (float)(z >> 40) * (1.0f / 16777216.0f);
+  }
+}
+struct Agreement {
+  size_t errors = 0;
+  double max_abs = 0, max_rel = 0;
+  void add(float v1, float v2) {
+    const double d = std::fabs((double)v1 - (double)v2);
+    if (v1 / v2 > 1.0001 || v2 / v1 > 1.0001 || d > 1e-5) errors++;
+    max_abs = std::max(max_abs, d);
+    const double m = std::max(std::fabs((double)v1), std::fabs((double)v2));
+    if (m > 0) max_rel = std::max(max_rel, d / m);
+  }
+};
+// narrows `host` to fp16 on the device (the reference's convertFp32ToFp16 step)
+static void upload_as_f16(const std::vector<float> &host, DeviceBuffer &f16) {
+  DeviceBuffer f32(host.size() * 4);
+  PRINT_IF_ERROR(hipMemcpy(f32.get(), host.data(), host.size() * 4, hipMemcpyHostToDevice));
+  TCU_CHECK(tcu_convert_f32_to_f16(f16.get(), f32.get(), host.size(), nullptr));
+  PRINT_IF_ERROR(hipDeviceSynchronize());
+}
+
+void run_gemm_accuracy(benchmark::State &state, const char *name) {
+  guarded(state, [&] {
+    const size_t M = state.range(0), N = state.range(1), K = state.range(2);
+    if (M * N > ((size_t)1 << 26)) throw unsupported(std::string(name) + ": outputs beyond 2^26 elements are not compared on the host");
+    const float alpha = 1.1f, beta = 1.2f;
+    std::vector<float> hA(M * K), hB(N * K), hC(M * N);
+    fill_uniform01_f32(hA, flags().seed);
+    fill_uniform01_f32(hB, flags().seed + 1);
+    fill_uniform01_f32(hC, flags().seed + 2);
+    DeviceBuffer A(M * K * 2), B(N * K * 2), C(M * N * 4), D_direct(M * N * 4), D_tiled(M * N * 4);
+    upload_as_f16(hA, A);
+    upload_as_f16(hB, B);
+    PRINT_IF_ERROR(hipMemcpy(C.get(), hC.data(), M * N * 4, hipMemcpyHostToDevice));
+    // first: one tile per wave straight from global memory; second: the LDS-tiled kernel
+    TCU_CHECK(tcu_gemm_f16_f32(A.get(), B.get(), C.get(), D_direct.get(), M, N, K, alpha, beta, TCU_VARIANT_MFMA_16N, nullptr));
+    EventPair ev;
+    for (auto _ : state) {
+      ev.start();
+      TCU_CHECK(tcu_gemm_f16_f32(A.get(), B.get(), C.get(), D_tiled.get(), M, N, K, alpha, beta, TCU_VARIANT_AUTO, nullptr));
+      const float ms = ev.stop_ms();
+      state.PauseTiming();
+      state.SetIterationTime(ms / 1000);
+      state.ResumeTiming();
+    }
+    std::vector<float> h1(M * N), h2(M * N);
+    PRINT_IF_ERROR(hipMemcpy(h1.data(), D_direct.get(), M * N * 4, hipMemcpyDeviceToHost));
+    PRINT_IF_ERROR(hipMemcpy(h2.data(), D_tiled.get(), M * N * 4, hipMemcpyDeviceToHost));
+    Agreement ag;
+    for (size_t i = 0; i < M * N; i++) ag.add(h1[i], h2[i]);
+    state.counters.insert({{"M", (double)M}, {"N", (double)N}, {"K", (double)K}, {"errors", (double)ag.errors}, {"max_abs_diff", ag.max_abs}, {"max_rel_diff", ag.max_rel}});
+  });
+}
+
+void run_gemv_accuracy(benchmark::State &state, const char *name) {
+  guarded(state, [&] {
+    const size_t M = state.range(0), K = state.range(1);
+    if (M * K > ((size_t)1 << 28)) throw unsupported(std::string(name) + ": matrices beyond 2^28 elements are not multiplied on the host");
+    const float alpha = 1.0f, beta = 0.0f;
+    std::vector<float> hA(M * K), hx(K);
+    fill_uniform01_f32(hA, flags().seed);
+    fill_uniform01_f32(hx, flags().seed + 1);
+    DeviceBuffer A(M * K * 2), x(K * 2), y(M * 4);
+    upload_as_f16(hA, A);
+    upload_as_f16(hx, x);
+    PRINT_IF_ERROR(hipMemset(y.get(), 0, M * 4));
+    EventPair ev;
+    for (auto _ : state) {  // first: the 16-wide MFMA form on the fp16 operands
+      ev.start();
+      TCU_CHECK(tcu_gemv_f16_f32(A.get(), x.get(), y.get(), M, K, alpha, beta, TCU_VARIANT_MFMA_16N, nullptr));
+      const float ms = ev.stop_ms();
+      state.PauseTiming();
+      state.SetIterationTime(ms / 1000);
+      state.ResumeTiming();
+    }
+    std::vector<float> got(M);
+    PRINT_IF_ERROR(hipMemcpy(got.data(), y.get(), M * 4, hipMemcpyDeviceToHost));
+    // second: a single-precision product of the fp32 operands (the reference calls cublasSgemv)
+    Agreement ag;
+    for (size_t m = 0; m < M; m++) {
+      float s = 0.0f;
+      for (size_t k = 0; k < K; k++) s += hA[m * K + k] * hx[k];
+      ag.add(alpha * s, got[m]);
+    }
+    state.counters.insert({{"M", (double)M}, {"N", (double)K}, {"errors", (double)ag.errors}, {"max_abs_diff", ag.max_abs}, {"max_rel_diff", ag.max_rel}});
   });
 }
 

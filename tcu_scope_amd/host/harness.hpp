@@ -92,8 +92,13 @@ void run_seg_scan_offsets(benchmark::State &state, const char *name);
 void run_seg_scan(benchmark::State &state, int variant, int tiles_per_wave, int waves_per_block, bool with_totals, const char *name);
 void run_full_reduce(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
 void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
-void run_gemv(benchmark::State &state, int variant, const char *name);
-void run_gemm(benchmark::State &state, int variant, const char *name);
+// half_out: y (GEMV) or C and D (GEMM) in fp16, the reference's H* benchmarks
+void run_gemv(benchmark::State &state, int variant, const char *name, bool half_out = false);
+void run_gemm(benchmark::State &state, int variant, const char *name, bool half_out = false);
+// two computations of one product compared under the reference's agreement rule
+// (src/gemm/accuracy.cu:259-268, src/gemv/accuracy.cu:314-323); counters: errors, max_abs_diff, max_rel_diff
+void run_gemm_accuracy(benchmark::State &state, const char *name);
+void run_gemv_accuracy(benchmark::State &state, const char *name);
 // the reference's CPU verification loop (fp32 running sum per segment, fp16 result) timed on
 // `threads` host threads; scan = prefix sums instead of totals
 void run_cpu_segmented(benchmark::State &state, bool scan, int threads);

@@ -188,19 +188,22 @@ void check_blas(rocblas_status s, const char *what) {
 }  // namespace
 
 // D (M x N row-major) = alpha * A (M x K row-major) * B (K x N column-major) + beta * C, the
-// layouts of tcu_gemm_f16_f32.  In rocBLAS's column-major terms: D^T (N x M) = op(B) * A'.
-static void CUBLAS_WMMA_GEMM(benchmark::State &state) {
+// layouts of tcu_gemm_f16_f32 / tcu_gemm_f16_f16 (half_out: C and D in fp16, as the reference's
+// CUBLAS_WMMA_HGEMM, src/gemm/cublas.cu:623; fp32 accumulation either way).  In rocBLAS's
+// column-major terms: D^T (N x M) = op(B) * A'.
+static void blas_gemm(benchmark::State &state, bool half_out) {
   guarded(state, [&] {
     const size_t M = state.range(0), N = state.range(1), K = state.range(2);
     const float alpha = 1.1f, beta = 1.2f;
-    DeviceBuffer A(M * K * 2), B(N * K * 2), C(M * N * 4), D(M * N * 4);
+    const size_t out_size = half_out ? 2 : 4;
+    const rocblas_datatype out_type = half_out ? rocblas_datatype_f16_r : rocblas_datatype_f32_r;
+    DeviceBuffer A(M * K * 2), B(N * K * 2), C(M * N * out_size), D(M * N * out_size);
     TCU_CHECK(tcu_generate_f16(A.get(), M * K, harness::flags().seed, TCU_DIST_NORMAL, 0, nullptr));
     TCU_CHECK(tcu_generate_f16(B.get(), N * K, harness::flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
-    PRINT_IF_ERROR(hipMemset(C.get(), 0, M * N * 4));
+    PRINT_IF_ERROR(hipMemset(C.get(), 0, M * N * out_size));
     auto run = [&] {
       check_blas(rocblas_gemm_ex(blas(), rocblas_operation_transpose, rocblas_operation_none, (rocblas_int)N, (rocblas_int)M, (rocblas_int)K, &alpha, B.get(), rocblas_datatype_f16_r, (rocblas_int)K, A.get(),
-                                 rocblas_datatype_f16_r, (rocblas_int)K, &beta, C.get(), rocblas_datatype_f32_r, (rocblas_int)N, D.get(), rocblas_datatype_f32_r, (rocblas_int)N, rocblas_datatype_f32_r,
-                                 rocblas_gemm_algo_standard, 0, 0),
+                                 rocblas_datatype_f16_r, (rocblas_int)K, &beta, C.get(), out_type, (rocblas_int)N, D.get(), out_type, (rocblas_int)N, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0),
                  "rocblas_gemm_ex");
     };
     run();
@@ -213,6 +216,9 @@ static void CUBLAS_WMMA_GEMM(benchmark::State &state) {
                            {"mfma_peak_fraction", {state.iterations() * 2.0 * M * N * K / 2.5e15, benchmark::Counter::kAvgThreadsRate}}});
   });
 }
+static void CUBLAS_WMMA_GEMM(benchmark::State &state) { blas_gemm(state, false); }
+static void CUBLAS_WMMA_HGEMM(benchmark::State &state) { blas_gemm(state, true); }
+BENCHMARK(CUBLAS_WMMA_HGEMM)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUBLAS_WMMA_GEMM)->Apply(GemmArgs)->UseManualTime();
 
 // y (M) = alpha * A (M x K row-major) x + beta * y as a one-column GEMM (fp16 in, fp32 out)

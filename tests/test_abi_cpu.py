@@ -51,6 +51,10 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.tcu_full_scan_f16(None, None, 1 << 20, None, None, 0, 0, 0, None) == 1
     assert lib.tcu_gemv_f16_f32(p, p, p, 4, 8, 1.0, 0.0, 5, None) == 2
     assert lib.tcu_gemm_f16_f32(p, p, None, p, 64, 64, 64, 1.0, 0.0, 8, None) == 2  # LDS kernel needs multiples of 128
+    assert lib.tcu_gemv_f16_f16(p, p, p, 4, 8, 1.0, 0.0, 5, None) == 2
+    assert lib.tcu_gemm_f16_f16(p, p, None, p, 64, 64, 64, 1.0, 0.0, 8, None) == 2
+    assert lib.tcu_gemm_f16_f16(p, p, None, p, 64, 64, 64, 1.0, 1.0, 0, None) == 1 and "tcu_gemm_f16_f16" in err()  # beta != 0 needs C
+    assert lib.tcu_gemv_f16_f16(None, p, p, 4, 8, 1.0, 0.0, 0, None) == 1 and "tcu_gemv_f16_f16" in err()
     assert lib.tcu_seg_reduce_offsets_f16(p, p, 0, p, p, 32, 0, None) == 0      # no segments: no launch
     assert lib.tcu_seg_reduce_offsets_f16(p, p, 4, p, p, 16, 0, None) == 1 and "offset_bits" in err()
     assert lib.tcu_seg_reduce_offsets_f16(p, p, 4, None, p, 64, 0, None) == 1 and "null" in err()

@@ -36,6 +36,8 @@ def emu():
     L.emu_full_scan_f16.argtypes = [vp, vp, sz, vp, ctypes.POINTER(sz), ci, sz, ci]
     L.emu_gemv_f16_f32.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci]
     L.emu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
+    L.emu_gemv_f16_f16.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci]
+    L.emu_gemm_f16_f16.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
     L.emu_set_option.argtypes = [ctypes.c_char_p, ci]
     L.emu_seg_reduce_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz]
     L.emu_seg_scan_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz]
@@ -249,6 +251,12 @@ def test_gemv_gemm_and_generator(emu, oracle):
                 assert K % 8
                 continue
             assert rc == 0 and oracle.check_f32_rel(y[:M], oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0), 1e-4, float(np.sqrt(K)))[0] == 0, (M, K, v)
+            # fp16 y: same sums, rounded once
+            y0h = y0.astype(np.float16)
+            yh = copy_in(y0h.view(np.uint16))
+            rc = emu.emu_gemv_f16_f16(Ai.ctypes.data, xi.ctypes.data, yh.ctypes.data, M, K, 1.5, -0.5, v)
+            ref = oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0h.astype(np.float32))
+            assert rc == 0 and oracle.check_f16(yh[:M], ref, K)[0] == 0, (M, K, v)
     for M, N, K in ((128, 128, 64), (256, 512, 64), (64, 32, 48), (33, 17, 20)):
         A, B = oracle.generate_f16(M * K, 5, oracle.DIST_SMALLINT), oracle.generate_f16(N * K, 6, oracle.DIST_SMALLINT)
         C0 = (np.arange(M * N) % 7).astype(np.float32)
@@ -259,6 +267,11 @@ def test_gemv_gemm_and_generator(emu, oracle):
             if rc == 2:
                 continue
             assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A, B, M, N, K, 2.0, 3.0, C0)), (M, N, K, v)
+            # fp16 C and D: the fp32 result is exact for these inputs, so D is its one rounding
+            Ch = copy_in(C0.astype(np.float16).view(np.uint16))
+            Dh = aligned(M * N, np.uint16, 0x7e00)
+            rc = emu.emu_gemm_f16_f16(Ai.ctypes.data, Bi.ctypes.data, Ch.ctypes.data, Dh.ctypes.data, M, N, K, 1.5, 3.0, v)
+            assert rc == 0 and np.array_equal(Dh.reshape(M, N), oracle.gemm_f64(A, B, M, N, K, 1.5, 3.0, C0).astype(np.float16).view(np.uint16)), (M, N, K, v)
     # the 256 x 256 tile kernels: register-staged (K step 32 / 64, every prefetch depth that
     # divides the step count) and direct-to-LDS (3 and 4 buffers)
     M, N, K = 256, 256, 192
@@ -273,6 +286,9 @@ def test_gemv_gemm_and_generator(emu, oracle):
             D = aligned(M * N, np.float32, -777)
             rc = emu.emu_gemm_f16_f32(Ai.ctypes.data, Bi.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), ref), (direct_lds, bk64, depth)
+            Dh = copy_in(C0.astype(np.float16).view(np.uint16))  # in place: C == D
+            rc = emu.emu_gemm_f16_f16(Ai.ctypes.data, Bi.ctypes.data, Dh.ctypes.data, Dh.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
+            assert rc == 0 and np.array_equal(Dh.reshape(M, N), ref.astype(np.float16).view(np.uint16)), (direct_lds, bk64, depth)
     finally:
         for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4)):
             emu.emu_set_option(name, val)

@@ -114,6 +114,14 @@ def test_gemv(tcu, oracle, M, K):
             assert bad == 0, (v.name, alpha, beta, bad, worst, first)
             bad, worst, first = oracle.check_f32_rel(y.cpu().numpy(), ref, 1e-4, float(np.sqrt(K)))
             assert bad == 0, ("tight", v.name, alpha, beta, bad, worst, first)
+            # fp16 y (tcu_gemv_f16_f16): the same fp32 sums, rounded once
+            y0h = y0.astype(np.float16)
+            yh = torch.from_numpy(y0h.copy()).cuda()
+            tcu.gemv(Ad, xd, alpha, beta, y=yh, variant=v)
+            torch.cuda.synchronize()
+            ref = oracle.gemv_f64(A, x, M, K, alpha, beta, y0h.astype(np.float32))
+            bad, worst, first = oracle.check_f16(yh.cpu().numpy().view(np.uint16), ref, K, ulps=1.0, abs_per_sqrt=1e-4)
+            assert bad == 0, ("fp16 y", v.name, alpha, beta, bad, worst, first)
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 256), (512, 384, 160), (96, 64, 48), (33, 17, 20)])
@@ -141,6 +149,17 @@ def test_gemm_small_exact_and_normal(tcu, oracle, M, N, K):
                 else:
                     bad, worst, first = oracle.check_f32_rel(got, ref, 1e-2, float(np.sqrt(K)))
                     assert bad == 0, (v.name, alpha, beta, bad, worst, first)
+                # fp16 C and D (tcu_gemm_f16_f16)
+                Ch = torch.from_numpy(C0.astype(np.float16)).cuda().view(M, N)
+                Dh = tcu.gemm(Ad, Bd, alpha, beta, C=Ch, variant=v)
+                torch.cuda.synchronize()
+                assert Dh.dtype == torch.float16
+                goth = Dh.cpu().numpy()
+                if exact:  # the fp32 result is exact, so the output is its one rounding to fp16
+                    assert np.array_equal(goth.view(np.uint16), ref.astype(np.float16).view(np.uint16)), ("fp16", v.name, alpha, beta)
+                else:
+                    bad, worst, first = oracle.check_f16(goth.view(np.uint16), ref, K, ulps=1.0, abs_per_sqrt=1e-4)
+                    assert bad == 0, ("fp16", v.name, alpha, beta, bad, worst, first)
 
 
 def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
@@ -170,6 +189,13 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
                 D = tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd, variant=tcu.Variant.BLOCK_LDS)  # in place
                 torch.cuda.synchronize()
                 assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("in place", K, direct_lds, bk64, depth)
+                # the same kernels with fp16 C and D, out of place and in place
+                Dh = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS, out_dtype=torch.float16)
+                Ch = torch.from_numpy(C0.astype(np.float16)).cuda().view(M, N)
+                tcu.gemm(Ad, Bd, 2.0, -1.0, C=Ch, out=Ch, variant=tcu.Variant.BLOCK_LDS)
+                torch.cuda.synchronize()
+                assert np.array_equal(Dh.cpu().numpy().view(np.uint16), ref0.astype(np.float16).view(np.uint16)), ("fp16", K, direct_lds, bk64, depth)
+                assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("fp16 in place", K, direct_lds, bk64, depth)
     finally:
         tcu.set_option("gemm_direct_lds", -1)
         tcu.set_option("gemm_bk64", 0)
@@ -191,3 +217,13 @@ def test_gemm_8192(tcu, oracle):
         ref = oracle.gemm_f64(A, B, M, N, K, row0=r, rows=1)
         bad, worst, first = oracle.check_f32_rel(D[r].cpu().numpy(), ref, 1e-2, float(np.sqrt(K)))
         assert bad == 0, (r, bad, worst, first)
+    # fp16 C and D with the benchmark's alpha and beta (reference src/gemm/wmma.cu:679-680)
+    Ch = tcu.generate(M * N, 13, tcu.Dist.NORMAL).view(M, N)
+    C32 = to_host(Ch).ravel().view(np.float16).astype(np.float32)
+    Dh = tcu.gemm(Ad, Bd, 1.1, 1.2, C=Ch)
+    torch.cuda.synchronize()
+    assert Dh.dtype == torch.float16
+    for r in rows[::2]:
+        ref = oracle.gemm_f64(A, B, M, N, K, 1.1, 1.2, C32, row0=r, rows=1)
+        bad, worst, first = oracle.check_f16(Dh[r].cpu().numpy().view(np.uint16), ref, K, ulps=1.0, abs_per_sqrt=1e-4)
+        assert bad == 0, ("fp16", r, bad, worst, first)

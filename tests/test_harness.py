@@ -49,6 +49,13 @@ def test_benchmark_names_follow_the_reference_grammar():
         "CUB_FULL_REDUCTION/num_elements:1073741824/manual_time",
         "CUB_FULL_PREFIXSUM/num_elements:1073741824/manual_time",
         "CUBLAS_WMMA_GEMM/M:8192/N:8192/K:8192/manual_time",
+        # fp16-output twins (reference src/gemm/wmma.cu:777, wmma_naive.cu:340, src/gemv/wmma_naive.cu:358, src/gemm/cublas.cu:623)
+        "CUDA_WMMA_HGEMM/M:8192/N:8192/K:8192/manual_time",
+        "CUDA_WMMA_HGEMM_NAIVE/M:8192/N:8192/K:8192/manual_time",
+        "CUDA_WMMA_HGEMV_NAIVE/M:16384/N:16384/manual_time",
+        "CUBLAS_WMMA_HGEMM/M:8192/N:8192/K:8192/manual_time",
+        "CUDA_WMMA_GEMM_ACCURACY/M:1024/N:1024/K:1024/manual_time",
+        "CUDA_WMMA_GEMV_ACCURACY/M:4096/N:4096/manual_time",
     ]:
         assert n in have, n
     # the filter is a regular expression over those names
@@ -62,9 +69,9 @@ def test_harness_runs_verifies_and_reports(tmp_path):
     filt = ("(CUDA_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16<1, 4>|256<1, 4>|16N<4>|256N<4>|256N_BLOCK<4>)|CUB_(WARP|BLOCK)_SEGMENTED_(REDUCTION|PREFIXSUM)<(256, 16|512, 32, BLOCK_(SCAN|REDUCE)_RAKING)>"
             "|TCU_AUTO_SEGMENTED_(REDUCTION|PREFIXSUM))/.*num_elements:4194304/"
             "|CUDA_WMMA_FULL_(REDUCTION_(2KERS_BASE_16|ATOMIC_W_BLOCK_SYNC)|PREFIXSUM_(3KERS|CG))<8 \\* 256, 4>/num_elements:4194304/"
-            "|CUDA_WMMA_GEM[MV](_NAIVE)?/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/"
+            "|CUDA_WMMA_H?GEM[MV](_NAIVE)?/M:512/|TCU_WAVE_H?GEMV/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/"
             "|CUDA_UNSAFE_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16N<4>|256N_BLOCK<4>)/.*num_elements:4194304/"
-            "|CUB_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/|CUB_DEVICE_SEGMENTED_REDUCTION/.*segment_size:256/num_elements:4194304/|CUBLAS_(WMMA_GEMM|GEMV)/M:512/")
+            "|CUB_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/|CUB_DEVICE_SEGMENTED_REDUCTION/.*segment_size:256/num_elements:4194304/|CUBLAS_(WMMA_H?GEMM|GEMV)/M:512/")
     p = subprocess.run([BENCH, f"--benchmark_filter={filt}", "--benchmark_min_time=0.02", f"--benchmark_out={out}", "--benchmark_out_format=json", "--tcu_verify=all", "--v=1"],
                        capture_output=True, text=True, timeout=300)
     assert p.returncode == 0, p.stdout + p.stderr
@@ -75,6 +82,18 @@ def test_harness_runs_verifies_and_reports(tmp_path):
     for r in rows:
         assert r["iterations"] >= 1 and r["real_time"] > 0 and r["flops"] > 0, r
         assert r["name"].endswith("/manual_time")
+    # the accuracy comparisons report agreement counters instead of rates
+    out2 = tmp_path / "acc.json"
+    p = subprocess.run([BENCH, "--benchmark_filter=CUDA_WMMA_GEM[MV]_ACCURACY/M:(512|96)/", "--benchmark_min_time=0.01", f"--benchmark_out={out2}", "--benchmark_out_format=json"],
+                       capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0 and "ERROR OCCURRED" not in p.stdout, p.stdout + p.stderr
+    acc = {r["name"]: r for r in json.loads(out2.read_text())["benchmarks"]}
+    assert len(acc) == 4
+    for name, r in acc.items():
+        # GEMM: two kernels that add the same fp32 products in different groupings; GEMV: fp16-rounded operands
+        # against the fp32 originals (relative error of a sum of positive terms stays near 2^-11)
+        assert r["max_rel_diff"] < (1e-5 if "GEMM" in name else 1e-3), r
+        assert r["errors"] >= 0 and r["max_abs_diff"] >= 0
     # precondition failures surface as skipped benchmarks, as in the reference
     p = subprocess.run([BENCH, "--benchmark_filter=CUDA_WMMA_FULL_REDUCTION_2KERS_BASE_16<16 \\* 256, 1>/num_elements:4096/", "--benchmark_min_time=0.01"], capture_output=True, text=True, timeout=120)
     assert p.returncode == 0 and "ERROR OCCURRED" not in p.stdout  # 4096 is a multiple of 4096: runs
