@@ -91,8 +91,9 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step
  *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more)
  *   "gemm_big_tiles"  0/1, default 1: 256 x 256 block tiles where M and N allow
- *   "gemm_direct_lds" -1/0/3/4/64, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
- *                     buffers; 64 = K step 64, two buffers; 0 = register-staged kernel; -1 = chosen by shape
+ *   "gemm_direct_lds" -1/0/3/4/64/65, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
+ *                     buffers; 64 = K step 64, two buffers; 65 = K step 64, three buffers for A and two for B;
+ *                     0 = register-staged kernel; -1 = 65 where K is a multiple of 64, else 4
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
  * Unknown names return TCU_ERR_INVALID_ARG. */

@@ -36,7 +36,7 @@ struct Options {
   bool static_order = false;
   bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
-  int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 0: register-staged kernel; -1: by shape
+  int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
@@ -772,14 +772,15 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
   if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && options().gemm_big_tiles) {
     const size_t grid = (M / kGemmBigBM) * (N / kGemmBigBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    // measured: the transfer kernel is the faster one (1.15-1.22 vs 1.0-1.1 PFLOP/s at 8192^3)
-    // except when rows are a multiple of 32 KiB apart (K % 16384 == 0: 0.85 vs 0.98 PFLOP/s);
-    // its K-step-64 form (whole 128-byte lines per row and transfer, but only two LDS buffers)
-    // gains 5-6 % up to 8192 x 8192 outputs (1223 vs 1154 at 8192^3, 1096 vs 1040 at 4096^3)
-    // and loses 2 % at 16384 x 16384
-    const int direct_lds = options().gemm_direct_lds >= 0 ? options().gemm_direct_lds : (K % 16384 == 0 ? 0 : (K % 64 == 0 && M * N <= (size_t)8192 * 8192 ? 64 : 4));
+    // measured (2048^3 ... 16384^3, K = 4096 ... 16448): the transfer kernels with K step 64 (whole
+    // 128-byte lines per row and transfer) beat the K-step-32 and the register-staged forms at
+    // every size (8192^3: 1305 vs 1225 vs 1128 TFLOP/s), and of the two the one with three A and
+    // two B buffers is equal or faster everywhere (16384^3: 1313 vs 1083)
+    const int direct_lds = options().gemm_direct_lds >= 0 ? options().gemm_direct_lds : (K % 64 == 0 ? 65 : 4);
     if (direct_lds > 0 && K <= ((size_t)1 << 22)) {
-      if (direct_lds == 64 && K % 64 == 0)
+      if (direct_lds == 65 && K % 64 == 0)
+        launch(gemm_dlds_a3b2_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      else if (direct_lds >= 64 && K % 64 == 0)
         launch(gemm_dlds_kernel<64, 2, OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       else if (direct_lds == 3)
         launch(gemm_dlds_kernel<32, 3, OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);

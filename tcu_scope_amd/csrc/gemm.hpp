@@ -353,8 +353,11 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
 // are read under the first 8 MFMAs and up to 8 transfers of step s + NBUF - 1 (into the
 // buffer of step s - 1, free since that step's barrier) are issued under the other 8;
 // before the last substep a wave waits for its own transfers of step s + 1, the barrier
-// publishes everybody's, and the fragments of step s + 1, substep 0, are read while the
-// last 16 MFMAs of step s run.
+// publishes everybody's, the fragments of step s + 1, substep 0, are read while the last 16
+// MFMAs of step s run, and the first half of the transfers of step s + NBUF already go out
+// into the buffer that barrier has just freed (measured: every substep of extra flight time
+// is worth 2-7 %; issuing more than half of a step's transfers in that one substep loses it
+// again).
 template <int BK, int NBUF, typename OUT>
 __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
   constexpr int ROWH = BK;                           // halves per LDS row
@@ -365,7 +368,8 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
   constexpr int OPH = kGemmBigBM * ROWH;             // halves per operand per stage
   constexpr int P = NBUF - 1;                        // prefetch distance in steps
   constexpr int TPW = kGemmBigBM / RPT / 4;          // transfer instructions per wave, operand and step
-  static_assert((BK == 32 || BK == 64) && 2 * TPW <= 8 * (SUB - 1) && 2 * TPW * (P - 1) <= 63, "transfers must fit the substeps and the counter");
+  constexpr int EARLY = TPW;                         // transfers of a step issued one substep ahead of the others
+  static_assert((BK == 32 || BK == 64) && EARLY <= 8 && 2 * TPW - EARLY <= 8 * (SUB - 1) && 2 * TPW * (P - 1) + EARLY <= 63, "transfers must fit the substeps and the counter");
   __shared__ __attribute__((aligned(1024))) half_t lds_a[NBUF][OPH];
   __shared__ __attribute__((aligned(1024))) half_t lds_b[NBUF][OPH];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -411,7 +415,9 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
   for (int d = 0; d < P; d++)
 #pragma unroll
     for (int x = 0; x < 2 * TPW; x++) issue((size_t)d, d, x);
-  wait_vector_loads<2 * TPW * (P - 1)>();
+#pragma unroll
+  for (int x = 0; x < EARLY; x++) issue((size_t)P, P, x);
+  wait_vector_loads<2 * TPW * (P - 1) + EARLY>();
   block_barrier_lds_only();
 
   // fragment of row r, k chunk kc: slot kc ^ f(r); rows of a lane differ by multiples of 32
@@ -454,7 +460,7 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
         sched_fence();
 #pragma unroll
         for (int t = 0; t < 8; t++) {
-          const int i = 2 + t / 4, j = t % 4, x = kk * 8 + t;
+          const int i = 2 + t / 4, j = t % 4, x = EARLY + kk * 8 + t;
           if (x < 2 * TPW) issue(s + P, fill, x);
           acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
           sched_fence();
@@ -469,8 +475,10 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
           fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[nxt][fa0 + i * 32 * ROWH + ko[0]]);
           fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[nxt][fb0 + i * 32 * ROWH + ko[0]]);
         }
+        // the buffer of step s is free from this barrier on: the first transfers of step
+        // s + NBUF go out here, one substep ahead of the rest
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 2; i++)
 #pragma unroll
           for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
 #pragma unroll
@@ -478,11 +486,157 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
           sched_group<kSchedDsRead, 1>();
           sched_group<kSchedMfma, 1>();
         }
-        sched_group<kSchedMfma, 8>();
         sched_fence();
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const int i = 2 + t / 4, j = t % 4;
+          if (t < EARLY) issue(s + NBUF, cur, t);
+          acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+          sched_fence();
+        }
       }
     }
     cur = nxt;
+  }
+  wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) gemm_store_tile(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 32, tile_n * kGemmBigBN + wn * 128 + j * 32, acc[i][j], lane, alpha, beta);
+}
+
+// M % 256 == 0, N % 256 == 0, K % 64 == 0, K <= 2^22; 256 threads.
+// gemm_dlds_kernel<64, 2> with the whole 160 KiB of LDS in use: three buffers for A, two for
+// B.  After the barrier of step s the B tile of step s + 2 goes out into the B buffer the
+// barrier has freed (all of it under the last 8 MFMAs of the step); the A tile of step s + 3
+// follows under substeps 0 and 1 of step s + 1, into the A buffer of step s.  Every transfer
+// then has at least a whole step (four substeps) of flight time, those of A almost two
+// (measured against gemm_dlds_kernel<64, 2>: +1.5-3 % at 8192^3, +7 % at 12288^3, +17-21 % at
+// 16384^3, where rows a multiple of 32 KiB apart make the loads slow; spreading the A tile
+// over substeps 0-2 or 1-2 instead measures the same, all of it in substep 0 1 % less).
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemm_dlds_a3b2_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+  constexpr int BK = 64, ROWH = BK, CPR = 8, RPT = 8, RS = 1, SUB = 4, NA = 3, NB = 2;
+  constexpr int OPH = kGemmBigBM * ROWH;     // halves per operand per stage
+  constexpr int TPW = kGemmBigBM / RPT / 4;  // transfer instructions per wave, operand and step (8)
+  __shared__ __attribute__((aligned(1024))) half_t lds_a[NA][OPH];
+  __shared__ __attribute__((aligned(1024))) half_t lds_b[NB][OPH];
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  size_t tile_m, tile_n;
+  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, &tile_m, &tile_n);
+  const size_t k_chunks = K / 8;
+  const size_t steps = K / BK;
+  uint32_t goff[TPW];
+#pragma unroll
+  for (int t = 0; t < TPW; t++) {
+    const int row = (wave * TPW + t) * RPT + lane / CPR;
+    const int chunk = (lane % CPR) ^ ((row >> RS) & (CPR - 1));
+    goff[t] = (uint32_t)(((size_t)row * k_chunks + chunk) * 16);
+  }
+  const char *ga = reinterpret_cast<const char *>(A + tile_m * kGemmBigBM * k_chunks);
+  const char *gb = reinterpret_cast<const char *>(B + tile_n * kGemmBigBN * k_chunks);
+  constexpr lds_addr_t STAGE = OPH * 2, TBYTES = 1024, STEPB = BK * 2;
+  const lds_addr_t ta = wave_uniform(lds_address_of(&lds_a[0][0]) + wave * TPW * TBYTES);
+  const lds_addr_t tb = wave_uniform(lds_address_of(&lds_b[0][0]) + wave * TPW * TBYTES);
+  // steps past the end: a harmless re-read of the last step into a free buffer
+  auto issue_a = [&](size_t step, int buf, int t) { load_chunk_to_lds(ga + (step < steps ? step : steps - 1) * STEPB, goff[t], ta + buf * STAGE + t * TBYTES); };
+  auto issue_b = [&](size_t step, int buf, int t) { load_chunk_to_lds(gb + (step < steps ? step : steps - 1) * STEPB, goff[t], tb + buf * STAGE + t * TBYTES); };
+
+  float16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+  // in flight at the first barrier: A0 B0 | A1 B1 (the wave's counter returns in issue order)
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_a(0, 0, t);
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_b(0, 0, t);
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_a(1, 1, t);
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_b(1, 1, t);
+  wait_vector_loads<2 * TPW>();
+  block_barrier_lds_only();
+
+  const int frow = lane & 31, khalf = lane >> 5, fsw = (frow >> RS) & (CPR - 1);
+  const int fa0 = (wm * 128 + frow) * ROWH, fb0 = (wn * 128 + frow) * ROWH;
+  int ko[SUB];
+#pragma unroll
+  for (int kk = 0; kk < SUB; kk++) ko[kk] = ((2 * kk + khalf) ^ fsw) * 8;
+  half8_t fa[2][4], fb[2][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[0][fa0 + i * 32 * ROWH + ko[0]]);
+    fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[0][fb0 + i * 32 * ROWH + ko[0]]);
+  }
+  int ca = 0, cb = 0;  // s % NA, s % NB
+  for (size_t s = 0; s < steps; s++) {
+    const int na = ca + 1 == NA ? 0 : ca + 1, nb = cb ^ 1;
+    const int fill_a = ca == 0 ? NA - 1 : ca - 1;  // A buffer of step s - 1 = of step s + 2
+#pragma unroll
+    for (int kk = 0; kk < SUB; kk++) {
+      const int p = kk & 1, q = p ^ 1;
+      if (kk < SUB - 1) {
+        sched_fence();
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + i * 32 * ROWH + ko[kk + 1]]);
+          fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[cb][fb0 + i * 32 * ROWH + ko[kk + 1]]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          sched_group<kSchedDsRead, 1>();
+          sched_group<kSchedMfma, 1>();
+        }
+        sched_fence();
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const int i = 2 + t / 4, j = t % 4;
+          if (kk < 2 && t % 2 == 0) issue_a(s + 2, fill_a, kk * 4 + t / 2);  // A tile of step s + 2: four transfers in each of substeps 0 and 1
+          acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+          sched_fence();
+        }
+      } else {
+        // own transfers of step s + 1 done (the A tile of step s + 2 may still fly), barrier,
+        // fragments of step s + 1, B tile of step s + 2 into the B buffer of step s
+        wait_vector_loads<TPW>();
+        block_barrier_lds_only();
+        sched_fence();
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + i * 32 * ROWH + ko[0]]);
+          fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[nb][fb0 + i * 32 * ROWH + ko[0]]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          sched_group<kSchedDsRead, 1>();
+          sched_group<kSchedMfma, 1>();
+        }
+        sched_fence();
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const int i = 2 + t / 4, j = t % 4;
+          issue_b(s + 2, cb, t);
+          acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+          sched_fence();
+        }
+      }
+    }
+    ca = na;
+    cb = nb;
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
 #pragma unroll

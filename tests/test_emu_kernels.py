@@ -280,7 +280,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
     Ai, Bi, Ci = copy_in(A), copy_in(B), copy_in(C0, np.float32)
     ref = oracle.gemm_f64(A, B, M, N, K, 1.5, 2.0, C0)
     try:
-        for direct_lds, bk64, depth in ((3, 0, 4), (4, 0, 4), (64, 0, 4), (0, 0, 1), (0, 0, 2), (0, 0, 3), (0, 0, 4), (0, 1, 1), (0, 1, 2)):
+        for direct_lds, bk64, depth in ((3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4), (0, 0, 1), (0, 0, 2), (0, 0, 3), (0, 0, 4), (0, 1, 1), (0, 1, 2)):
             for name, val in ((b"gemm_direct_lds", direct_lds), (b"gemm_bk64", bk64), (b"gemm_depth", depth)):
                 assert emu.emu_set_option(name, val) == 0
             D = aligned(M * N, np.float32, -777)

@@ -177,7 +177,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
             ref0 = oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0)
             ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
-            shapes = [(0, bk64, depth) for bk64 in (0, 1) for depth in (1, 2, 3, 4)] + [(3, 0, 4), (4, 0, 4), (64, 0, 4)]
+            shapes = [(0, bk64, depth) for bk64 in (0, 1) for depth in (1, 2, 3, 4)] + [(3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4)]
             for direct_lds, bk64, depth in shapes:
                 tcu.set_option("gemm_direct_lds", direct_lds)
                 tcu.set_option("gemm_bk64", bk64)
