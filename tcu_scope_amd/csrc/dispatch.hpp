@@ -468,6 +468,37 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
 
 template <typename OFF>
 inline int seg_scan_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_segments, const OFF *begin, const OFF *end, size_t expected, void *stream) {
+  // expected length of 2048 halves and more: a block per run of at most about 65536 halves of one
+  // segment, one 128-bit chunk per thread and round (256 ... 1024 threads); with more than one run
+  // per segment the runs' sums are taken first (fp32, stream-ordered temporary memory) and turned
+  // into carry-ins.  (Groups of 16 lanes walking a segment: 226-313 us for 2048 ... 32768 at
+  // N = 2^28 and milliseconds beyond, against 175-200 and 290 us this way.)
+  if (expected >= 2048) {
+    const int vec = aligned16(in) && aligned16(out) ? 1 : 0;
+    const bool ntl = options().nontemporal;
+    size_t slices = (expected + 65535) / 65536;
+    if (slices > 4096) slices = 4096;
+    unsigned threads = 256;
+    while (threads < 1024 && (size_t)threads * 16 < expected) threads *= 2;  // two rounds per block measure better than one
+    const size_t blocks = num_segments * slices;
+    if (blocks > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_offsets_f16: grid exceeds the launch limit");
+    float *sums = nullptr;
+    if (slices > 1) {
+      sums = static_cast<float *>(stream_alloc(blocks * sizeof(float), stream));
+      if (!sums) return fail(TCU_ERR_RUNTIME, "tcu_seg_scan_offsets_f16: no temporary device memory for the slice sums");
+      if (ntl)
+        launch(seg_scan_offsets_slice_sums_kernel<OFF, true>, (unsigned)blocks, threads, stream, in, sums, begin, end, (unsigned)slices, vec);
+      else
+        launch(seg_scan_offsets_slice_sums_kernel<OFF, false>, (unsigned)blocks, threads, stream, in, sums, begin, end, (unsigned)slices, vec);
+      launch(slice_prefix_kernel, (unsigned)num_segments, 64u, stream, sums, (unsigned)slices);
+    }
+    if (ntl)
+      launch(seg_scan_offsets_sliced_kernel<OFF, true>, (unsigned)blocks, threads, stream, in, out, static_cast<const float *>(sums), begin, end, (unsigned)slices, vec);
+    else
+      launch(seg_scan_offsets_sliced_kernel<OFF, false>, (unsigned)blocks, threads, stream, in, out, static_cast<const float *>(sums), begin, end, (unsigned)slices, vec);
+    if (sums) stream_free(sums, stream);
+    return TCU_OK;
+  }
   // lanes per segment: about one 128-bit chunk per lane and round for the expected length, at most 16
   int g_log2 = 4;
   if (expected) {

@@ -385,4 +385,120 @@ __global__ __launch_bounds__(256) void seg_scan_offsets_kernel(const uint16_t *i
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Long segments given by offsets: `slices` blocks share a segment.  The aligned 128-bit
+// chunks a segment touches are split into `slices` equal runs; pass 1 writes the fp32 sum of
+// every run, pass 2 turns the sums of a segment into exclusive prefixes (in place), pass 3
+// scans every run with its prefix as the carry-in.  Six bytes of traffic per element where
+// the short-segment kernel moves four, but every segment is spread over the whole chip.
+// ---------------------------------------------------------------------------------------
+struct OffsetsSlice {
+  size_t b, e;        // the segment, in halves (b == e when empty)
+  size_t c_lo, c_hi;  // the slice's aligned chunks
+};
+template <typename OFF>
+TCU_DEVICE OffsetsSlice offsets_slice(const OFF *__restrict__ begin, const OFF *__restrict__ end, size_t seg, size_t p, unsigned slices) {
+  OffsetsSlice s{0, 0, 0, 0};
+  const OFF ob = begin[seg], oe = end[seg];
+  if (oe > ob) {
+    s.b = (size_t)ob;
+    s.e = (size_t)oe;
+    const size_t c_first = s.b / 8, c_end = (s.e + 7) / 8;
+    const size_t per = (c_end - c_first + slices - 1) / slices;
+    s.c_lo = c_first + p * per;
+    s.c_hi = s.c_lo + per;
+    if (s.c_lo > c_end) s.c_lo = c_end;
+    if (s.c_hi > c_end) s.c_hi = c_end;
+  }
+  return s;
+}
+// the chunk's halves that lie inside [b, e), others zero
+template <bool NT>
+TCU_DEVICE half8_t offsets_masked_chunk(const uint16_t *in, size_t c, size_t b, size_t e, int vector, bool *full) {
+  const size_t lo = c * 8;
+  *full = vector && lo >= b && lo + 8 <= e;
+  if (*full) return load_chunk<NT>(reinterpret_cast<const half8_t *>(in) + c);
+  half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+    if (lo + i >= b && lo + i < e) v[i] = __builtin_bit_cast(half_t, in[lo + i]);
+  return v;
+}
+
+template <typename OFF, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void seg_scan_offsets_slice_sums_kernel(const uint16_t *__restrict__ in, float *__restrict__ sums, const OFF *__restrict__ begin, const OFF *__restrict__ end,
+                                                                                unsigned slices, int vector) {
+  __shared__ float wave_total[kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const OffsetsSlice s = offsets_slice(begin, end, blockIdx.x / slices, blockIdx.x % slices, slices);
+  float acc = 0.0f;
+  for (size_t c = s.c_lo + threadIdx.x; c < s.c_hi; c += blockDim.x) {
+    bool full;
+    acc = sum8(offsets_masked_chunk<NT>(in, c, s.b, s.e, vector, &full), acc);
+  }
+  acc = lane_group_sum<6>(acc);
+  if (lane == 63) wave_total[wave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.0f;
+    for (unsigned w = 0; w < (blockDim.x >> 6); w++) t += wave_total[w];
+    sums[blockIdx.x] = t;
+  }
+}
+
+// sums[j * slices + p] -> sum of slices 0 .. p-1 of segment j; one wave per segment
+__global__ __launch_bounds__(64) void slice_prefix_kernel(float *sums, unsigned slices) {
+  const int lane = lane_id();
+  float *row = sums + (size_t)blockIdx.x * slices;
+  float carry = 0.0f;
+  for (unsigned base = 0; base < slices; base += 64) {
+    const unsigned i = base + lane;
+    const float x = i < slices ? row[i] : 0.0f;
+    const float excl = lane_group_exclusive_scan<6>(x, lane) + carry;
+    if (i < slices) row[i] = excl;
+    carry = readlane(excl + x, 63);
+  }
+}
+
+template <typename OFF, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void seg_scan_offsets_sliced_kernel(const uint16_t *in, uint16_t *out, const float *__restrict__ prefixes, const OFF *__restrict__ begin,
+                                                                            const OFF *__restrict__ end, unsigned slices, int vector) {
+  __shared__ float wave_total[2][kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  const OffsetsSlice s = offsets_slice(begin, end, blockIdx.x / slices, blockIdx.x % slices, slices);
+  float carry = prefixes ? prefixes[blockIdx.x] : 0.0f;  // no prefixes: one slice per segment
+  unsigned parity = 0;
+  // every thread of the block runs the same number of rounds (barriers inside)
+  for (size_t c0 = s.c_lo; c0 < s.c_hi; c0 += blockDim.x) {
+    const size_t c = c0 + threadIdx.x;
+    const bool any = c < s.c_hi;
+    bool full = false;
+    half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (any) v = offsets_masked_chunk<NT>(in, c, s.b, s.e, vector, &full);
+    const float t = sum8(v, 0.0f);
+    const float excl = lane_group_exclusive_scan<6>(t, lane);
+    const float wt = lane_group_sum<6>(t);
+    if (lane == 63) wave_total[parity][wave] = wt;
+    __syncthreads();
+    float before = 0.0f, all = 0.0f;
+    for (int w = 0; w < WPB; w++) {
+      const float x = wave_total[parity][w];
+      if (w < wave) before += x;
+      all += x;
+    }
+    parity ^= 1u;
+    const uint4_t packed = chunk_scan_packed(v, carry + before + excl);
+    carry += all;
+    if (full) {
+      store_chunk<NT>(reinterpret_cast<uint4_t *>(out) + c, packed);
+    } else if (any) {
+      const size_t lo = c * 8;
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        if (lo + i >= s.b && lo + i < s.e) out[lo + i] = (uint16_t)(packed[i / 2] >> (16 * (i & 1)));
+    }
+  }
+}
+
 }  // namespace tcu

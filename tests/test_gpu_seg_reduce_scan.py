@@ -324,7 +324,7 @@ def test_segmented_scan_over_offsets(tcu, oracle):
         exact = np.nanmax(np.abs(wg)) < 4096
         for dtype in (torch.int32, torch.int64):
             bd, ed = torch.from_numpy(begin).to(dtype).cuda(), torch.from_numpy(end).to(dtype).cuda()
-            for expected in (0, 16, 40, 100, 5000):
+            for expected in (0, 16, 40, 100, 5000) + ((1 << 16, 300000) if nseg <= 500 else ()):  # the last two: several blocks per segment
                 out = torch.full((n,), -7.0, dtype=torch.float16, device="cuda")
                 tcu.seg_scan_offsets(xd, bd, ed, expected_segment_size=expected, out=out)
                 got = to_host(out)
@@ -336,7 +336,7 @@ def test_segmented_scan_over_offsets(tcu, oracle):
                 if exact:
                     og = to_host(tcu.seg_scan_offsets(gd, bd, ed, expected_segment_size=expected))
                     assert np.array_equal(og[inside], wg[inside].astype(np.float16).view(np.uint16)), (nseg, str(dtype), expected)
-    for seg in (16, 48, 2048):
+    for seg in (16, 48, 2048, 1 << 17):
         nseg = (1 << 20) // seg
         off = (torch.arange(nseg + 1, dtype=torch.int64) * seg).to(torch.int32).cuda()
         buf = gd[: nseg * seg].clone()
