@@ -212,6 +212,14 @@ int tcu_generate_f16(void *d, size_t n, uint64_t seed, int dist, size_t first, v
  * written to d_dst), mode 2 only writes d_dst.  Used to calibrate hardware counters and
  * to report what fraction of peak a pure copy reaches.  bytes must be a multiple of 16. */
 int tcu_stream_probe(void *d_dst, const void *d_src, size_t bytes, int mode, int tiles_per_wave, int waves_per_block, void *stream);
+/* The next kernel that this host thread launches through the library carries the two events
+ * (hipEvent_t created with timing enabled; either may be NULL): its dispatch stamps
+ * start_event with the time the kernel begins and stop_event with the time it ends, so that
+ * hipEventElapsedTime(start, stop) is the kernel's own duration, without the event packets a
+ * hipEventRecord pair puts on the stream around it.  Meant for entry points that launch one
+ * kernel; with several, only the first carries the events.  The reference brackets its
+ * launches with cudaEventRecord (e.g. src/reduction/seg_wmma_16n.cu:57-73). */
+int tcu_time_next_launch(void *start_event, void *stop_event);
 /* Runs every cross-lane primitive the kernels rely on (MFMA 16x16x32 / 32x32x16 operand
  * layouts, DPP controls, lane swaps) on lane-indexed inputs and writes the raw results
  * to d_out (fp32 / u32 words; see tcu_scope_amd/csrc/probe.hpp for the record layout).

@@ -32,4 +32,5 @@ from .binding import (  # noqa: F401
     seg_scan,
     set_option,
     stream_probe,
+    time_next_launch,
 )

@@ -13,7 +13,7 @@ EXPORTS = [
     "tcu_abi_version", "tcu_last_error", "tcu_init", "tcu_device_info", "tcu_set_option",
     "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_offsets_f16", "tcu_add_partial_sums_f16",
     "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32", "tcu_gemv_f16_f16", "tcu_gemm_f16_f16",
-    "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_lane_probe",
+    "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_time_next_launch", "tcu_lane_probe",
 ]
 
 
@@ -97,6 +97,7 @@ def lib():
         L.tcu_generate_f16.argtypes = [vp, sz, c.c_uint64, ci, sz, vp]
         L.tcu_stream_probe.argtypes = [vp, vp, sz, ci, ci, ci, vp]
         L.tcu_lane_probe.argtypes = [vp, c.POINTER(sz), vp]
+        L.tcu_time_next_launch.argtypes = [vp, vp]
         for name in EXPORTS:
             if name not in ("tcu_last_error",):
                 getattr(L, name).restype = ci
@@ -313,6 +314,13 @@ def generate(n, seed, dist=Dist.UNIFORM, first=0, out=None, device="cuda", strea
 
 def stream_probe(dst, src, nbytes, mode, tiles_per_wave=0, waves_per_block=0, stream=None):
     _check(lib().tcu_stream_probe(_ptr(dst), _ptr(src), nbytes, mode, tiles_per_wave, waves_per_block, _stream(stream)))
+
+
+def time_next_launch(start, stop):
+    """The next kernel launched through the library stamps the torch events `start` and `stop`
+    (enable_timing=True, already recorded once so that their handles exist) with its own begin
+    and end: start.elapsed_time(stop) is then the kernel's duration."""
+    _check(lib().tcu_time_next_launch(start.cuda_event, stop.cuda_event))
 
 
 def lane_probe(device="cuda", stream=None):

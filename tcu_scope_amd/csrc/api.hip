@@ -147,6 +147,13 @@ int tcu_stream_probe(void *d_dst, const void *d_src, size_t bytes, int mode, int
   return after_launch("tcu_stream_probe", before, tcu::stream_probe_dispatch(d_dst, d_src, bytes, mode, tiles_per_wave, waves_per_block, stream));
 }
 
+int tcu_time_next_launch(void *start_event, void *stop_event) {
+  tcu::LaunchEvents &ev = tcu::next_launch_events();
+  ev.start = static_cast<hipEvent_t>(start_event);
+  ev.stop = static_cast<hipEvent_t>(stop_event);
+  return TCU_OK;
+}
+
 int tcu_lane_probe(void *d_out, size_t *out_words, void *stream) { const unsigned long before = tcu::launch_count();
   return after_launch("tcu_lane_probe", before, tcu::lane_probe_dispatch(d_out, out_words, stream)); }
 

@@ -3,6 +3,7 @@
 #ifndef TCU_LAUNCH_HPP
 #define TCU_LAUNCH_HPP
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
 namespace tcu {
@@ -14,10 +15,26 @@ inline unsigned long &launch_count() {
   return n;
 }
 
+// Events that the next launch of this host thread carries: the dispatch itself stamps them
+// with the time the kernel starts and the time it ends (no separate packets on the stream).
+struct LaunchEvents {
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+inline LaunchEvents &next_launch_events() {
+  static thread_local LaunchEvents e;
+  return e;
+}
+
 template <typename... KArgs, typename... Args>
 inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void *stream, Args... args) {
   launch_count()++;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, static_cast<hipStream_t>(stream), static_cast<KArgs>(args)...);
+  LaunchEvents &ev = next_launch_events();
+  if (ev.start || ev.stop) {
+    hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, static_cast<hipStream_t>(stream), ev.start, ev.stop, 0, static_cast<KArgs>(args)...);
+    ev = LaunchEvents{};
+  } else {
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, static_cast<hipStream_t>(stream), static_cast<KArgs>(args)...);
+  }
 }
 
 // Temporary device memory in stream order (from the device's default memory pool: after the

@@ -342,3 +342,31 @@ def test_segmented_scan_over_offsets(tcu, oracle):
         buf = gd[: nseg * seg].clone()
         tcu.seg_scan_offsets(buf, off[:-1], off[1:], expected_segment_size=seg, out=buf)  # in place
         assert np.array_equal(to_host(buf), oracle.seg_scan_f64(g, nseg, seg).astype(np.float16).view(np.uint16)), seg
+
+
+def test_time_next_launch(tcu):
+    """tcu_time_next_launch: the events are stamped by the kernel itself, only the next launch carries them, and the
+    duration lies between what the bytes need at 8 TB/s and the wall-clock time of the call."""
+    import time
+
+    import torch
+
+    n = 1 << 26
+    x = tcu.generate(n, 5, tcu.Dist.UNIFORM)
+    out = torch.empty_like(x)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    b.record()  # creates the handles
+    tcu.seg_scan(x, 256, out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    tcu.time_next_launch(a, b)
+    tcu.seg_scan(x, 256, out=out)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = a.elapsed_time(b)
+    assert 4 * n / 8e12 * 1e3 < ms < wall_ms, (ms, wall_ms)
+    first = ms
+    tcu.seg_scan(x, 256, out=out)  # no events any more: the stamps stay
+    torch.cuda.synchronize()
+    assert a.elapsed_time(b) == first
