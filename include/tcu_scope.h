@@ -168,8 +168,11 @@ int tcu_full_scan_f16(const void *d_in, void *d_out, size_t n, void *d_workspace
  * Replaces compute_wmma_gemv_naive / compute_wmma_gemv_sharedmem (reference
  * src/gemv/wmma_naive.cu:29-94, wmma_sharedmem.cu:43-137); note the reference stores A
  * column-major and returns y as column 0 of an M x 16 matrix.
- * variant: TCU_VARIANT_AUTO, TCU_VARIANT_WAVE_SHUFFLE (dot products + DPP) or
- * TCU_VARIANT_MFMA_16N (16-row strips on MFMA with x as a replicated B operand). */
+ * variant: TCU_VARIANT_AUTO, TCU_VARIANT_WAVE_SHUFFLE (dot products + DPP),
+ * TCU_VARIANT_MFMA_16N (16-row strips on MFMA with x as a replicated B operand, the
+ * reference's formulation) or TCU_VARIANT_MFMA_256N (a 1 KiB tile of a row as the MFMA A
+ * operand, the matching tile of x as the B operand, trace of the accumulated product: the
+ * launch shapes and loads of the dot-product form with the arithmetic on the matrix unit). */
 int tcu_gemv_f16_f32(const void *d_A, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, int variant, void *stream);
 
 /* D = alpha * A B + beta * C.  A: M x K row-major fp16; B: K x N column-major fp16

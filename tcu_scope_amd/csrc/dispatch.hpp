@@ -719,7 +719,9 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
 // OUT = float: tcu_gemv_f16_f32; OUT = half_t: tcu_gemv_f16_f16 (y in fp16)
 template <typename OUT>
 inline int gemv_dispatch_typed(const char *what, const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
-  if (!(variant == TCU_VARIANT_AUTO || variant == TCU_VARIANT_WAVE_SHUFFLE || variant == TCU_VARIANT_MFMA_16N)) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": variant must be AUTO, WAVE_SHUFFLE or MFMA_16N");
+  if (!(variant == TCU_VARIANT_AUTO || variant == TCU_VARIANT_WAVE_SHUFFLE || variant == TCU_VARIANT_MFMA_16N || variant == TCU_VARIANT_MFMA_256N))
+    return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": variant must be AUTO, WAVE_SHUFFLE, MFMA_16N or MFMA_256N");
+  const bool trace = variant == TCU_VARIANT_MFMA_256N;  // row tile x x tile on the matrix unit, same launch shapes as the dot-product form
   if (M == 0) return TCU_OK;
   if (!y || (K && (!A || !x))) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
   const bool vec_ok = K % 8 == 0 && K > 0 && aligned16(A) && aligned16(x);
@@ -753,6 +755,17 @@ inline int gemv_dispatch_typed(const char *what, const void *A, const void *x, v
     const unsigned bw = options().gemv_waves ? (unsigned)options().gemv_waves : (fit >= 16 ? 16u : fit >= 8 ? 8u : 4u);
     const size_t bgrid = (M + rows - 1) / rows;
     if (bgrid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    if (trace) {  // the default shapes only
+      if (rows != 2 || bu > 2) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the MFMA_256N form takes gemv_rows = 2 and gemv_tiles <= 2");
+      if (bu == 2) {
+        if (nt) launch(gemv_block_kernel<2, 2, true, OUT, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
+        else launch(gemv_block_kernel<2, 2, false, OUT, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
+      } else {
+        if (nt) launch(gemv_block_kernel<2, 1, true, OUT, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
+        else launch(gemv_block_kernel<2, 1, false, OUT, true>, (unsigned)bgrid, bw * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
+      }
+      return TCU_OK;
+    }
 #define TCU_GEMV_BLOCK(R_, U_)                                                                                              \
   if (rows == R_ && bu == U_) {                                                                                            \
     if (nt)                                                                                                                \
@@ -772,6 +785,11 @@ inline int gemv_dispatch_typed(const char *what, const void *A, const void *x, v
   const size_t waves = (M + ROWS - 1) / ROWS;
   const size_t grid = (waves + 3) / 4;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+  if (trace) {
+    if (nt) launch(gemv_dot_kernel<ROWS, UK, true, OUT, true>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+    else launch(gemv_dot_kernel<ROWS, UK, false, OUT, true>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+    return TCU_OK;
+  }
   if (nt)
     launch(gemv_dot_kernel<ROWS, UK, true, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
   else

@@ -15,6 +15,9 @@
 //                      the 16 columns, the B operand.  Lane (r, b) reads 64 contiguous
 //                      bytes of row r per 4 MFMAs (k order inside a step is permuted
 //                      identically for A and x, which a contraction does not see).
+//   Both of the first two also run with the matrix unit in place of the dot products
+//   (GemvAcc<true>: a row tile times the x tile, trace of the product), which keeps their
+//   access shape.
 //   gemv_generic_kernel : any M, K (scalar loads).
 #pragma once
 
@@ -35,16 +38,41 @@ TCU_DEVICE float dot8(half8_t a, half8_t x, float acc) {
   return acc;
 }
 
+// Accumulator of one row's dot product, one tile (64 chunks, lane l holding chunk l of the row
+// and of x) at a time.  MFMA = false: packed fp16 dot products per lane.  MFMA = true: the row
+// tile is the 16 x 32 A operand of v_mfma_f32_16x16x32_f16 and the x tile, loaded the same way,
+// the 32 x 16 B operand.  Lane i + 16 b supplies A[i][8b .. 8b+7] and B[8b .. 8b+7][i], i.e. the
+// same 8 positions of the row and of x, so the diagonal D[i][i] = sum_k A[i][k] B[k][i] is the
+// dot product over the 32 positions of lanes i, i + 16, i + 32, i + 48, and the trace of the
+// accumulated D is the dot product of the whole tiles: a GEMV on the matrix unit whose loads
+// are as contiguous as those of the dot-product form (15 of 16 products are discarded, which
+// a bandwidth-bound kernel does not notice).
+template <bool MFMA>
+struct GemvAcc {
+  float v = 0.0f;
+  TCU_DEVICE void add(half8_t a, half8_t x) { v = dot8(a, x, v); }
+  TCU_DEVICE float lane_value(int) const { return v; }
+};
+template <>
+struct GemvAcc<true> {
+  float4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
+  TCU_DEVICE void add(half8_t a, half8_t x) { v = mfma_16x16x32(a, x, v); }
+  // lane l holds D[4 * (l / 16) + j][l % 16], j = 0 .. 3: a diagonal element iff (l % 16) / 4 == l / 16, at j = l % 4
+  TCU_DEVICE float lane_value(int lane) const {
+    const int j = lane & 3;
+    const float d = j == 0 ? v[0] : j == 1 ? v[1] : j == 2 ? v[2] : v[3];
+    return ((lane & 15) >> 2) == (lane >> 4) ? d : 0.0f;
+  }
+};
+
 // K must be a multiple of 8; rows are 16-byte aligned.
-template <int ROWS, int UK, bool NT, typename OUT>
+template <int ROWS, int UK, bool NT, typename OUT, bool MFMA = false>
 __global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t k_chunks, float alpha,
                                                               float beta) {
   const int lane = lane_id();
   const size_t row0 = ((size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block()) * ROWS;
   if (row0 >= M) return;
-  float acc[ROWS];
-#pragma unroll
-  for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+  GemvAcc<MFMA> acc[ROWS];
   const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
   for (size_t c0 = 0; c0 < k_chunks; c0 += (size_t)64 * UK) {
     half8_t xv[UK], av[UK][ROWS];
@@ -62,11 +90,11 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__re
 #pragma unroll
     for (int u = 0; u < UK; u++)
 #pragma unroll
-      for (int r = 0; r < ROWS; r++) acc[r] = dot8(av[u][r], xv[u], acc[r]);
+      for (int r = 0; r < ROWS; r++) acc[r].add(av[u][r], xv[u]);
   }
 #pragma unroll
   for (int r = 0; r < ROWS; r++) {
-    const float s = lane_group_sum<6>(acc[r]);
+    const float s = lane_group_sum<6>(acc[r].lane_value(lane));
     if (lane == 63 && row0 + r < M) gemv_update(y + row0 + r, s, alpha, beta);
   }
 }
@@ -75,7 +103,7 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_dot_kernel(const half8_t *__re
 // w*U .. w*U+U-1 of every step of WPB*U tiles (the x chunks it loads serve all ROWS rows),
 // partial dot products meet in LDS.  Same access shape as the block-per-segment reduction,
 // which is what moves long contiguous rows fastest.
-template <int ROWS, int U, bool NT, typename OUT>
+template <int ROWS, int U, bool NT, typename OUT, bool MFMA = false>
 __global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t k_chunks, float alpha,
                                                                 float beta) {
   __shared__ float partial[ROWS][kMaxWaves];
@@ -83,9 +111,7 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__
   const int WPB = (int)(blockDim.x >> 6);
   const size_t row0 = (size_t)blockIdx.x * ROWS;
   const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  float acc[ROWS];
-#pragma unroll
-  for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+  GemvAcc<MFMA> acc[ROWS];
   for (size_t c0 = (size_t)wave * U * 64; c0 < k_chunks; c0 += (size_t)WPB * U * 64) {
     half8_t xv[U], av[ROWS][U];
 #pragma unroll
@@ -102,11 +128,11 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__
 #pragma unroll
     for (int u = 0; u < U; u++)
 #pragma unroll
-      for (int r = 0; r < ROWS; r++) acc[r] = dot8(av[r][u], xv[u], acc[r]);
+      for (int r = 0; r < ROWS; r++) acc[r].add(av[r][u], xv[u]);
   }
 #pragma unroll
   for (int r = 0; r < ROWS; r++) {
-    const float s = lane_group_sum<6>(acc[r]);
+    const float s = lane_group_sum<6>(acc[r].lane_value(lane));
     if (lane == 63) partial[r][wave] = s;
   }
   __syncthreads();

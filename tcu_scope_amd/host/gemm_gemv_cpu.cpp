@@ -19,7 +19,9 @@ BENCHMARK(CUDA_WMMA_GEMM_SHAREDMEM)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUDA_WMMA_GEMM_NAIVE)->Apply(GemmArgs)->UseManualTime();
 
 static void CUDA_WMMA_GEMV_NAIVE(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMV_NAIVE"); }
-static void CUDA_WMMA_GEMV_SHAREDMEM(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_GEMV_SHAREDMEM"); }
+// the reference's second GEMV kernel stages tiles through shared memory to make its loads contiguous
+// (src/gemv/wmma_sharedmem.cu:43-137); the MFMA form with contiguous loads here is the trace form
+static void CUDA_WMMA_GEMV_SHAREDMEM(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_256N, "CUDA_WMMA_GEMV_SHAREDMEM"); }
 static void TCU_WAVE_GEMV(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_WAVE_SHUFFLE, "TCU_WAVE_GEMV"); }
 static void CUDA_WMMA_HGEMV_NAIVE(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_MFMA_16N, "CUDA_WMMA_HGEMV_NAIVE", true); }
 static void TCU_WAVE_HGEMV(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_WAVE_SHUFFLE, "TCU_WAVE_HGEMV", true); }

@@ -240,11 +240,11 @@ def test_gemv_gemm_and_generator(emu, oracle):
         out = aligned(5000, np.uint16)
         assert emu.emu_generate_f16(out.ctypes.data, 5000, 42, dist, 77) == 0
         assert np.array_equal(out, oracle.generate_f16(5000, 42, dist, first=77))
-    for M, K in ((64, 512), (37, 256), (5, 24), (7, 4608)):
+    for M, K in ((64, 512), (37, 256), (5, 24), (7, 4608), (3, 8192 + 264)):
         A, x = oracle.generate_f16(M * K, 1, oracle.DIST_NORMAL), oracle.generate_f16(K, 2, oracle.DIST_NORMAL)
         y0 = np.linspace(-1, 1, M).astype(np.float32)
         Ai, xi = copy_in(A), copy_in(x)
-        for v in (V_AUTO, V_WAVE, V_MFMA_16N):
+        for v in (V_AUTO, V_WAVE, V_MFMA_16N, V_MFMA_256N):
             y = copy_in(y0, np.float32)
             rc = emu.emu_gemv_f16_f32(Ai.ctypes.data, xi.ctypes.data, y.ctypes.data, M, K, 1.5, -0.5, v)
             if rc == 2:

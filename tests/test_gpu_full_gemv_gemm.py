@@ -99,7 +99,7 @@ def test_gemv(tcu, oracle, M, K):
     x = oracle.generate_f16(K, 2, oracle.DIST_NORMAL)
     y0 = np.linspace(-1, 1, M).astype(np.float32)
     Ad, xd = to_dev(A).view(M, K), to_dev(x)
-    for v in (tcu.Variant.AUTO, tcu.Variant.WAVE_SHUFFLE, tcu.Variant.MFMA_16N):
+    for v in (tcu.Variant.AUTO, tcu.Variant.WAVE_SHUFFLE, tcu.Variant.MFMA_16N, tcu.Variant.MFMA_256N):
         for alpha, beta in [(1.0, 0.0), (1.5, -0.5)]:
             y = torch.from_numpy(y0.copy()).cuda()
             try:
