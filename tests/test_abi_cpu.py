@@ -49,9 +49,9 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.tcu_full_reduce_f16(None, None, 1 << 30, None, ctypes.byref(need), 0, 0, 0, None) == 0 and need.value > 0
     assert lib.tcu_full_reduce_f16(None, None, 1000, None, ctypes.byref(need), 2, 2048, 0, None) == 2  # n % segment_size
     assert lib.tcu_full_scan_f16(None, None, 1 << 20, None, None, 0, 0, 0, None) == 1
-    assert lib.tcu_gemv_f16_f32(p, p, p, 4, 8, 1.0, 0.0, 5, None) == 2
+    assert lib.tcu_gemv_f16_f32(p, p, p, 4, 8, 1.0, 0.0, 6, None) == 2
     assert lib.tcu_gemm_f16_f32(p, p, None, p, 64, 64, 64, 1.0, 0.0, 8, None) == 2  # LDS kernel needs multiples of 128
-    assert lib.tcu_gemv_f16_f16(p, p, p, 4, 8, 1.0, 0.0, 5, None) == 2
+    assert lib.tcu_gemv_f16_f16(p, p, p, 4, 8, 1.0, 0.0, 6, None) == 2
     assert lib.tcu_gemm_f16_f16(p, p, None, p, 64, 64, 64, 1.0, 0.0, 8, None) == 2
     assert lib.tcu_gemm_f16_f16(p, p, None, p, 64, 64, 64, 1.0, 1.0, 0, None) == 1 and "tcu_gemm_f16_f16" in err()  # beta != 0 needs C
     assert lib.tcu_gemv_f16_f16(None, p, p, 4, 8, 1.0, 0.0, 0, None) == 1 and "tcu_gemv_f16_f16" in err()
