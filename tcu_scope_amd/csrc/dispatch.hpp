@@ -34,7 +34,7 @@ inline int fail(int code, const std::string &msg) {
 struct Options {
   bool nontemporal = true;
   bool static_order = false;
-  bool gemm_big_tiles = true;  // 256 x 256 block tiles where the shape allows
+  int gemm_big_tiles = -1;     // 256 x 256 block tiles: 1 wherever M and N allow, 0 never, -1 where there are at least 128 of them
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
@@ -51,7 +51,7 @@ inline int set_option(const char *name, int value) {
   Options &o = options();
   if (n == "nontemporal") o.nontemporal = value != 0;
   else if (n == "static_order") o.static_order = value != 0;
-  else if (n == "gemm_big_tiles") o.gemm_big_tiles = value != 0;
+  else if (n == "gemm_big_tiles") o.gemm_big_tiles = value < 0 ? -1 : (value != 0);
   else if (n == "gemm_direct_lds") o.gemm_direct_lds = value;
   else if (n == "gemm_depth") o.gemm_depth = value;
   else if (n == "gemv_rows") o.gemv_rows = value;
@@ -818,7 +818,10 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
   OUT *d = static_cast<OUT *>(D);
   if (variant == TCU_VARIANT_BLOCK_LDS && !lds_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the LDS kernel needs M, N multiples of 128 and K a multiple of 32");
   if (variant == TCU_VARIANT_MFMA_16N && !direct_ok) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": the direct kernel needs M, N multiples of 32 and K a multiple of 16");
-  if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && options().gemm_big_tiles) {
+  // fewer than 128 tiles of 256 x 256 leave more than half of the 256 compute units idle: the
+  // 128 x 128 kernel then wins (2048^3: 37.8 vs 51.9 us; 2560^3, 100 tiles: 55.8 vs 62.4; 3072^3, 144 tiles: 126 vs 72.5)
+  const bool big_tiles = options().gemm_big_tiles > 0 || (options().gemm_big_tiles < 0 && (M / kGemmBigBM) * (N / kGemmBigBN) >= 128);
+  if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && big_tiles) {
     const size_t grid = (M / kGemmBigBM) * (N / kGemmBigBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     // measured (2048^3 ... 16384^3, K = 4096 ... 16448): the transfer kernels with K step 64 (whole

@@ -280,6 +280,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
     Ai, Bi, Ci = copy_in(A), copy_in(B), copy_in(C0, np.float32)
     ref = oracle.gemm_f64(A, B, M, N, K, 1.5, 2.0, C0)
     try:
+        assert emu.emu_set_option(b"gemm_big_tiles", 1) == 0  # one tile: the default would take the 128 x 128 kernel
         for direct_lds, bk64, depth in ((3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4), (0, 0, 1), (0, 0, 2), (0, 0, 3), (0, 0, 4), (0, 1, 1), (0, 1, 2)):
             for name, val in ((b"gemm_direct_lds", direct_lds), (b"gemm_bk64", bk64), (b"gemm_depth", depth)):
                 assert emu.emu_set_option(name, val) == 0
@@ -290,5 +291,5 @@ def test_gemv_gemm_and_generator(emu, oracle):
             rc = emu.emu_gemm_f16_f16(Ai.ctypes.data, Bi.ctypes.data, Dh.ctypes.data, Dh.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(Dh.reshape(M, N), ref.astype(np.float16).view(np.uint16)), (direct_lds, bk64, depth)
     finally:
-        for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4)):
+        for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1)):
             emu.emu_set_option(name, val)

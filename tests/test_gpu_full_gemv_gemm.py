@@ -170,6 +170,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
 
     M, N = 512, 256
     try:
+        tcu.set_option("gemm_big_tiles", 1)  # two tiles: the default would take the 128 x 128 kernel
         for K in (64, 96, 160, 384, 768):
             A = oracle.generate_f16(M * K, 11, oracle.DIST_SMALLINT)
             B = oracle.generate_f16(N * K, 12, oracle.DIST_SMALLINT)
@@ -200,6 +201,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
         tcu.set_option("gemm_direct_lds", -1)
         tcu.set_option("gemm_bk64", 0)
         tcu.set_option("gemm_depth", 4)
+        tcu.set_option("gemm_big_tiles", -1)
 
 
 def test_gemm_8192(tcu, oracle):
