@@ -98,10 +98,12 @@ static void TCU_SHAPE_SEGMENTED_PREFIXSUM(benchmark::State &state) {
   SHAPE_WAVES(NAME, V, 8)
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_REDUCTION, TCU_VARIANT_MFMA_16N);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_REDUCTION, TCU_VARIANT_MFMA_16N_BLOCK);
+SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_REDUCTION, TCU_VARIANT_MFMA_256N_BLOCK);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_REDUCTION, TCU_VARIANT_WAVE_SHUFFLE);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_REDUCTION, TCU_VARIANT_BLOCK_LDS);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_MFMA_16N);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_MFMA_16N_BLOCK);
+SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_MFMA_256N_BLOCK);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_WAVE_SHUFFLE);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_BLOCK_LDS);
 
