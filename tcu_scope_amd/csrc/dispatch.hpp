@@ -339,15 +339,20 @@ inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t nu
     g_log2 = 1;
     while (g_log2 < 6 && ((size_t)8 << g_log2) < expected) g_log2++;
   }
-  const size_t threads = num_segments << g_log2;
-  const size_t grid = (threads + 255) / 256;
+  // one chunk per lane in flight is too little (120 us at N = 2^28): up to 1024 halves expected, a block takes two
+  // runs of segments and has the first load of both in flight (107-111 us)
+  const int passes = expected && expected <= 1024 ? 2 : 1;  // four passes measure worse (131 us: registers)
+  const size_t segs_per_block = ((size_t)256 >> g_log2) * passes;
+  const size_t grid = (num_segments + segs_per_block - 1) / segs_per_block;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_offsets_f16: grid exceeds the launch limit");
-#define TCU_OFFSETS_CASE(GL)                                                                                                              \
-  case GL:                                                                                                                               \
-    if (nt)                                                                                                                              \
-      launch(seg_reduce_offsets_kernel<OFF, GL, true>, (unsigned)grid, 256u, stream, in, out, num_segments, begin, end, vector);          \
-    else                                                                                                                                 \
-      launch(seg_reduce_offsets_kernel<OFF, GL, false>, (unsigned)grid, 256u, stream, in, out, num_segments, begin, end, vector);         \
+#define TCU_OFFSETS_LAUNCH(GL, NT_, P_) launch(seg_reduce_offsets_kernel<OFF, GL, NT_, P_>, (unsigned)grid, 256u, stream, in, out, num_segments, begin, end, vector)
+#define TCU_OFFSETS_CASE(GL)                                                      \
+  case GL:                                                                       \
+    if (nt) {                                                                    \
+      if (passes == 2) TCU_OFFSETS_LAUNCH(GL, true, 2); else TCU_OFFSETS_LAUNCH(GL, true, 1);   \
+    } else {                                                                     \
+      if (passes == 2) TCU_OFFSETS_LAUNCH(GL, false, 2); else TCU_OFFSETS_LAUNCH(GL, false, 1); \
+    }                                                                            \
     break
   switch (g_log2) {
     TCU_OFFSETS_CASE(1);
@@ -359,6 +364,7 @@ inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t nu
       TCU_OFFSETS_CASE(6);
   }
 #undef TCU_OFFSETS_CASE
+#undef TCU_OFFSETS_LAUNCH
   return TCU_OK;
 }
 

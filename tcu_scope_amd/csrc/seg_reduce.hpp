@@ -261,52 +261,131 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_generic_kernel(const uin
 // Segments given by offsets: segment j = in[begin[j], end[j]) in halves, empty when
 // end[j] <= begin[j]; segments may start anywhere, overlap or leave gaps (the interface of
 // cub::DeviceSegmentedReduce::Sum as the reference calls it, src/reduction/seg_cub_device.cu:46-48).
-// G = 2^G_LOG2 adjacent lanes share a segment: the part between the first and the last
-// 16-byte boundary inside the segment goes through 128-bit loads (lane `sub` takes chunks
-// sub, sub + G, ..., four in flight), the ragged head and tail (< 8 halves each) through
-// 2-byte loads, and a DPP butterfly adds the G partial sums.  With `vector` false (input not
-// 16-byte aligned) everything takes the 2-byte path.
+// G = 2^G_LOG2 adjacent lanes share a segment: the aligned 16-byte chunks it touches are dealt
+// out round-robin (lane `sub` takes the chunks sub, sub + G, ... counted from the segment's
+// first chunk, four in flight); whole chunks are one 128-bit load, the ragged first and last
+// chunk go through 2-byte loads, and a DPP butterfly adds the G partial sums.  With `vector`
+// false (input not 16-byte aligned) every chunk takes the 2-byte path.
 // this lane's share of the sum over in[b, e): lane `sub` of `g` lanes that split the range
+// The sum is taken in two steps so that a caller with several ranges can have the first load of
+// each in flight before it consumes any: range_begin issues the lane's first whole chunk,
+// range_finish adds it and walks the rest.
+struct RangeCursor {
+  size_t b, e, c, c_full_end, c_end;
+  half8_t first;
+  float head;
+  bool has_first;
+};
+TCU_DEVICE float range_partial_chunk(const uint16_t *__restrict__ in, size_t c, size_t b, size_t e) {  // the halves of chunk c inside [b, e), one by one
+  float s = 0.0f;
+  const size_t lo = c * 8;
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+    if (lo + i >= b && lo + i < e) s += (float)__builtin_bit_cast(half_t, in[lo + i]);
+  return s;
+}
 template <bool NT>
-TCU_DEVICE float offsets_range_sum(const uint16_t *__restrict__ in, size_t b, size_t e, size_t sub, size_t g, int vector) {
-  size_t body_b = (b + 7) & ~(size_t)7, body_e = e & ~(size_t)7;  // aligned part [body_b, body_e)
-  if (!vector || body_b >= body_e) body_b = body_e = e;            // none: the head is the whole range
-  float acc = 0.0f, acc1 = 0.0f;
-  for (size_t i = b + sub; i < body_b; i += g) acc += (float)__builtin_bit_cast(half_t, in[i]);
-  for (size_t i = body_e + sub; i < e; i += g) acc += (float)__builtin_bit_cast(half_t, in[i]);
+TCU_DEVICE RangeCursor range_begin(const uint16_t *__restrict__ in, size_t b, size_t e, size_t sub, size_t g, int vector) {
+  RangeCursor r;
+  r.b = b;
+  r.e = e;
+  r.head = 0.0f;
+  r.has_first = false;
+  r.first = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  if (b >= e) {
+    r.c = r.c_full_end = r.c_end = 0;
+    return r;
+  }
+  // the aligned chunks the range touches are dealt out round-robin: lane `sub` takes chunks
+  // c_first + sub, + g, ...; only the first and the last chunk can be partial
+  const size_t c_first = b >> 3;
+  r.c_end = (e + 7) >> 3;
+  r.c_full_end = e >> 3;
+  r.c = c_first + sub;
+  if (!vector) return r;
+  if (r.c == c_first && (b & 7) != 0 && r.c < r.c_end) {
+    r.head = range_partial_chunk(in, r.c, b, e);
+    r.c += g;
+  }
+  if (r.c < r.c_full_end) {
+    r.first = load_chunk<NT>(reinterpret_cast<const half8_t *>(in) + r.c);
+    r.has_first = true;
+    r.c += g;
+  }
+  return r;
+}
+template <bool NT>
+TCU_DEVICE float range_finish(const uint16_t *__restrict__ in, const RangeCursor &r, size_t g, int vector) {
   const half8_t *chunks = reinterpret_cast<const half8_t *>(in);
-  size_t c = body_b / 8 + sub;
-  const size_t ce = body_e / 8;
-  for (; c + 3 * g < ce; c += 4 * g) {
+  float acc = r.head, acc1 = 0.0f;
+  size_t c = r.c;
+  if (!vector) {
+    for (; c < r.c_end; c += g) acc += range_partial_chunk(in, c, r.b, r.e);
+    return acc;
+  }
+  if (r.has_first) acc = sum8(r.first, acc);
+  for (; c + 3 * g < r.c_full_end; c += 4 * g) {
     const half8_t v0 = load_chunk<NT>(chunks + c), v1 = load_chunk<NT>(chunks + c + g), v2 = load_chunk<NT>(chunks + c + 2 * g), v3 = load_chunk<NT>(chunks + c + 3 * g);
     acc = sum8(v0, acc);
     acc1 = sum8(v1, acc1);
     acc = sum8(v2, acc);
     acc1 = sum8(v3, acc1);
   }
-  for (; c < ce; c += g) acc = sum8(load_chunk<NT>(chunks + c), acc);
+  for (; c < r.c_full_end; c += g) acc = sum8(load_chunk<NT>(chunks + c), acc);
+  if (c == r.c_full_end && c < r.c_end) acc1 += range_partial_chunk(in, c, r.b, r.e);  // the ragged last chunk
   return acc + acc1;
 }
+template <bool NT>
+TCU_DEVICE float offsets_range_sum(const uint16_t *__restrict__ in, size_t b, size_t e, size_t sub, size_t g, int vector) {
+  return range_finish<NT>(in, range_begin<NT>(in, b, e, sub, g, vector), g, vector);
+}
 
-template <typename OFF, int G_LOG2, bool NT>
+// A block takes PASSES * SEGS consecutive segments, SEGS = 256 / G at a time, and has the first
+// load of every pass in flight before it consumes one: with a single 16-byte chunk per lane in
+// flight the wave slots of a compute unit do not hold enough bytes to cover the memory latency
+// (one pass: 120 us at N = 2^28 for segments up to 512 halves, two: 107-111 us, four: 131 us).
+template <typename OFF, int G_LOG2, bool NT, int PASSES>
 __global__ __launch_bounds__(256) void seg_reduce_offsets_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, size_t num_segments, const OFF *__restrict__ begin,
                                                                  const OFF *__restrict__ end, int vector) {
   constexpr int G = 1 << G_LOG2;
+  constexpr int SEGS = 256 >> G_LOG2;  // segments per block and pass
+  constexpr int passes = PASSES;
+  __shared__ __attribute__((aligned(16))) uint16_t stage[SEGS * PASSES];
   const int lane = lane_id();
   const int sub = lane & (G - 1);
-  const size_t seg = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> G_LOG2;
-  const bool live = seg < num_segments;
-  size_t b = 0, e = 0;
-  if (live) {
-    const OFF ob = begin[seg], oe = end[seg];
-    if (oe > ob) {
-      b = (size_t)ob;
-      e = (size_t)oe;
+  const bool holder = G_LOG2 <= 4 ? sub == 0 : sub == G - 1;
+  const size_t seg0 = (size_t)blockIdx.x * SEGS * passes;
+  RangeCursor cur[PASSES];
+#pragma unroll
+  for (int p = 0; p < PASSES; p++) {  // every pass's first load goes out before any is consumed
+    const size_t seg = seg0 + (size_t)p * SEGS + (threadIdx.x >> G_LOG2);
+    size_t b = 0, e = 0;
+    if (seg < num_segments) {
+      const OFF ob = begin[seg], oe = end[seg];
+      if (oe > ob) {
+        b = (size_t)ob;
+        e = (size_t)oe;
+      }
+    }
+    cur[p] = range_begin<NT>(in, b, e, (size_t)sub, (size_t)G, vector);
+  }
+#pragma unroll
+  for (int p = 0; p < PASSES; p++) {
+    const float total = lane_group_sum<G_LOG2>(range_finish<NT>(in, cur[p], (size_t)G, vector));
+    if (holder) stage[p * SEGS + (threadIdx.x >> G_LOG2)] = f16_bits(total);
+  }
+  __syncthreads();
+  // the block's results are consecutive in `out`: they leave as 128-bit stores where they can
+  const int n_out = SEGS * passes;
+  for (int i0 = (int)threadIdx.x * 8; i0 < n_out; i0 += 256 * 8) {
+    const size_t s = seg0 + (size_t)i0;
+    if (i0 + 8 <= n_out && s + 8 <= num_segments && (reinterpret_cast<uintptr_t>(out + s) & 15u) == 0) {
+      *reinterpret_cast<uint4_t *>(out + s) = *reinterpret_cast<const uint4_t *>(&stage[i0]);
+    } else {
+      for (int i = 0; i < 8; i++)
+        if (i0 + i < n_out && s + i < num_segments) out[s + i] = stage[i0 + i];
     }
   }
-  const float total = lane_group_sum<G_LOG2>(offsets_range_sum<NT>(in, b, e, (size_t)sub, (size_t)G, vector));
-  const bool holder = G_LOG2 <= 4 ? sub == 0 : sub == G - 1;
-  if (live && holder) out[seg] = f16_bits(total);
 }
 
 // Long segments: `slices` blocks share a segment.  Block (segment j, slice p) adds the p-th of
