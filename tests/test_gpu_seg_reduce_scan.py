@@ -97,6 +97,31 @@ def test_reference_fixture_constant_fill(tcu, oracle):
         assert np.all(np.abs(red - seg * c) <= 0.1) and np.all(np.abs(sc - (np.arange(seg) + 1) * c) <= 0.01)  # the reference's own tolerances
 
 
+def test_results_beyond_fp16_range_become_infinity(tcu, oracle):
+    """Sums past 65504 round to +/-inf exactly where the rounded fp64 sum does (the reference's constant-fill
+    benchmark silently runs into this from 6.5e7 elements on): every variant, reduce, scan, full reduce and scan."""
+    import torch
+
+    seg = 1 << 17
+    n = 4 * seg
+    for value in (1.0, -1.0):
+        x = torch.full((n,), value, dtype=torch.float16, device="cuda")
+        want_red = np.full(4, value * seg)
+        want_scan = np.tile(value * (np.arange(seg) + 1.0), 4)
+        inf_bits = np.float16(value * np.inf).view(np.uint16)
+        for v in (tcu.Variant.AUTO, tcu.Variant.WAVE_SHUFFLE, tcu.Variant.MFMA_16N, tcu.Variant.BLOCK_LDS, tcu.Variant.MFMA_256N_BLOCK):
+            red = to_host(tcu.seg_reduce(x, seg, variant=v))
+            assert np.all(red == inf_bits), (v.name, value)
+            sc = to_host(tcu.seg_scan(x, seg, variant=v))
+            expect_ok(oracle, sc, want_scan, seg, f"scan into inf {v.name}")
+            first_inf = int(np.argmax(sc[:seg] == inf_bits))
+            assert first_inf == 65519 and np.all(sc[first_inf:seg] == inf_bits) and np.all(sc[:first_inf] != inf_bits), (v.name, first_inf)  # 65520 is the first sum that rounds to inf
+        assert to_host(tcu.full_reduce(x))[0] == inf_bits
+        full = to_host(tcu.full_scan(x))
+        assert np.all(full[65519:] == inf_bits) and np.all(full[:65519] != inf_bits)
+        expect_ok(oracle, to_host(tcu.seg_reduce(x, seg)), want_red, seg, "reduce into inf")
+
+
 def test_ragged_and_edge_cases(tcu, oracle):
     import torch
 
