@@ -79,16 +79,17 @@ TCU_DEVICE float row_group_exclusive_scan(float t, int n) {
   return e;
 }
 
-// 8 inclusive prefixes of one chunk started at `e`, rounded to fp16 and packed.
+// 8 inclusive prefixes of one chunk started at `e`, rounded to fp16 and packed.  The even
+// positions are a plain addition, not a dot product with the weights (1, 0): 0 * inf and
+// 0 * NaN would otherwise carry a non-finite value of position 2i + 1 back to position 2i.
 TCU_DEVICE uint4_t chunk_scan_packed(half8_t v, float e) {
-  const half2_t one_zero = {(half_t)1.0f, (half_t)0.0f};
   const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
   const half2_t h01 = __builtin_shufflevector(v, v, 0, 1), h23 = __builtin_shufflevector(v, v, 2, 3);
   const half2_t h45 = __builtin_shufflevector(v, v, 4, 5), h67 = __builtin_shufflevector(v, v, 6, 7);
-  const float x0 = fdot2(h01, one_zero, e), x1 = fdot2(h01, ones, e);
-  const float x2 = fdot2(h23, one_zero, x1), x3 = fdot2(h23, ones, x1);
-  const float x4 = fdot2(h45, one_zero, x3), x5 = fdot2(h45, ones, x3);
-  const float x6 = fdot2(h67, one_zero, x5), x7 = fdot2(h67, ones, x5);
+  const float x0 = e + (float)v[0], x1 = fdot2(h01, ones, e);
+  const float x2 = x1 + (float)v[2], x3 = fdot2(h23, ones, x1);
+  const float x4 = x3 + (float)v[4], x5 = fdot2(h45, ones, x3);
+  const float x6 = x5 + (float)v[6], x7 = fdot2(h67, ones, x5);
   uint4_t r = {pack_f16x2(x0, x1), pack_f16x2(x2, x3), pack_f16x2(x4, x5), pack_f16x2(x6, x7)};
   return r;
 }

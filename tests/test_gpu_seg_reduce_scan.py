@@ -122,6 +122,51 @@ def test_results_beyond_fp16_range_become_infinity(tcu, oracle):
         expect_ok(oracle, to_host(tcu.seg_reduce(x, seg)), want_red, seg, "reduce into inf")
 
 
+@pytest.mark.parametrize("seg", [16, 256, 2048, 16384])
+def test_non_finite_inputs_stay_in_their_segment(tcu, oracle, seg):
+    """A NaN or an infinity in one segment reaches that segment's sum and the prefixes from its position on, and nothing
+    else (AUTO and the DPP / LDS variants; the MFMA variants multiply by 0/1 matrices, where 0 * inf is NaN, and are
+    only required to keep what lies outside the wave's span of at most 8 tiles clean)."""
+    import torch
+
+    n = 1 << 20
+    nseg = n // seg
+    x_host = oracle.generate_f16(n, 31, oracle.DIST_UNIFORM)
+    ref_red = oracle.seg_reduce_f64(x_host, nseg, seg)
+    ref_scan = oracle.seg_scan_f64(x_host, nseg, seg)
+    for bits, name in ((0x7E00, "nan"), (0x7C00, "inf")):
+        hit_seg, hit_pos = nseg // 3, seg // 2 + 3
+        xh = x_host.copy()
+        xh[hit_seg * seg + hit_pos] = bits
+        x = to_dev(xh)
+        for v in (tcu.Variant.AUTO, tcu.Variant.WAVE_SHUFFLE, tcu.Variant.BLOCK_LDS):
+            try:
+                red = to_host(tcu.seg_reduce(x, seg, variant=v)).view(np.float16).astype(np.float64)
+                sc = to_host(tcu.seg_scan(x, seg, variant=v)).view(np.float16).astype(np.float64).reshape(nseg, seg)
+            except tcu.TcuError as e:
+                assert e.status == 2
+                continue
+            bad = (lambda a: np.isnan(a)) if name == "nan" else (lambda a: np.isinf(a) & (a > 0))
+            assert bad(red[hit_seg]) and np.all(bad(sc[hit_seg, hit_pos:])), (v.name, name)
+            keep = np.ones(nseg, bool)
+            keep[hit_seg] = False
+            assert np.all(np.isfinite(red[keep])) and np.all(np.isfinite(sc[keep])) and np.all(np.isfinite(sc[hit_seg, :hit_pos])), (v.name, name)
+            assert oracle.check_f16(red[keep].astype(np.float16).view(np.uint16), ref_red[keep], seg)[0] == 0
+            assert oracle.check_f16(sc[keep].astype(np.float16).view(np.uint16), ref_scan.reshape(nseg, seg)[keep], seg)[0] == 0
+        # MFMA flavour: whatever lies outside the 8 tiles (4096 halves) around the value and outside its segment is untouched
+        red = to_host(tcu.seg_reduce(x, seg, variant=tcu.Variant.MFMA_16N)).view(np.float16).astype(np.float64)
+        sc = to_host(tcu.seg_scan(x, seg, variant=tcu.Variant.MFMA_16N)).view(np.float16).astype(np.float64)
+        span = (hit_seg * seg + hit_pos) // 4096
+        clean = np.ones(n, bool)
+        lo = min(span * 4096, hit_seg * seg)
+        hi = max((span + 1) * 4096, (hit_seg + 1) * seg)
+        clean[lo:hi] = False
+        assert np.all(np.isfinite(sc[clean])), name
+        seg_clean = np.ones(nseg, bool)
+        seg_clean[lo // seg:(hi + seg - 1) // seg] = False
+        assert np.all(np.isfinite(red[seg_clean])), name
+
+
 def test_ragged_and_edge_cases(tcu, oracle):
     import torch
 
