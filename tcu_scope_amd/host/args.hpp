@@ -7,56 +7,65 @@
 
 #include "minibench.hpp"
 
-static inline int64_t two_power_i(int64_t p) { return static_cast<int64_t>(1) << p; }
+// The generators are plain functions of run-time parameters; the names the benchmark files
+// use (ARGS, SEG_<S>_ARGS, Tuning<base>_x_<log2>) are thin wrappers that fix the parameters.
+namespace argspace {
+using Bench = benchmark::internal::Benchmark;
 
-constexpr int64_t kMinElementsLog2 = 12, kMaxElementsLog2 = 30;
+inline int64_t pow2(int64_t exponent) { return int64_t{1} << exponent; }
+constexpr int64_t kSmallestLog2 = 12, kLargestLog2 = 30;  // element counts 2^12 .. 2^30
 
-static inline void ArgsParams(benchmark::internal::Benchmark *b) {
-  for (int64_t l = kMinElementsLog2; l <= kMaxElementsLog2; l++) b->Args({two_power_i(l)});
+// {num_elements}
+inline void element_counts(Bench *b) {
   b->ArgNames({"num_elements"});
+  for (int64_t e = kSmallestLog2; e <= kLargestLog2; ++e) b->Args({pow2(e)});
 }
-
-template <int BASE_SEGMENT_SIZE>
-static inline void ArgsParamsSegmented(benchmark::internal::Benchmark *b) {
-  for (int64_t l = kMinElementsLog2; l <= kMaxElementsLog2; l++) {
-    const int64_t num_elements = two_power_i(l);
-    b->Args({num_elements / BASE_SEGMENT_SIZE, BASE_SEGMENT_SIZE, num_elements});
-  }
+// {num_segments, segment_size, num_elements} for one segment size over all element counts
+inline void fixed_segment_size(Bench *b, int64_t segment_size) {
   b->ArgNames({"num_segments", "segment_size", "num_elements"});
+  for (int64_t e = kSmallestLog2; e <= kLargestLog2; ++e) b->Args({pow2(e) / segment_size, segment_size, pow2(e)});
 }
-
-#define ARGS() Apply(ArgsParams)
-#define SEG_16_ARGS() Apply(ArgsParamsSegmented<16>)
-#define SEG_32_ARGS() Apply(ArgsParamsSegmented<32>)
-#define SEG_64_ARGS() Apply(ArgsParamsSegmented<64>)
-#define SEG_128_ARGS() Apply(ArgsParamsSegmented<128>)
-#define SEG_256_ARGS() Apply(ArgsParamsSegmented<256>)
-#define SEG_512_ARGS() Apply(ArgsParamsSegmented<512>)
-#define SEG_1024_ARGS() Apply(ArgsParamsSegmented<1024>)
-#define SEG_2048_ARGS() Apply(ArgsParamsSegmented<2048>)
-#define SEG_4096_ARGS() Apply(ArgsParamsSegmented<4096>)
-#define SEG_8192_ARGS() Apply(ArgsParamsSegmented<8192>)
-#define SEG_16384_ARGS() Apply(ArgsParamsSegmented<16384>)
-
-// fixed element count 2^MAX_ELEMENTS_LOG2, segment size swept from the base upwards
-template <int BASE_SEGMENT_SIZE, int MAX_ELEMENTS_LOG2>
-static inline void TuningArgs(benchmark::internal::Benchmark *b) {
-  const int64_t num_elements = two_power_i(MAX_ELEMENTS_LOG2);
-  for (int64_t num_segments = num_elements / BASE_SEGMENT_SIZE; num_segments >= 1; num_segments /= 2) {
-    const int64_t segment_size = num_elements / num_segments;
-    if (segment_size < BASE_SEGMENT_SIZE) continue;
-    b->Args({num_segments, segment_size, BASE_SEGMENT_SIZE, MAX_ELEMENTS_LOG2});
-  }
+// {num_segments, segment_size, base_segment_size, max_elements_log2}: 2^log2_elements elements cut
+// into ever longer segments, from the base size up to one segment
+inline void growing_segments(Bench *b, int64_t base_segment_size, int64_t log2_elements) {
   b->ArgNames({"num_segments", "segment_size", "base_segment_size", "max_elements_log2"});
+  for (int64_t segment_size = base_segment_size; segment_size <= pow2(log2_elements); segment_size *= 2)
+    b->Args({pow2(log2_elements) / segment_size, segment_size, base_segment_size, log2_elements});
 }
-static inline void Tuning16_x_22(benchmark::internal::Benchmark *b) { TuningArgs<16, 22>(b); }
-static inline void Tuning256_x_22(benchmark::internal::Benchmark *b) { TuningArgs<256, 22>(b); }
-static inline void Tuning16_x_26(benchmark::internal::Benchmark *b) { TuningArgs<16, 26>(b); }
-static inline void Tuning256_x_26(benchmark::internal::Benchmark *b) { TuningArgs<256, 26>(b); }
-static inline void Tuning16_x_28(benchmark::internal::Benchmark *b) { TuningArgs<16, 28>(b); }
-static inline void Tuning256_x_28(benchmark::internal::Benchmark *b) { TuningArgs<256, 28>(b); }
-static inline void Tuning16_x_30(benchmark::internal::Benchmark *b) { TuningArgs<16, 30>(b); }
-static inline void Tuning256_x_30(benchmark::internal::Benchmark *b) { TuningArgs<256, 30>(b); }
+template <int64_t SEGMENT_SIZE>
+void with_segment_size(Bench *b) {
+  fixed_segment_size(b, SEGMENT_SIZE);
+}
+template <int64_t BASE, int64_t LOG2_ELEMENTS>
+void with_growing_segments(Bench *b) {
+  growing_segments(b, BASE, LOG2_ELEMENTS);
+}
+}  // namespace argspace
+
+static inline int64_t two_power_i(int64_t p) { return argspace::pow2(p); }
+
+#define ARGS() Apply(argspace::element_counts)
+#define TCU_SEG_ARGS(S) Apply(argspace::with_segment_size<S>)
+#define SEG_16_ARGS() TCU_SEG_ARGS(16)
+#define SEG_32_ARGS() TCU_SEG_ARGS(32)
+#define SEG_64_ARGS() TCU_SEG_ARGS(64)
+#define SEG_128_ARGS() TCU_SEG_ARGS(128)
+#define SEG_256_ARGS() TCU_SEG_ARGS(256)
+#define SEG_512_ARGS() TCU_SEG_ARGS(512)
+#define SEG_1024_ARGS() TCU_SEG_ARGS(1024)
+#define SEG_2048_ARGS() TCU_SEG_ARGS(2048)
+#define SEG_4096_ARGS() TCU_SEG_ARGS(4096)
+#define SEG_8192_ARGS() TCU_SEG_ARGS(8192)
+#define SEG_16384_ARGS() TCU_SEG_ARGS(16384)
+
+constexpr auto Tuning16_x_22 = argspace::with_growing_segments<16, 22>;
+constexpr auto Tuning256_x_22 = argspace::with_growing_segments<256, 22>;
+constexpr auto Tuning16_x_26 = argspace::with_growing_segments<16, 26>;
+constexpr auto Tuning256_x_26 = argspace::with_growing_segments<256, 26>;
+constexpr auto Tuning16_x_28 = argspace::with_growing_segments<16, 28>;
+constexpr auto Tuning256_x_28 = argspace::with_growing_segments<256, 28>;
+constexpr auto Tuning16_x_30 = argspace::with_growing_segments<16, 30>;
+constexpr auto Tuning256_x_30 = argspace::with_growing_segments<256, 30>;
 
 static inline void GemmArgs(benchmark::internal::Benchmark *b) {
   static const int64_t sizes[] = {16, 32, 48, 64, 96, 128, 192, 256, 512, 768, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 7168, 8192, 9216, 10240, 12288, 14336, 16384};
