@@ -866,6 +866,15 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
   } else if (lds_ok && variant != TCU_VARIANT_MFMA_16N) {
     const size_t grid = (M / kGemmBM) * (N / kGemmBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    // the transfer kernel with 128 x 128 tiles (two blocks per compute unit) unless the register-staged
+    // kernel is asked for (gemm_direct_lds = 0) or K is beyond the 32-bit lane offsets
+    if (options().gemm_direct_lds != 0 && K <= ((size_t)1 << 22)) {
+      if (K % 64 == 0)
+        launch(gemm_dlds_kernel<64, 2, OUT, 128>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      else
+        launch(gemm_dlds_kernel<32, 4, OUT, 128>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      return TCU_OK;
+    }
     launch(gemm_lds_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
   } else if (direct_ok) {
     const size_t tiles = (M / 32) * (N / 32);

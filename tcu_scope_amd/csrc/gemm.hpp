@@ -10,10 +10,11 @@
 //                        two LDS buffers (one barrier per step).  Counterpart of the
 //                        reference's shared-memory kernels (src/gemm/wmma.cu:171-365,
 //                        wmma_sharedmem.cu:43-123).
-//   gemm_lds256_kernel, gemm_dlds_kernel : 256 x 256 block tile, 4 waves of 128 x 128 (all 256
-//                        accumulation registers), hand-pipelined; operands staged through
-//                        registers or moved global -> LDS directly (described at the kernels).
-//                        These run whenever M and N are multiples of 256.
+//   gemm_lds256_kernel, gemm_dlds_kernel, gemm_dlds_a3b2_kernel : 256 x 256 block tile, 4 waves
+//                        of 128 x 128 (all 256 accumulation registers), hand-pipelined;
+//                        operands staged through registers or moved global -> LDS directly
+//                        (described at the kernels).  gemm_dlds_kernel also comes with
+//                        128 x 128 block tiles for outputs too small to fill the chip.
 //   gemm_direct_kernel : one 32 x 32 tile per wave, fragments loaded straight from global
 //                        memory (reference compute_gemm_naive, src/gemm/wmma_naive.cu:33-88).
 //   gemm_generic_kernel: any M, N, K; one thread per output element.
@@ -340,8 +341,10 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
     for (int j = 0; j < 4; j++) gemm_store_tile(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 32, tile_n * kGemmBigBN + wn * 128 + j * 32, acc[i][j], lane, alpha, beta);
 }
 
-// M % 256 == 0, N % 256 == 0, K % BK == 0, K <= 2^22 (lane offsets are 32-bit); 256 threads.
-// Same tiling as gemm_lds256_kernel (256 x 256 x BK block tile, 2 x 2 waves of 128 x 128), but
+// M % TILE == 0, N % TILE == 0, K % BK == 0, K <= 2^22 (lane offsets are 32-bit); 256 threads.
+// TILE = 256: same tiling as gemm_lds256_kernel (256 x 256 x BK block tile, 2 x 2 waves of
+// 128 x 128); TILE = 128: 2 x 2 waves of 64 x 64, 64 KiB of LDS, two blocks per compute unit
+// (outputs too small to fill the chip with 256 x 256 tiles).  In both,
 // the operands travel from global memory straight into LDS (load_chunk_to_lds), NBUF K steps
 // deep: no staging registers, no LDS store instructions, prefetch distance NBUF - 1 steps.
 // LDS rows are dense (BK halves = CPR chunks of 16 bytes).  A transfer instruction fills
@@ -358,24 +361,26 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
 // into the buffer that barrier has just freed (measured: every substep of extra flight time
 // is worth 2-7 %; issuing more than half of a step's transfers in that one substep loses it
 // again).
-template <int BK, int NBUF, typename OUT>
+template <int BK, int NBUF, typename OUT, int TILE = kGemmBigBM>
 __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
   constexpr int ROWH = BK;                           // halves per LDS row
   constexpr int CPR = BK / 8;                        // chunks per row
   constexpr int RPT = 64 / CPR;                      // rows per transfer instruction
   constexpr int RS = CPR == 4 ? 2 : 1;               // f(r) = (r >> RS) & (CPR - 1)
   constexpr int SUB = BK / 16;                       // 16-wide k substeps per step
-  constexpr int OPH = kGemmBigBM * ROWH;             // halves per operand per stage
+  constexpr int W = TILE / 64;                       // 32 x 32 accumulators per wave and dimension (wave tile TILE/2 x TILE/2)
+  constexpr int HALF = W * W / 2;                    // MFMAs per half substep
+  constexpr int OPH = TILE * ROWH;                   // halves per operand per stage
   constexpr int P = NBUF - 1;                        // prefetch distance in steps
-  constexpr int TPW = kGemmBigBM / RPT / 4;          // transfer instructions per wave, operand and step
-  constexpr int EARLY = TPW;                         // transfers of a step issued one substep ahead of the others
-  static_assert((BK == 32 || BK == 64) && EARLY <= 8 && 2 * TPW - EARLY <= 8 * (SUB - 1) && 2 * TPW * (P - 1) + EARLY <= 63, "transfers must fit the substeps and the counter");
+  constexpr int TPW = TILE / RPT / 4;                // transfer instructions per wave, operand and step
+  constexpr int EARLY = TPW < HALF ? TPW : HALF;     // transfers of a step issued one substep ahead of the others
+  static_assert((TILE == 128 || TILE == 256) && (BK == 32 || BK == 64) && 2 * TPW - EARLY <= HALF * (SUB - 1) && 2 * TPW * (P - 1) + EARLY <= 63, "transfers must fit the substeps and the counter");
   __shared__ __attribute__((aligned(1024))) half_t lds_a[NBUF][OPH];
   __shared__ __attribute__((aligned(1024))) half_t lds_b[NBUF][OPH];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   size_t tile_m, tile_n;
-  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, &tile_m, &tile_n);
+  gemm_tile_of_block(M / TILE, N / TILE, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
   const size_t steps = K / BK;
   // transfer t of this wave (t = 0 .. TPW-1) fills rows RPT * (wave * TPW + t) .. + RPT-1; the
@@ -389,8 +394,8 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
     const int chunk = (lane % CPR) ^ ((row >> RS) & (CPR - 1));
     goff[t] = (uint32_t)(((size_t)row * k_chunks + chunk) * 16);
   }
-  const char *ga = reinterpret_cast<const char *>(A + tile_m * kGemmBigBM * k_chunks);
-  const char *gb = reinterpret_cast<const char *>(B + tile_n * kGemmBigBN * k_chunks);
+  const char *ga = reinterpret_cast<const char *>(A + tile_m * TILE * k_chunks);
+  const char *gb = reinterpret_cast<const char *>(B + tile_n * TILE * k_chunks);
   constexpr lds_addr_t STAGE = OPH * 2, TBYTES = 1024, STEPB = BK * 2;  // bytes per stage and operand, per transfer, per step and row
   const lds_addr_t ta = wave_uniform(lds_address_of(&lds_a[0][0]) + wave * TPW * TBYTES);
   const lds_addr_t tb = wave_uniform(lds_address_of(&lds_b[0][0]) + wave * TPW * TBYTES);
@@ -403,11 +408,11 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
       load_chunk_to_lds(gb + st * STEPB, goff[x / 2], tb + buf * STAGE + (x / 2) * TBYTES);
   };
 
-  float16_t acc[4][4];
+  float16_t acc[W][W];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < W; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < W; j++)
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
@@ -422,13 +427,13 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
 
   // fragment of row r, k chunk kc: slot kc ^ f(r); rows of a lane differ by multiples of 32
   const int frow = lane & 31, khalf = lane >> 5, fsw = (frow >> RS) & (CPR - 1);
-  const int fa0 = (wm * 128 + frow) * ROWH, fb0 = (wn * 128 + frow) * ROWH;
+  const int fa0 = (wm * (TILE / 2) + frow) * ROWH, fb0 = (wn * (TILE / 2) + frow) * ROWH;
   int ko[SUB];
 #pragma unroll
   for (int kk = 0; kk < SUB; kk++) ko[kk] = ((2 * kk + khalf) ^ fsw) * 8;
-  half8_t fa[2][4], fb[2][4];
+  half8_t fa[2][W], fb[2][W];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < W; i++) {
     fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[0][fa0 + i * 32 * ROWH + ko[0]]);
     fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[0][fb0 + i * 32 * ROWH + ko[0]]);
   }
@@ -442,25 +447,25 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
       if (kk < SUB - 1) {
         sched_fence();
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < W; i++) {
           fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[cur][fa0 + i * 32 * ROWH + ko[kk + 1]]);
           fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[cur][fb0 + i * 32 * ROWH + ko[kk + 1]]);
         }
         // first half of the MFMAs with the fragment reads, second half with one transfer each
         // (the transfers are opaque to the scheduler, so fences pin them in place)
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < W / 2; i++)
 #pragma unroll
-          for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+          for (int j = 0; j < W; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-          sched_group<kSchedDsRead, 1>();
+        for (int t = 0; t < HALF; t++) {
+          sched_group<kSchedDsRead, 2 * W / HALF>();
           sched_group<kSchedMfma, 1>();
         }
         sched_fence();
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-          const int i = 2 + t / 4, j = t % 4, x = EARLY + kk * 8 + t;
+        for (int t = 0; t < HALF; t++) {
+          const int i = W / 2 + t / W, j = t % W, x = EARLY + kk * HALF + t;
           if (x < 2 * TPW) issue(s + P, fill, x);
           acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
           sched_fence();
@@ -471,25 +476,25 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
         block_barrier_lds_only();
         sched_fence();
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < W; i++) {
           fa[q][i] = *reinterpret_cast<const half8_t *>(&lds_a[nxt][fa0 + i * 32 * ROWH + ko[0]]);
           fb[q][i] = *reinterpret_cast<const half8_t *>(&lds_b[nxt][fb0 + i * 32 * ROWH + ko[0]]);
         }
         // the buffer of step s is free from this barrier on: the first transfers of step
         // s + NBUF go out here, one substep ahead of the rest
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < W / 2; i++)
 #pragma unroll
-          for (int j = 0; j < 4; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
+          for (int j = 0; j < W; j++) acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-          sched_group<kSchedDsRead, 1>();
+        for (int t = 0; t < HALF; t++) {
+          sched_group<kSchedDsRead, 2 * W / HALF>();
           sched_group<kSchedMfma, 1>();
         }
         sched_fence();
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-          const int i = 2 + t / 4, j = t % 4;
+        for (int t = 0; t < HALF; t++) {
+          const int i = W / 2 + t / W, j = t % W;
           if (t < EARLY) issue(s + NBUF, cur, t);
           acc[i][j] = mfma_32x32x16(fa[p][i], fb[p][j], acc[i][j]);
           sched_fence();
@@ -500,9 +505,9 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < W; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) gemm_store_tile(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 32, tile_n * kGemmBigBN + wn * 128 + j * 32, acc[i][j], lane, alpha, beta);
+    for (int j = 0; j < W; j++) gemm_store_tile(D, C, N, tile_m * TILE + wm * (TILE / 2) + i * 32, tile_n * TILE + wn * (TILE / 2) + j * 32, acc[i][j], lane, alpha, beta);
 }
 
 // M % 256 == 0, N % 256 == 0, K % 64 == 0, K <= 2^22; 256 threads.

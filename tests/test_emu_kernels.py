@@ -257,7 +257,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
             rc = emu.emu_gemv_f16_f16(Ai.ctypes.data, xi.ctypes.data, yh.ctypes.data, M, K, 1.5, -0.5, v)
             ref = oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0h.astype(np.float32))
             assert rc == 0 and oracle.check_f16(yh[:M], ref, K)[0] == 0, (M, K, v)
-    for M, N, K in ((128, 128, 64), (256, 512, 64), (64, 32, 48), (33, 17, 20)):
+    for M, N, K in ((128, 128, 64), (256, 512, 64), (128, 256, 96), (64, 32, 48), (33, 17, 20)):
         A, B = oracle.generate_f16(M * K, 5, oracle.DIST_SMALLINT), oracle.generate_f16(N * K, 6, oracle.DIST_SMALLINT)
         C0 = (np.arange(M * N) % 7).astype(np.float32)
         Ai, Bi, Ci = copy_in(A), copy_in(B), copy_in(C0, np.float32)

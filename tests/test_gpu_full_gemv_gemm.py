@@ -124,7 +124,7 @@ def test_gemv(tcu, oracle, M, K):
             assert bad == 0, ("fp16 y", v.name, alpha, beta, bad, worst, first)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (512, 384, 160), (96, 64, 48), (33, 17, 20)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (512, 384, 160), (384, 640, 1088), (96, 64, 48), (33, 17, 20)])
 def test_gemm_small_exact_and_normal(tcu, oracle, M, N, K):
     import torch
 
