@@ -290,6 +290,15 @@ def test_gemv_gemm_and_generator(emu, oracle):
             Dh = copy_in(C0.astype(np.float16).view(np.uint16))  # in place: C == D
             rc = emu.emu_gemm_f16_f16(Ai.ctypes.data, Bi.ctypes.data, Dh.ctypes.data, Dh.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(Dh.reshape(M, N), ref.astype(np.float16).view(np.uint16)), (direct_lds, bk64, depth)
+        # 128 x 128 tiles: the transfer kernel (K step 64 and 32) and the register-staged one
+        assert emu.emu_set_option(b"gemm_big_tiles", 0) == 0
+        for direct_lds, Ks in ((-1, 192), (-1, 96), (0, 96)):
+            assert emu.emu_set_option(b"gemm_direct_lds", direct_lds) == 0
+            A2, B2 = oracle.generate_f16(M * Ks, 9, oracle.DIST_SMALLINT), oracle.generate_f16(N * Ks, 10, oracle.DIST_SMALLINT)
+            A2i, B2i = copy_in(A2), copy_in(B2)
+            D = aligned(M * N, np.float32, -777)
+            rc = emu.emu_gemm_f16_f32(A2i.ctypes.data, B2i.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, Ks, 1.5, 2.0, V_BLOCK)
+            assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A2, B2, M, N, Ks, 1.5, 2.0, C0)), (direct_lds, Ks)
     finally:
         for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1)):
             emu.emu_set_option(name, val)

@@ -197,6 +197,20 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
                 torch.cuda.synchronize()
                 assert np.array_equal(Dh.cpu().numpy().view(np.uint16), ref0.astype(np.float16).view(np.uint16)), ("fp16", K, direct_lds, bk64, depth)
                 assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("fp16 in place", K, direct_lds, bk64, depth)
+        # 128 x 128 tiles: the transfer kernel (K step 64 and 32) and the register-staged one
+        tcu.set_option("gemm_big_tiles", 0)
+        tcu.set_option("gemm_bk64", 0)
+        for direct_lds, K in ((-1, 64), (-1, 448), (-1, 224), (0, 224)):
+            tcu.set_option("gemm_direct_lds", direct_lds)
+            A = oracle.generate_f16(M * K, 21, oracle.DIST_SMALLINT)
+            B = oracle.generate_f16(N * K, 22, oracle.DIST_SMALLINT)
+            Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
+            Cd = torch.from_numpy(C0.copy()).cuda().view(M, N)
+            tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd, variant=tcu.Variant.BLOCK_LDS)
+            Dh = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS, out_dtype=torch.float16)
+            torch.cuda.synchronize()
+            assert np.array_equal(Cd.cpu().numpy().astype(np.float64), oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)), ("128 tiles", direct_lds, K)
+            assert np.array_equal(Dh.cpu().numpy().view(np.uint16), oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0).astype(np.float16).view(np.uint16)), ("128 tiles fp16", direct_lds, K)
     finally:
         tcu.set_option("gemm_direct_lds", -1)
         tcu.set_option("gemm_bk64", 0)
