@@ -92,9 +92,10 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more)
  *   "gemm_big_tiles"  -1/0/1, default -1: 256 x 256 block tiles wherever M and N allow (1), never (0), or
  *                     where the output has at least 128 of them (-1; smaller outputs take 128 x 128 tiles)
- *   "gemm_direct_lds" -1/0/3/4/64/65, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
+ *   "gemm_direct_lds" -1/0/3/4/64/65/66, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
  *                     buffers; 64 = K step 64, two buffers; 65 = K step 64, three buffers for A and two for B;
- *                     0 = register-staged kernel; -1 = 65 where K is a multiple of 64, else 4
+ *                     66 = as 65 on 16x16x32 instead of 32x32x16 MFMAs (C and D aligned to four outputs, else 65);
+ *                     0 = register-staged kernel; -1 = 66 where K is a multiple of 64, else 4
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
  * Unknown names return TCU_ERR_INVALID_ARG. */

@@ -36,7 +36,7 @@ struct Options {
   bool static_order = false;
   int gemm_big_tiles = -1;     // 256 x 256 block tiles: 1 wherever M and N allow, 0 never, -1 where there are at least 128 of them
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
-  int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 0: register-staged kernel; -1: by shape
+  int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
@@ -833,10 +833,16 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
     // measured (2048^3 ... 16384^3, K = 4096 ... 16448): the transfer kernels with K step 64 (whole
     // 128-byte lines per row and transfer) beat the K-step-32 and the register-staged forms at
     // every size (8192^3: 1305 vs 1225 vs 1128 TFLOP/s), and of the two the one with three A and
-    // two B buffers is equal or faster everywhere (16384^3: 1313 vs 1083)
-    const int direct_lds = options().gemm_direct_lds >= 0 ? options().gemm_direct_lds : (K % 64 == 0 ? 65 : 4);
+    // two B buffers is equal or faster everywhere (16384^3: 1313 vs 1083).  The same kernel on
+    // 16x16x32 MFMAs (66) draws less power per multiply-add and is the default: 8192^3 with fp16
+    // outputs 783 vs 852 us, fp32 outputs 850 vs 866; 16384^3 fp16 6.36 vs 6.80 ms (same run)
+    const int direct_lds = options().gemm_direct_lds >= 0 ? options().gemm_direct_lds : (K % 64 == 0 ? 66 : 4);
     if (direct_lds > 0 && K <= ((size_t)1 << 22)) {
-      if (direct_lds == 65 && K % 64 == 0)
+      // the 16x16x32 kernel moves four adjacent outputs per access (16 bytes of fp32, 8 of fp16)
+      const bool al4 = ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & (4 * sizeof(OUT) - 1)) == 0;
+      if (direct_lds == 66 && K % 64 == 0 && al4)
+        launch(gemm_dlds_a3b2_m16_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      else if (direct_lds >= 65 && K % 64 == 0)
         launch(gemm_dlds_a3b2_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       else if (direct_lds >= 64 && K % 64 == 0)
         launch(gemm_dlds_kernel<64, 2, OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);

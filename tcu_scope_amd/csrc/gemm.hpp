@@ -10,11 +10,13 @@
 //                        two LDS buffers (one barrier per step).  Counterpart of the
 //                        reference's shared-memory kernels (src/gemm/wmma.cu:171-365,
 //                        wmma_sharedmem.cu:43-123).
-//   gemm_lds256_kernel, gemm_dlds_kernel, gemm_dlds_a3b2_kernel : 256 x 256 block tile, 4 waves
-//                        of 128 x 128 (all 256 accumulation registers), hand-pipelined;
-//                        operands staged through registers or moved global -> LDS directly
-//                        (described at the kernels).  gemm_dlds_kernel also comes with
-//                        128 x 128 block tiles for outputs too small to fill the chip.
+//   gemm_lds256_kernel, gemm_dlds_kernel, gemm_dlds_a3b2_kernel, gemm_dlds_a3b2_m16_kernel :
+//                        256 x 256 block tile, 4 waves of 128 x 128 (all 256 accumulation
+//                        registers), hand-pipelined; operands staged through registers or
+//                        moved global -> LDS directly (described at the kernels); the last
+//                        one on v_mfma_f32_16x16x32_f16 (less power per multiply-add), the
+//                        others on 32x32x16.  gemm_dlds_kernel also comes with 128 x 128
+//                        block tiles for outputs too small to fill the chip.
 //   gemm_direct_kernel : one 32 x 32 tile per wave, fragments loaded straight from global
 //                        memory (reference compute_gemm_naive, src/gemm/wmma_naive.cu:33-88).
 //   gemm_generic_kernel: any M, N, K; one thread per output element.
@@ -27,7 +29,7 @@ namespace tcu {
 constexpr int kGemmBM = 128, kGemmBN = 128, kGemmBK = 32;
 constexpr int kGemmLdsStride = 40;  // halves per LDS row (32 + 8 pad)
 
-TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_m, size_t *tile_n);
+TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t b, size_t *tile_m, size_t *tile_n);
 
 // D and C are streamed once: non-temporal accesses keep them from displacing the A and B
 // panels that other tiles reuse from L2.  All of a tile's C values are read before its first
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   size_t tile_m, tile_n;
-  gemm_tile_of_block(M / kGemmBM, N / kGemmBN, &tile_m, &tile_n);
+  gemm_tile_of_block(M / kGemmBM, N / kGemmBN, blockIdx.x, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
   // global -> LDS copy assignment: 128 rows x 4 chunks = 512 chunks per operand, 2 per thread
   const int crow = tid >> 2, cchunk = tid & 3;  // rows crow and crow + 64
@@ -159,8 +161,8 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict
 // with its own L2.  Block ids are first regrouped so that an XCD owns a contiguous range of
 // tile ids, and tile ids walk bands of 4 tile rows column by column, so that the ~32 blocks
 // an XCD runs at a time form a 4 x 8 patch sharing A row panels and B column panels in L2.
-TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t *tile_m, size_t *tile_n) {
-  const size_t nb = tiles_m * tiles_n, b = blockIdx.x;
+TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t b, size_t *tile_m, size_t *tile_n) {
+  const size_t nb = tiles_m * tiles_n;
   const size_t id = nb % 8 == 0 ? (b % 8) * (nb / 8) + b / 8 : b;
   constexpr size_t GM = 4;
   const size_t band = id / (GM * tiles_n);
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(256) void gemm_lds256_kernel(const half8_t *__restr
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   size_t tile_m, tile_n;
-  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, &tile_m, &tile_n);
+  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, blockIdx.x, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
   // Copy assignment: CPR consecutive lanes take one row's BK halves (one or two full cache
   // lines of global memory), 16 consecutive lanes 16 / CPR consecutive rows.  Inside LDS the
@@ -380,7 +382,7 @@ __global__ __launch_bounds__(256) void gemm_dlds_kernel(const half8_t *__restric
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   size_t tile_m, tile_n;
-  gemm_tile_of_block(M / TILE, N / TILE, &tile_m, &tile_n);
+  gemm_tile_of_block(M / TILE, N / TILE, blockIdx.x, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
   const size_t steps = K / BK;
   // transfer t of this wave (t = 0 .. TPW-1) fills rows RPT * (wave * TPW + t) .. + RPT-1; the
@@ -529,7 +531,7 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_kernel(const half8_t *__re
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   size_t tile_m, tile_n;
-  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, &tile_m, &tile_n);
+  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, blockIdx.x, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
   const size_t steps = K / BK;
   uint32_t goff[TPW];
@@ -648,6 +650,186 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_kernel(const half8_t *__re
   for (int i = 0; i < 4; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) gemm_store_tile(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 32, tile_n * kGemmBigBN + wn * 128 + j * 32, acc[i][j], lane, alpha, beta);
+}
+
+// One row of eight 16 x 16 tiles whose accumulators came from mfma_16x16x32 with the B fragment
+// as the first operand (the product is formed transposed): the lane owns row (lane & 15) and
+// the four adjacent columns 4 * (lane >> 4) .. + 3 of every tile, i.e. one 128-bit (fp32) or
+// 64-bit (fp16) access per tile.  All C values of the row are read before its first store.
+template <typename OUT>
+TCU_DEVICE void gemm_store_row_of_tiles16(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8], int lane, float alpha, float beta) {
+  const size_t base = (row0 + (lane & 15)) * ldc + col0 + 4 * (lane >> 4);
+  if constexpr (sizeof(OUT) == 4) {
+    float4_t *d4 = reinterpret_cast<float4_t *>(D + base);
+    if (beta == 0.0f) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) __builtin_nontemporal_store(alpha * acc[j], d4 + j * 4);
+    } else {
+      const float4_t *c4 = reinterpret_cast<const float4_t *>(C + base);
+      float4_t c[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) c[j] = __builtin_nontemporal_load(c4 + j * 4);
+#pragma unroll
+      for (int j = 0; j < 8; j++) __builtin_nontemporal_store(alpha * acc[j] + beta * c[j], d4 + j * 4);
+    }
+  } else {
+    uint2_t *d2 = reinterpret_cast<uint2_t *>(D + base);
+    if (beta == 0.0f) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        uint2_t v;
+        v[0] = pack_f16x2(alpha * acc[j][0], alpha * acc[j][1]);
+        v[1] = pack_f16x2(alpha * acc[j][2], alpha * acc[j][3]);
+        __builtin_nontemporal_store(v, d2 + j * 4);
+      }
+    } else {
+      const uint2_t *c2 = reinterpret_cast<const uint2_t *>(C + base);
+      uint2_t c[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) c[j] = __builtin_nontemporal_load(c2 + j * 4);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const uint32_t w01 = c[j][0], w23 = c[j][1];  // scalars first: a bit cast straight from a vector element reads element 0
+        const half2_t c01 = __builtin_bit_cast(half2_t, w01), c23 = __builtin_bit_cast(half2_t, w23);
+        uint2_t v;
+        v[0] = pack_f16x2(alpha * acc[j][0] + beta * (float)c01[0], alpha * acc[j][1] + beta * (float)c01[1]);
+        v[1] = pack_f16x2(alpha * acc[j][2] + beta * (float)c23[0], alpha * acc[j][3] + beta * (float)c23[1]);
+        __builtin_nontemporal_store(v, d2 + j * 4);
+      }
+    }
+  }
+}
+
+// gemm_dlds_a3b2_kernel on v_mfma_f32_16x16x32_f16: the same block tile, buffers and transfer
+// schedule, but a wave's 128 x 128 tile is 8 x 8 accumulators of 16 x 16 and a K step of 64 is
+// two substeps of 32, each 16 fragment reads for 64 MFMAs.  Per multiply-add this shape reads
+// the A/B fragment registers twice as often and the accumulator registers half as often as
+// 32x32x16; the accumulators being four times as many words, the register traffic is lower,
+// and so is the power: with operands held in registers the chip sustains 1865 TFLOP/s in this
+// shape against 1600 in the other (normally distributed inputs, 40 ms launches), and the
+// kernel is limited by power, not by issue slots.  C and D must be aligned to four outputs
+// (16 bytes of fp32, 8 of fp16).
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+  constexpr int BK = 64, ROWH = BK, CPR = 8, RPT = 8, RS = 1, SUB = 2, NA = 3, NB = 2;
+  constexpr int OPH = kGemmBigBM * ROWH;     // halves per operand per stage
+  constexpr int TPW = kGemmBigBM / RPT / 4;  // transfer instructions per wave, operand and step (8)
+  __shared__ __attribute__((aligned(1024))) half_t lds_a[NA][OPH];
+  __shared__ __attribute__((aligned(1024))) half_t lds_b[NB][OPH];
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  size_t tile_m, tile_n;
+  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, blockIdx.x, &tile_m, &tile_n);
+  const size_t k_chunks = K / 8;
+  const size_t steps = K / BK;
+  uint32_t goff[TPW];
+#pragma unroll
+  for (int t = 0; t < TPW; t++) {
+    const int row = (wave * TPW + t) * RPT + lane / CPR;
+    const int chunk = (lane % CPR) ^ ((row >> RS) & (CPR - 1));
+    goff[t] = (uint32_t)(((size_t)row * k_chunks + chunk) * 16);
+  }
+  constexpr lds_addr_t STAGE = OPH * 2, TBYTES = 1024, STEPB = BK * 2;
+  const char *ga = reinterpret_cast<const char *>(A + tile_m * kGemmBigBM * k_chunks);
+  const char *gb = reinterpret_cast<const char *>(B + tile_n * kGemmBigBN * k_chunks);
+  const lds_addr_t ta = wave_uniform(lds_address_of(&lds_a[0][0]) + wave * TPW * TBYTES);
+  const lds_addr_t tb = wave_uniform(lds_address_of(&lds_b[0][0]) + wave * TPW * TBYTES);
+  auto issue_a = [&](size_t step, int buf, int t) { load_chunk_to_lds(ga + (step < steps ? step : steps - 1) * STEPB, goff[t], ta + buf * STAGE + t * TBYTES); };
+  auto issue_b = [&](size_t step, int buf, int t) { load_chunk_to_lds(gb + (step < steps ? step : steps - 1) * STEPB, goff[t], tb + buf * STAGE + t * TBYTES); };
+
+  float4_t acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
+
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_a(0, 0, t);
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_b(0, 0, t);
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_a(1, 1, t);
+#pragma unroll
+  for (int t = 0; t < TPW; t++) issue_b(1, 1, t);
+  wait_vector_loads<2 * TPW>();
+  block_barrier_lds_only();
+
+  // fragment of row r, k chunk kc: slot kc ^ f(r); the lane supplies row (lane & 15) of a
+  // 16-row tile and chunk (lane >> 4) of the substep's four; rows of a lane differ by multiples of 16
+  const int frow = lane & 15, kq = lane >> 4, fsw = (frow >> RS) & (CPR - 1);
+  const int fa0 = (wm * 128 + frow) * ROWH, fb0 = (wn * 128 + frow) * ROWH;
+  int ko[SUB];
+#pragma unroll
+  for (int kk = 0; kk < SUB; kk++) ko[kk] = ((4 * kk + kq) ^ fsw) * 8;
+  half8_t fa[2][8], fb[2][8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[0][fa0 + i * 16 * ROWH + ko[0]]);
+    fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[0][fb0 + i * 16 * ROWH + ko[0]]);
+  }
+  int ca = 0, cb = 0;  // s % NA, s % NB
+  for (size_t s = 0; s < steps; s++) {
+    const int na = ca + 1 == NA ? 0 : ca + 1, nb = cb ^ 1;
+    const int fill_a = ca == 0 ? NA - 1 : ca - 1;  // A buffer of step s - 1 = of step s + 2
+    // substep 0: fragments of substep 1 under the first 32 MFMAs, the A tile of step s + 2 under the others
+    sched_fence();
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      fa[1][i] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + i * 16 * ROWH + ko[1]]);
+      fb[1][i] = *reinterpret_cast<const half8_t *>(&lds_b[cb][fb0 + i * 16 * ROWH + ko[1]]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc[i][j] = mfma_16x16x32(fb[0][j], fa[0][i], acc[i][j]);
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+      sched_group<kSchedDsRead, 1>();
+      sched_group<kSchedMfma, 2>();
+    }
+    sched_fence();
+#pragma unroll
+    for (int t = 0; t < 32; t++) {
+      const int i = 4 + t / 8, j = t % 8;
+      if (t % 4 == 0) issue_a(s + 2, fill_a, t / 4);
+      acc[i][j] = mfma_16x16x32(fb[0][j], fa[0][i], acc[i][j]);
+      sched_fence();
+    }
+    // substep 1: own transfers of step s + 1 done (the A tile of step s + 2 may still fly),
+    // barrier, fragments of step s + 1, B tile of step s + 2 into the B buffer of step s
+    wait_vector_loads<TPW>();
+    block_barrier_lds_only();
+    sched_fence();
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + i * 16 * ROWH + ko[0]]);
+      fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[nb][fb0 + i * 16 * ROWH + ko[0]]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc[i][j] = mfma_16x16x32(fb[1][j], fa[1][i], acc[i][j]);
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+      sched_group<kSchedDsRead, 1>();
+      sched_group<kSchedMfma, 2>();
+    }
+    sched_fence();
+#pragma unroll
+    for (int t = 0; t < 32; t++) {
+      const int i = 4 + t / 8, j = t % 8;
+      if (t % 4 == 0) issue_b(s + 2, cb, t / 4);
+      acc[i][j] = mfma_16x16x32(fb[1][j], fa[1][i], acc[i][j]);
+      sched_fence();
+    }
+    ca = na;
+    cb = nb;
+  }
+  wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
+#pragma unroll
+  for (int i = 0; i < 8; i++) gemm_store_row_of_tiles16(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 16, tile_n * kGemmBigBN + wn * 128, acc[i], lane, alpha, beta);
 }
 
 // M % 32 == 0, N % 32 == 0, K % 16 == 0; one 32 x 32 tile per wave.

@@ -281,7 +281,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
     ref = oracle.gemm_f64(A, B, M, N, K, 1.5, 2.0, C0)
     try:
         assert emu.emu_set_option(b"gemm_big_tiles", 1) == 0  # one tile: the default would take the 128 x 128 kernel
-        for direct_lds, bk64, depth in ((3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4), (0, 0, 1), (0, 0, 2), (0, 0, 3), (0, 0, 4), (0, 1, 1), (0, 1, 2)):
+        for direct_lds, bk64, depth in ((3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4), (66, 0, 4), (0, 0, 1), (0, 0, 2), (0, 0, 3), (0, 0, 4), (0, 1, 1), (0, 1, 2)):
             for name, val in ((b"gemm_direct_lds", direct_lds), (b"gemm_bk64", bk64), (b"gemm_depth", depth)):
                 assert emu.emu_set_option(name, val) == 0
             D = aligned(M * N, np.float32, -777)

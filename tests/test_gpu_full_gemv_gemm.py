@@ -178,7 +178,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
             ref0 = oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0)
             ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
-            shapes = [(0, bk64, depth) for bk64 in (0, 1) for depth in (1, 2, 3, 4)] + [(3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4)]
+            shapes = [(0, bk64, depth) for bk64 in (0, 1) for depth in (1, 2, 3, 4)] + [(3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4), (66, 0, 4)]
             for direct_lds, bk64, depth in shapes:
                 tcu.set_option("gemm_direct_lds", direct_lds)
                 tcu.set_option("gemm_bk64", bk64)
@@ -197,6 +197,26 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
                 torch.cuda.synchronize()
                 assert np.array_equal(Dh.cpu().numpy().view(np.uint16), ref0.astype(np.float16).view(np.uint16)), ("fp16", K, direct_lds, bk64, depth)
                 assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("fp16 in place", K, direct_lds, bk64, depth)
+        # default kernel choice with outputs that are 4-byte but not 8- or 16-byte aligned: the kernel that
+        # moves four adjacent outputs per access must not be picked
+        tcu.set_option("gemm_direct_lds", -1)
+        K = 384
+        A = oracle.generate_f16(M * K, 13, oracle.DIST_SMALLINT)
+        B = oracle.generate_f16(N * K, 14, oracle.DIST_SMALLINT)
+        Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
+        ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
+        buf32 = torch.zeros(M * N + 4, dtype=torch.float32, device="cuda")
+        buf16 = torch.zeros(M * N + 4, dtype=torch.float16, device="cuda")
+        for off32, off16 in ((0, 0), (1, 2)):
+            Cd = buf32[off32:off32 + M * N].view(M, N)
+            Cd.copy_(torch.from_numpy(C0).view(M, N))
+            Ch = buf16[off16:off16 + M * N].view(M, N)
+            Ch.copy_(torch.from_numpy(C0.astype(np.float16)).view(M, N))
+            tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd)
+            tcu.gemm(Ad, Bd, 2.0, -1.0, C=Ch, out=Ch)
+            torch.cuda.synchronize()
+            assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("offset", off32)
+            assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("offset fp16", off16)
         # 128 x 128 tiles: the transfer kernel (K step 64 and 32) and the register-staged one
         tcu.set_option("gemm_big_tiles", 0)
         tcu.set_option("gemm_bk64", 0)
