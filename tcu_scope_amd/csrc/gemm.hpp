@@ -22,6 +22,8 @@
 //   gemm_generic_kernel: any M, N, K; one thread per output element.
 #pragma once
 
+#include <type_traits>
+
 #include "wave_ops.hpp"
 
 namespace tcu {
@@ -652,51 +654,60 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_kernel(const half8_t *__re
     for (int j = 0; j < 4; j++) gemm_store_tile(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 32, tile_n * kGemmBigBN + wn * 128 + j * 32, acc[i][j], lane, alpha, beta);
 }
 
-// One row of eight 16 x 16 tiles whose accumulators came from mfma_16x16x32 with the B fragment
-// as the first operand (the product is formed transposed): the lane owns row (lane & 15) and
-// the four adjacent columns 4 * (lane >> 4) .. + 3 of every tile, i.e. one 128-bit (fp32) or
-// 64-bit (fp16) access per tile.  All C values of the row are read before its first store.
+// Epilogue of a 128-column strip of 16 x 16 tiles whose accumulators came from mfma_16x16x32
+// with the B fragment as the first operand (the product is formed transposed): the lane owns
+// row (lane & 15) and the four adjacent columns 4 * (lane >> 4) .. + 3 of every tile, i.e. one
+// 128-bit (fp32) or 64-bit (fp16) access per tile.  CRow16 holds a lane's C values of one row
+// of eight tiles.
 template <typename OUT>
-TCU_DEVICE void gemm_store_row_of_tiles16(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8], int lane, float alpha, float beta) {
-  const size_t base = (row0 + (lane & 15)) * ldc + col0 + 4 * (lane >> 4);
-  if constexpr (sizeof(OUT) == 4) {
-    float4_t *d4 = reinterpret_cast<float4_t *>(D + base);
-    if (beta == 0.0f) {
+struct CRow16 {
+  using word_t = typename std::conditional<sizeof(OUT) == 4, float4_t, uint2_t>::type;
+  word_t v[8];
+};
+template <typename OUT>
+TCU_DEVICE void gemm_load_c_row16(CRow16<OUT> &c, const OUT *C, size_t ldc, size_t row0, size_t col0, int lane) {
+  using word_t = typename CRow16<OUT>::word_t;
+  const word_t *p = reinterpret_cast<const word_t *>(C + (row0 + (lane & 15)) * ldc + col0 + 4 * (lane >> 4));
 #pragma unroll
-      for (int j = 0; j < 8; j++) __builtin_nontemporal_store(alpha * acc[j], d4 + j * 4);
+  for (int j = 0; j < 8; j++) c.v[j] = __builtin_nontemporal_load(p + j * 4);
+}
+// D = alpha * acc + beta * c for one row of eight tiles; c is not read when beta == 0
+template <typename OUT>
+TCU_DEVICE void gemm_store_row16(OUT *D, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8], const CRow16<OUT> &c, int lane, float alpha, float beta) {
+  using word_t = typename CRow16<OUT>::word_t;
+  word_t *p = reinterpret_cast<word_t *>(D + (row0 + (lane & 15)) * ldc + col0 + 4 * (lane >> 4));
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    float4_t r = alpha * acc[j];
+    if constexpr (sizeof(OUT) == 4) {
+      if (beta != 0.0f) r += beta * c.v[j];
+      __builtin_nontemporal_store(r, p + j * 4);
     } else {
-      const float4_t *c4 = reinterpret_cast<const float4_t *>(C + base);
-      float4_t c[8];
-#pragma unroll
-      for (int j = 0; j < 8; j++) c[j] = __builtin_nontemporal_load(c4 + j * 4);
-#pragma unroll
-      for (int j = 0; j < 8; j++) __builtin_nontemporal_store(alpha * acc[j] + beta * c[j], d4 + j * 4);
-    }
-  } else {
-    uint2_t *d2 = reinterpret_cast<uint2_t *>(D + base);
-    if (beta == 0.0f) {
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        uint2_t v;
-        v[0] = pack_f16x2(alpha * acc[j][0], alpha * acc[j][1]);
-        v[1] = pack_f16x2(alpha * acc[j][2], alpha * acc[j][3]);
-        __builtin_nontemporal_store(v, d2 + j * 4);
-      }
-    } else {
-      const uint2_t *c2 = reinterpret_cast<const uint2_t *>(C + base);
-      uint2_t c[8];
-#pragma unroll
-      for (int j = 0; j < 8; j++) c[j] = __builtin_nontemporal_load(c2 + j * 4);
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const uint32_t w01 = c[j][0], w23 = c[j][1];  // scalars first: a bit cast straight from a vector element reads element 0
+      if (beta != 0.0f) {
+        const uint32_t w01 = c.v[j][0], w23 = c.v[j][1];  // scalars first: a bit cast straight from a vector element reads element 0
         const half2_t c01 = __builtin_bit_cast(half2_t, w01), c23 = __builtin_bit_cast(half2_t, w23);
-        uint2_t v;
-        v[0] = pack_f16x2(alpha * acc[j][0] + beta * (float)c01[0], alpha * acc[j][1] + beta * (float)c01[1]);
-        v[1] = pack_f16x2(alpha * acc[j][2] + beta * (float)c23[0], alpha * acc[j][3] + beta * (float)c23[1]);
-        __builtin_nontemporal_store(v, d2 + j * 4);
+        r[0] += beta * (float)c01[0];
+        r[1] += beta * (float)c01[1];
+        r[2] += beta * (float)c23[0];
+        r[3] += beta * (float)c23[1];
       }
+      uint2_t v;
+      v[0] = pack_f16x2(r[0], r[1]);
+      v[1] = pack_f16x2(r[2], r[3]);
+      __builtin_nontemporal_store(v, p + j * 4);
     }
+  }
+}
+// The whole strip: eight rows of tiles, each row's C values read just before its stores (C may
+// be the same buffer as D: a lane reads only elements it will itself write).  Reading one to
+// three rows ahead of the stores measured the same or up to 1 % slower (8192^3, same run).
+template <typename OUT>
+TCU_DEVICE void gemm_store_strip16(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8][8], int lane, float alpha, float beta) {
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    CRow16<OUT> c;
+    if (beta != 0.0f) gemm_load_c_row16(c, C, ldc, row0 + i * 16, col0, lane);
+    gemm_store_row16(D, ldc, row0 + i * 16, col0, acc[i], c, lane, alpha, beta);
   }
 }
 
@@ -745,6 +756,7 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *
 #pragma unroll
       for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
 
+  // in flight at the first barrier: A0 B0 | A1 B1 (the wave's counter returns in issue order)
 #pragma unroll
   for (int t = 0; t < TPW; t++) issue_a(0, 0, t);
 #pragma unroll
@@ -773,63 +785,43 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *
   for (size_t s = 0; s < steps; s++) {
     const int na = ca + 1 == NA ? 0 : ca + 1, nb = cb ^ 1;
     const int fill_a = ca == 0 ? NA - 1 : ca - 1;  // A buffer of step s - 1 = of step s + 2
-    // substep 0: fragments of substep 1 under the first 32 MFMAs, the A tile of step s + 2 under the others
-    sched_fence();
+    // substep 0: MFMA t works on tile (t / 8, t % 8); fragment k of substep 1 (order: A0 B0..B7 A1..A7)
+    // is read before MFMA 2k
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      fa[1][i] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + i * 16 * ROWH + ko[1]]);
-      fb[1][i] = *reinterpret_cast<const half8_t *>(&lds_b[cb][fb0 + i * 16 * ROWH + ko[1]]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-      for (int j = 0; j < 8; j++) acc[i][j] = mfma_16x16x32(fb[0][j], fa[0][i], acc[i][j]);
-#pragma unroll
-    for (int t = 0; t < 16; t++) {
-      sched_group<kSchedDsRead, 1>();
-      sched_group<kSchedMfma, 2>();
-    }
-    sched_fence();
-#pragma unroll
-    for (int t = 0; t < 32; t++) {
-      const int i = 4 + t / 8, j = t % 8;
-      if (t % 4 == 0) issue_a(s + 2, fill_a, t / 4);
-      acc[i][j] = mfma_16x16x32(fb[0][j], fa[0][i], acc[i][j]);
+    for (int t = 0; t < 64; t++) {
+      if (t < 32 && t % 2 == 0) {
+        const int k = t / 2;
+        if (k == 0) fa[1][0] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + ko[1]]);
+        else if (k <= 8) fb[1][k - 1] = *reinterpret_cast<const half8_t *>(&lds_b[cb][fb0 + (k - 1) * 16 * ROWH + ko[1]]);
+        else fa[1][k - 8] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + (k - 8) * 16 * ROWH + ko[1]]);
+      }
+      if (t >= 32 && t % 4 == 0) issue_a(s + 2, fill_a, (t - 32) / 4);  // A tile of step s + 2 under the second half
+      acc[t / 8][t % 8] = mfma_16x16x32(fb[0][t % 8], fa[0][t / 8], acc[t / 8][t % 8]);
       sched_fence();
     }
-    // substep 1: own transfers of step s + 1 done (the A tile of step s + 2 may still fly),
-    // barrier, fragments of step s + 1, B tile of step s + 2 into the B buffer of step s
+    // substep 1: own transfers of step s + 1 done (the A tile of step s + 2 may still fly), barrier,
+    // fragments of step s + 1.  (Measured and dropped: the B tile under the first half of this
+    // substep, and the A tile a substep earlier, three steps ahead: 0-2 % slower.)
     wait_vector_loads<TPW>();
     block_barrier_lds_only();
     sched_fence();
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + i * 16 * ROWH + ko[0]]);
-      fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[nb][fb0 + i * 16 * ROWH + ko[0]]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-      for (int j = 0; j < 8; j++) acc[i][j] = mfma_16x16x32(fb[1][j], fa[1][i], acc[i][j]);
-#pragma unroll
-    for (int t = 0; t < 16; t++) {
-      sched_group<kSchedDsRead, 1>();
-      sched_group<kSchedMfma, 2>();
-    }
-    sched_fence();
-#pragma unroll
-    for (int t = 0; t < 32; t++) {
-      const int i = 4 + t / 8, j = t % 8;
-      if (t % 4 == 0) issue_b(s + 2, cb, t / 4);
-      acc[i][j] = mfma_16x16x32(fb[1][j], fa[1][i], acc[i][j]);
+    for (int t = 0; t < 64; t++) {
+      if (t < 32 && t % 2 == 0) {
+        const int k = t / 2;
+        if (k == 0) fa[0][0] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + ko[0]]);
+        else if (k <= 8) fb[0][k - 1] = *reinterpret_cast<const half8_t *>(&lds_b[nb][fb0 + (k - 1) * 16 * ROWH + ko[0]]);
+        else fa[0][k - 8] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + (k - 8) * 16 * ROWH + ko[0]]);
+      }
+      if (t >= 32 && t % 4 == 0) issue_b(s + 2, cb, (t - 32) / 4);  // B tile of step s + 2 into the B buffer of step s
+      acc[t / 8][t % 8] = mfma_16x16x32(fb[1][t % 8], fa[1][t / 8], acc[t / 8][t % 8]);
       sched_fence();
     }
     ca = na;
     cb = nb;
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
-#pragma unroll
-  for (int i = 0; i < 8; i++) gemm_store_row_of_tiles16(D, C, N, tile_m * kGemmBigBM + wm * 128 + i * 16, tile_n * kGemmBigBN + wn * 128, acc[i], lane, alpha, beta);
+  gemm_store_strip16(D, C, N, tile_m * kGemmBigBM + wm * 128, tile_n * kGemmBigBN + wn * 128, acc, lane, alpha, beta);
 }
 
 // M % 32 == 0, N % 32 == 0, K % 16 == 0; one 32 x 32 tile per wave.
