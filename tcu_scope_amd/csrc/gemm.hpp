@@ -165,7 +165,8 @@ __global__ __launch_bounds__(256) void gemm_lds_kernel(const half8_t *__restrict
 // an XCD runs at a time form a 4 x 8 patch sharing A row panels and B column panels in L2.
 TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t b, size_t *tile_m, size_t *tile_n) {
   const size_t nb = tiles_m * tiles_n;
-  const size_t id = nb % 8 == 0 ? (b % 8) * (nb / 8) + b / 8 : b;
+  const size_t nb8 = nb & ~(size_t)7;  // the last nb % 8 blocks keep their ids
+  const size_t id = b < nb8 ? (b % 8) * (nb8 / 8) + b / 8 : b;
   constexpr size_t GM = 4;
   const size_t band = id / (GM * tiles_n);
   const size_t rows = tiles_m - band * GM < GM ? tiles_m - band * GM : GM;

@@ -67,13 +67,17 @@ constexpr auto Tuning256_x_28 = argspace::with_growing_segments<256, 28>;
 constexpr auto Tuning16_x_30 = argspace::with_growing_segments<16, 30>;
 constexpr auto Tuning256_x_30 = argspace::with_growing_segments<256, 30>;
 
+// GEMM: the reference's cubes (src/gemm/args.hpp:6-66): irregular steps up to 9216, then every 512 up to 28160
 static inline void GemmArgs(benchmark::internal::Benchmark *b) {
-  static const int64_t sizes[] = {16, 32, 48, 64, 96, 128, 192, 256, 512, 768, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 7168, 8192, 9216, 10240, 12288, 14336, 16384};
-  for (int64_t s : sizes) b->Args({s, s, s});
+  static const int64_t small[] = {16, 32, 48, 64, 96, 128, 192, 256, 512, 768, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 7168, 8192};
+  for (int64_t s : small) b->Args({s, s, s});
+  for (int64_t s = 9216; s <= 28160; s += 512) b->Args({s, s, s});
   b->ArgNames({"M", "N", "K"});
 }
+// GEMV: the reference's squares (src/gemv/args.hpp:6-65): irregular steps up to 1536, then every 512 from 2048 to 25600
 static inline void GemvArgs(benchmark::internal::Benchmark *b) {
-  static const int64_t sizes[] = {16, 32, 48, 64, 96, 128, 192, 256, 512, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 7168, 8192, 9216, 10240, 12288, 14336, 16384, 20480, 24576};
-  for (int64_t s : sizes) b->Args({s, s});
+  static const int64_t small[] = {16, 32, 48, 64, 96, 128, 192, 256, 512, 1024, 1536};
+  for (int64_t s : small) b->Args({s, s});
+  for (int64_t s = 2048; s <= 25600; s += 512) b->Args({s, s});
   b->ArgNames({"M", "N"});
 }

@@ -36,6 +36,9 @@ def test_benchmark_names_follow_the_reference_grammar():
         "CUDA_WMMA_FULL_PREFIXSUM_3KERS<8 * 256, 8>/num_elements:1073741824/manual_time",
         "CUDA_WMMA_GEMM/M:8192/N:8192/K:8192/manual_time",
         "CUDA_WMMA_GEMM_NAIVE/M:8192/N:8192/K:8192/manual_time",
+        "CUDA_WMMA_GEMM/M:9728/N:9728/K:9728/manual_time",
+        "CUDA_WMMA_HGEMM/M:28160/N:28160/K:28160/manual_time",
+        "CUDA_WMMA_GEMV_NAIVE/M:25600/N:25600/manual_time",
         "CUDA_WMMA_GEMV_NAIVE/M:16384/N:16384/manual_time",
         "CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/segment_size:16/num_elements:1048576/manual_time",
         # the "unsafe" twins and the library baselines that the reference's plot specs select
