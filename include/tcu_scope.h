@@ -96,6 +96,11 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *                     buffers; 64 = K step 64, two buffers; 65 = K step 64, three buffers for A and two for B;
  *                     66 = as 65 on 16x16x32 instead of 32x32x16 MFMAs (C and D aligned to four outputs, else 65);
  *                     0 = register-staged kernel; -1 = 66 where K is a multiple of 64, else 4
+ *   "gemm_split_tail" 0/1/2, default 1: the K steps of the tiles of a last, partly filled round of the big-tile GEMM
+ *                     grid are spread over all compute units (fp32 shares in stream-ordered temporary memory, added
+ *                     in a fixed order by a second kernel): never, where it pays (round at most a third full,
+ *                     K >= 4096), or whenever there is such a round
+ *   "compute_units"   blocks of the big-tile GEMM kernel the device runs at a time (set by tcu_init; for tests)
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
  * Unknown names return TCU_ERR_INVALID_ARG. */

@@ -58,6 +58,7 @@ int tcu_init(int device_id) {
   s.lds_bytes = (int)prop.sharedMemPerBlock;
   s.gfx950 = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
   s.initialised = true;
+  if (s.compute_units > 0) tcu::options().compute_units = s.compute_units;
   if (!s.gfx950) return tcu::fail(TCU_ERR_UNSUPPORTED, std::string("tcu_init: this library is built for gfx950 only, device is ") + prop.gcnArchName);
   return TCU_OK;
 }

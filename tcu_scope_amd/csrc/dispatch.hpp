@@ -40,6 +40,8 @@ struct Options {
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
+  int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
+  int gemm_split_tail = 1;     // spread the K steps of the tiles of a last, partly filled round of the GEMM grid over all compute units: 0 never, 1 where it pays, 2 always
 };
 inline Options &options() {
   static Options o;
@@ -59,6 +61,8 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_waves") o.gemv_waves = value;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
+  else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
+  else if (n == "compute_units") o.compute_units = value < 1 ? 1 : value;
   else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
   return TCU_OK;
 }
@@ -840,8 +844,29 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
     if (direct_lds > 0 && K <= ((size_t)1 << 22)) {
       // the 16x16x32 kernel moves four adjacent outputs per access (16 bytes of fp32, 8 of fp16)
       const bool al4 = ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & (4 * sizeof(OUT) - 1)) == 0;
-      if (direct_lds == 66 && K % 64 == 0 && al4)
-        launch(gemm_dlds_a3b2_m16_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      if (direct_lds == 66 && K % 64 == 0 && al4) {
+        // the tiles of a last, sparsely filled round of the grid: their K steps are spread evenly over all compute
+        // units, in runs of at least 8 steps.  The shares cost up to 2 x 256 KiB of fp32 per block written and read
+        // back, which pays while the round is at most a third full and a tile takes long enough (8192^3 sizes, same
+        // run, with / without: 7168^3, 784 tiles on 256 units, 625 / 698 us; 6144^3 413 / 455; 9216^3 1300 / 1382;
+        // but 5120^3, 400 tiles, 340 / 262; 3072^3 128 / 87; 9728^3 1600 / 1522)
+        const size_t units = (size_t)options().compute_units, tail = grid % units, steps = K / 64;
+        const int mode = options().gemm_split_tail;  // 0 never, 1 by the rule above, 2 whenever there is a tail
+        if (tail && steps >= 16 && (mode == 2 || (mode == 1 && tail * 3 <= units && steps >= 64))) {
+          const size_t full = grid - tail, total = tail * steps;
+          size_t blocks = total / 8 < units ? total / 8 : units;
+          const size_t run = (total + blocks - 1) / blocks;  // <= steps, as tail < units
+          blocks = (total + run - 1) / run;
+          float *ws = static_cast<float *>(stream_alloc(2 * blocks * (size_t)(kGemmBigBM * kGemmBigBN) * sizeof(float), stream));
+          if (ws) {
+            launch(gemm_dlds_a3b2_m16_kernel<OUT>, (unsigned)(full + blocks), 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)full, (unsigned)run, ws);
+            launch(gemm_split_fixup_kernel<OUT>, (unsigned)(tail * 64), 256u, stream, static_cast<const float *>(ws), c, d, M, N, K, alpha, beta, (unsigned)full, (unsigned)run);
+            stream_free(ws, stream);
+            return TCU_OK;
+          }
+        }
+        launch(gemm_dlds_a3b2_m16_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)grid, 1u, static_cast<float *>(nullptr));
+      }
       else if (direct_lds >= 65 && K % 64 == 0)
         launch(gemm_dlds_a3b2_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       else if (direct_lds >= 64 && K % 64 == 0)

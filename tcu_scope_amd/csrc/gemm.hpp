@@ -721,8 +721,12 @@ TCU_DEVICE void gemm_store_strip16(OUT *D, const OUT *C, size_t ldc, size_t row0
 // shape against 1600 in the other (normally distributed inputs, 40 ms launches), and the
 // kernel is limited by power, not by issue slots.  C and D must be aligned to four outputs
 // (16 bytes of fp32, 8 of fp16).
+// One tile (or, with share != nullptr, the K steps step0 .. step0 + steps - 1 of one tile, whose raw fp32
+// accumulators go to `share` as a 256 x 256 row-major tile).  May be called several times by a block:
+// every wave waits for its own transfers before it leaves, and nothing reads LDS after the last barrier.
 template <typename OUT>
-__global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t N, size_t K, size_t tile_m, size_t tile_n, size_t step0, size_t steps,
+                                   float *share, float alpha, float beta) {
   constexpr int BK = 64, ROWH = BK, CPR = 8, RPT = 8, RS = 1, SUB = 2, NA = 3, NB = 2;
   constexpr int OPH = kGemmBigBM * ROWH;     // halves per operand per stage
   constexpr int TPW = kGemmBigBM / RPT / 4;  // transfer instructions per wave, operand and step (8)
@@ -730,10 +734,7 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *
   __shared__ __attribute__((aligned(1024))) half_t lds_b[NB][OPH];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  size_t tile_m, tile_n;
-  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, blockIdx.x, &tile_m, &tile_n);
   const size_t k_chunks = K / 8;
-  const size_t steps = K / BK;
   uint32_t goff[TPW];
 #pragma unroll
   for (int t = 0; t < TPW; t++) {
@@ -742,8 +743,8 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *
     goff[t] = (uint32_t)(((size_t)row * k_chunks + chunk) * 16);
   }
   constexpr lds_addr_t STAGE = OPH * 2, TBYTES = 1024, STEPB = BK * 2;
-  const char *ga = reinterpret_cast<const char *>(A + tile_m * kGemmBigBM * k_chunks);
-  const char *gb = reinterpret_cast<const char *>(B + tile_n * kGemmBigBN * k_chunks);
+  const char *ga = reinterpret_cast<const char *>(A + tile_m * kGemmBigBM * k_chunks) + step0 * STEPB;
+  const char *gb = reinterpret_cast<const char *>(B + tile_n * kGemmBigBN * k_chunks) + step0 * STEPB;
   const lds_addr_t ta = wave_uniform(lds_address_of(&lds_a[0][0]) + wave * TPW * TBYTES);
   const lds_addr_t tb = wave_uniform(lds_address_of(&lds_b[0][0]) + wave * TPW * TBYTES);
   auto issue_a = [&](size_t step, int buf, int t) { load_chunk_to_lds(ga + (step < steps ? step : steps - 1) * STEPB, goff[t], ta + buf * STAGE + t * TBYTES); };
@@ -822,7 +823,76 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *
     cb = nb;
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
-  gemm_store_strip16(D, C, N, tile_m * kGemmBigBM + wm * 128, tile_n * kGemmBigBN + wn * 128, acc, lane, alpha, beta);
+  if (share != nullptr)
+    gemm_store_strip16<float>(share, nullptr, kGemmBigBN, wm * 128, wn * 128, acc, lane, 1.0f, 0.0f);
+  else
+    gemm_store_strip16(D, C, N, tile_m * kGemmBigBM + wm * 128, tile_n * kGemmBigBN + wn * 128, acc, lane, alpha, beta);
+}
+
+// Blocks 0 .. full_tiles-1 take one tile each.  With T tiles on a chip that runs `units` blocks at a
+// time, the last T % units tiles would cost a whole round of the kernel's time however few they are:
+// their K steps, laid end to end (tile after tile), are instead cut into runs of `run` steps, one per
+// block of the rest of the grid, so that every compute unit gets the same share of the tail.  A run
+// covers the end of one tile and the start of the next at most (run <= K steps per tile); block j of
+// the tail stores its raw accumulators for the two at ws + (2 j + 0 or 1) * 65536 floats, and
+// gemm_split_fixup_kernel adds the shares of a tile in block order and applies alpha, beta and C.
+// full_tiles = grid size turns this off.
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta,
+                                                                 unsigned full_tiles, unsigned run, float *ws) {
+  const size_t tiles_m = M / kGemmBigBM, tiles_n = N / kGemmBigBN, steps = K / 64;
+  size_t tile_m, tile_n;
+  if (blockIdx.x < full_tiles) {  // block-uniform
+    gemm_tile_of_block(tiles_m, tiles_n, blockIdx.x, &tile_m, &tile_n);
+    gemm_a3b2_m16_tile(A, B, C, D, N, K, tile_m, tile_n, 0, steps, static_cast<float *>(nullptr), alpha, beta);
+    return;
+  }
+  const size_t j = blockIdx.x - full_tiles, total = (tiles_m * tiles_n - full_tiles) * steps;
+  size_t at = j * run;
+  const size_t end = at + run < total ? at + run : total;
+  for (int part = 0; at < end; part++) {
+    const size_t t = at / steps, k0 = at % steps;
+    const size_t len = end - at < steps - k0 ? end - at : steps - k0;
+    gemm_tile_of_block(tiles_m, tiles_n, full_tiles + t, &tile_m, &tile_n);
+    gemm_a3b2_m16_tile(A, B, C, D, N, K, tile_m, tile_n, k0, len, ws + (2 * j + part) * (size_t)(kGemmBigBM * kGemmBigBN), alpha, beta);
+    at += len;
+  }
+}
+
+// Second half of the K-split tail: tail tile t (tile id full_tiles + t) = alpha * (sum of its shares, in
+// block order) + beta * C.  One thread per four adjacent outputs, 64 blocks of 256 threads per tile.
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemm_split_fixup_kernel(const float *__restrict__ ws, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta, unsigned full_tiles, unsigned run) {
+  const size_t t = blockIdx.x / 64, steps = K / 64;
+  const int row = (int)(blockIdx.x % 64) * 4 + (int)(threadIdx.x >> 6), col = (int)(threadIdx.x & 63) * 4;
+  size_t tile_m, tile_n;
+  gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, full_tiles + t, &tile_m, &tile_n);
+  const size_t first = t * steps / run, last = ((t + 1) * steps - 1) / run;  // blocks of the tail with a share of this tile
+  float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (size_t j = first; j <= last; j++) {
+    const size_t part = j * run / steps == t ? 0 : 1;  // the tile is the first or the second that block j touches
+    sum += *reinterpret_cast<const float4_t *>(ws + (2 * j + part) * (size_t)(kGemmBigBM * kGemmBigBN) + (size_t)row * kGemmBigBN + col);
+  }
+  const size_t o = (tile_m * kGemmBigBM + row) * N + tile_n * kGemmBigBN + col;
+  float4_t r = alpha * sum;
+  if constexpr (sizeof(OUT) == 4) {
+    if (beta != 0.0f) r += beta * *reinterpret_cast<const float4_t *>(C + o);
+    *reinterpret_cast<float4_t *>(D + o) = r;
+  } else {
+    if (beta != 0.0f) {
+      const uint2_t c = *reinterpret_cast<const uint2_t *>(C + o);
+      const uint32_t w01 = c[0], w23 = c[1];
+      const half2_t c01 = __builtin_bit_cast(half2_t, w01), c23 = __builtin_bit_cast(half2_t, w23);
+      r[0] += beta * (float)c01[0];
+      r[1] += beta * (float)c01[1];
+      r[2] += beta * (float)c23[0];
+      r[3] += beta * (float)c23[1];
+    }
+    uint2_t v;
+    v[0] = pack_f16x2(r[0], r[1]);
+    v[1] = pack_f16x2(r[2], r[3]);
+    *reinterpret_cast<uint2_t *>(D + o) = v;
+  }
 }
 
 // M % 32 == 0, N % 32 == 0, K % 16 == 0; one 32 x 32 tile per wave.

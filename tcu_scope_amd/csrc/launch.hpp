@@ -37,12 +37,30 @@ inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void
   }
 }
 
-// Temporary device memory in stream order (from the device's default memory pool: after the
-// first use a request is served from the pool without a driver allocation).  The block may be
-// used by work enqueued on `stream` between the two calls.
+// Temporary device memory in stream order, from a memory pool of the library's own per device.
+// The pool keeps what it has handed out once (release threshold at its maximum): the default
+// pool gives unused memory back to the driver at every synchronisation, which turns the next
+// request into a real allocation of a millisecond or more.  The block may be used by work
+// enqueued on `stream` between stream_alloc and stream_free.
 inline void *stream_alloc(size_t bytes, void *stream) {
+  constexpr int kMaxDevices = 64;
+  static hipMemPool_t pools[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  if (!pools[dev]) {
+    hipMemPoolProps props = {};
+    props.allocType = hipMemAllocationTypePinned;
+    props.handleTypes = hipMemHandleTypeNone;
+    props.location.type = hipMemLocationTypeDevice;
+    props.location.id = dev;
+    hipMemPool_t pool = nullptr;
+    if (hipMemPoolCreate(&pool, &props) != hipSuccess) return nullptr;
+    uint64_t keep = ~uint64_t{0};
+    (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
+    pools[dev] = pool;
+  }
   void *p = nullptr;
-  if (hipMallocAsync(&p, bytes, static_cast<hipStream_t>(stream)) != hipSuccess) return nullptr;
+  if (hipMallocFromPoolAsync(&p, bytes, pools[dev], static_cast<hipStream_t>(stream)) != hipSuccess) return nullptr;
   return p;
 }
 inline void stream_free(void *p, void *stream) { (void)hipFreeAsync(p, static_cast<hipStream_t>(stream)); }

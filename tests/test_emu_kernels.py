@@ -290,6 +290,23 @@ def test_gemv_gemm_and_generator(emu, oracle):
             Dh = copy_in(C0.astype(np.float16).view(np.uint16))  # in place: C == D
             rc = emu.emu_gemm_f16_f16(Ai.ctypes.data, Bi.ctypes.data, Dh.ctypes.data, Dh.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(Dh.reshape(M, N), ref.astype(np.float16).view(np.uint16)), (direct_lds, bk64, depth)
+        # the K-split tail on a device of 4 units: 7 tiles -> the 48 K steps of the last 3 in 4 runs of 12, three of
+        # which cross from one tile into the next; 9 tiles -> the last one in 2 runs (tile ids regrouped for 8 XCDs);
+        # fp32 outputs in place, fp16 outputs with C
+        assert emu.emu_set_option(b"gemm_direct_lds", -1) == 0 and emu.emu_set_option(b"compute_units", 4) == 0 and emu.emu_set_option(b"gemm_split_tail", 2) == 0
+        for Ms, Ns, Ks in ((1792, 256, 1024), (768, 768, 1024)):
+            As, Bs = oracle.generate_f16(Ms * Ks, 15, oracle.DIST_SMALLINT), oracle.generate_f16(Ns * Ks, 16, oracle.DIST_SMALLINT)
+            Cs = (np.arange(Ms * Ns) % 5).astype(np.float32)
+            Asi, Bsi = copy_in(As), copy_in(Bs)
+            refs = oracle.gemm_f64(As, Bs, Ms, Ns, Ks, 0.5, 2.0, Cs)
+            Ds = copy_in(Cs, np.float32)
+            rc = emu.emu_gemm_f16_f32(Asi.ctypes.data, Bsi.ctypes.data, Ds.ctypes.data, Ds.ctypes.data, Ms, Ns, Ks, 0.5, 2.0, V_BLOCK)
+            assert rc == 0 and np.array_equal(Ds.reshape(Ms, Ns).astype(np.float64), refs), ("split tail", Ms, Ns, Ks)
+            Chs = copy_in(Cs.astype(np.float16).view(np.uint16))
+            Dhs = aligned(Ms * Ns, np.uint16, 0x7e00)
+            rc = emu.emu_gemm_f16_f16(Asi.ctypes.data, Bsi.ctypes.data, Chs.ctypes.data, Dhs.ctypes.data, Ms, Ns, Ks, 0.5, 2.0, V_BLOCK)
+            assert rc == 0 and np.array_equal(Dhs.reshape(Ms, Ns), refs.astype(np.float16).view(np.uint16)), ("split tail fp16", Ms, Ns, Ks)
+        assert emu.emu_set_option(b"compute_units", 256) == 0 and emu.emu_set_option(b"gemm_split_tail", 1) == 0
         # 128 x 128 tiles: the transfer kernel (K step 64 and 32) and the register-staged one
         assert emu.emu_set_option(b"gemm_big_tiles", 0) == 0
         for direct_lds, Ks in ((-1, 192), (-1, 96), (0, 96)):
@@ -300,5 +317,5 @@ def test_gemv_gemm_and_generator(emu, oracle):
             rc = emu.emu_gemm_f16_f32(A2i.ctypes.data, B2i.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, Ks, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A2, B2, M, N, Ks, 1.5, 2.0, C0)), (direct_lds, Ks)
     finally:
-        for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1)):
+        for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1), (b"compute_units", 256), (b"gemm_split_tail", 1)):
             emu.emu_set_option(name, val)

@@ -217,6 +217,29 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             torch.cuda.synchronize()
             assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("offset", off32)
             assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("offset fp16", off16)
+        # the K-split tail of the grid: 264 = 256 + 8 tiles (11 x 24), the last 8 in 16 shares each (K = 8192: 128 steps
+        # of 64, shares of at least 8), fp32 outputs in place and fp16 outputs.  Integer inputs: the result must equal,
+        # bit for bit, that of the same launch with the split switched off, and the oracle on four rows of every tile row
+        Ms, Ns, Ks = 2816, 6144, 8192
+        A = oracle.generate_f16(Ms * Ks, 41, oracle.DIST_SMALLINT)
+        B = oracle.generate_f16(Ns * Ks, 42, oracle.DIST_SMALLINT)
+        Cs = (np.arange(Ms * Ns) % 5).astype(np.float32)
+        Ad, Bd = to_dev(A).view(Ms, Ks), to_dev(B).view(Ns, Ks)
+        got = {}
+        for split in (1, 0):
+            tcu.set_option("gemm_split_tail", split)
+            Cd = torch.from_numpy(Cs.copy()).cuda().view(Ms, Ns)
+            tcu.gemm(Ad, Bd, 0.5, -1.0, C=Cd, out=Cd)
+            Ch = torch.from_numpy(Cs.astype(np.float16)).cuda().view(Ms, Ns)
+            Dh = tcu.gemm(Ad, Bd, 0.5, -1.0, C=Ch)
+            torch.cuda.synchronize()
+            got[split] = (Cd.cpu().numpy(), Dh.cpu().numpy().view(np.uint16))
+        tcu.set_option("gemm_split_tail", 1)
+        assert np.array_equal(got[1][0], got[0][0]) and np.array_equal(got[1][1], got[0][1]), "split tail vs unsplit"
+        for tm in range(Ms // 256):
+            ref = oracle.gemm_f64(A, B, Ms, Ns, Ks, 0.5, -1.0, Cs, row0=tm * 256 + 37, rows=4)
+            assert np.array_equal(got[1][0][tm * 256 + 37:tm * 256 + 41].astype(np.float64), ref), ("split tail", tm)
+            assert np.array_equal(got[1][1][tm * 256 + 37:tm * 256 + 41], ref.astype(np.float16).view(np.uint16)), ("split tail fp16", tm)
         # 128 x 128 tiles: the transfer kernel (K step 64 and 32) and the register-staged one
         tcu.set_option("gemm_big_tiles", 0)
         tcu.set_option("gemm_bk64", 0)
@@ -232,6 +255,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             assert np.array_equal(Cd.cpu().numpy().astype(np.float64), oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)), ("128 tiles", direct_lds, K)
             assert np.array_equal(Dh.cpu().numpy().view(np.uint16), oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0).astype(np.float16).view(np.uint16)), ("128 tiles fp16", direct_lds, K)
     finally:
+        tcu.set_option("gemm_split_tail", 1)
         tcu.set_option("gemm_direct_lds", -1)
         tcu.set_option("gemm_bk64", 0)
         tcu.set_option("gemm_depth", 4)
