@@ -835,7 +835,7 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
 // block of the rest of the grid, so that every compute unit gets the same share of the tail.  A run
 // covers the end of one tile and the start of the next at most (run <= K steps per tile); block j of
 // the tail stores its raw accumulators for the two at ws + (2 j + 0 or 1) * 65536 floats, and
-// gemm_split_fixup_kernel adds the shares of a tile in block order and applies alpha, beta and C.
+// gemm_split_fixup_kernel adds the shares of a tile in a fixed order and applies alpha, beta and C.
 // full_tiles = grid size turns this off.
 template <typename OUT>
 __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta,
@@ -859,8 +859,8 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *
   }
 }
 
-// Second half of the K-split tail: tail tile t (tile id full_tiles + t) = alpha * (sum of its shares, in
-// block order) + beta * C.  One thread per four adjacent outputs, 64 blocks of 256 threads per tile.
+// Second half of the K-split tail: tail tile t (tile id full_tiles + t) = alpha * (sum of its shares, in a
+// fixed order) + beta * C.  One thread per four adjacent outputs, 64 blocks of 256 threads per tile.
 template <typename OUT>
 __global__ __launch_bounds__(256) void gemm_split_fixup_kernel(const float *__restrict__ ws, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta, unsigned full_tiles, unsigned run) {
   const size_t t = blockIdx.x / 64, steps = K / 64;
@@ -868,11 +868,21 @@ __global__ __launch_bounds__(256) void gemm_split_fixup_kernel(const float *__re
   size_t tile_m, tile_n;
   gemm_tile_of_block(M / kGemmBigBM, N / kGemmBigBN, full_tiles + t, &tile_m, &tile_n);
   const size_t first = t * steps / run, last = ((t + 1) * steps - 1) / run;  // blocks of the tail with a share of this tile
-  float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (size_t j = first; j <= last; j++) {
-    const size_t part = j * run / steps == t ? 0 : 1;  // the tile is the first or the second that block j touches
-    sum += *reinterpret_cast<const float4_t *>(ws + (2 * j + part) * (size_t)(kGemmBigBM * kGemmBigBN) + (size_t)row * kGemmBigBN + col);
+  // only block `first` can have begun in the previous tile (this tile is then the second it touches); four
+  // independent partial sums keep four loads in flight, combined in a fixed order
+  constexpr size_t SHARE = (size_t)kGemmBigBM * kGemmBigBN;
+  const float *p = ws + (size_t)row * kGemmBigBN + col;
+  float4_t s0 = *reinterpret_cast<const float4_t *>(p + (2 * first + (first * run < t * steps ? 1 : 0)) * SHARE);
+  float4_t s1 = {0.0f, 0.0f, 0.0f, 0.0f}, s2 = s1, s3 = s1;
+  size_t j = first + 1;
+  for (; j + 3 <= last; j += 4) {
+    s1 += *reinterpret_cast<const float4_t *>(p + 2 * j * SHARE);
+    s2 += *reinterpret_cast<const float4_t *>(p + 2 * (j + 1) * SHARE);
+    s3 += *reinterpret_cast<const float4_t *>(p + 2 * (j + 2) * SHARE);
+    s0 += *reinterpret_cast<const float4_t *>(p + 2 * (j + 3) * SHARE);
   }
+  for (; j <= last; j++) s1 += *reinterpret_cast<const float4_t *>(p + 2 * j * SHARE);
+  const float4_t sum = (s0 + s1) + (s2 + s3);
   const size_t o = (tile_m * kGemmBigBM + row) * N + tile_n * kGemmBigBN + col;
   float4_t r = alpha * sum;
   if constexpr (sizeof(OUT) == 4) {
