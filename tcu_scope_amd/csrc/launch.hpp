@@ -54,13 +54,19 @@ inline void *stream_alloc(size_t bytes, void *stream) {
     props.location.type = hipMemLocationTypeDevice;
     props.location.id = dev;
     hipMemPool_t pool = nullptr;
-    if (hipMemPoolCreate(&pool, &props) != hipSuccess) return nullptr;
+    if (hipMemPoolCreate(&pool, &props) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
     uint64_t keep = ~uint64_t{0};
     (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
     pools[dev] = pool;
   }
   void *p = nullptr;
-  if (hipMallocFromPoolAsync(&p, bytes, pools[dev], static_cast<hipStream_t>(stream)) != hipSuccess) return nullptr;
+  if (hipMallocFromPoolAsync(&p, bytes, pools[dev], static_cast<hipStream_t>(stream)) != hipSuccess) {
+    (void)hipGetLastError();  // the caller reports the failure or does without; a later launch check must not see it
+    return nullptr;
+  }
   return p;
 }
 inline void stream_free(void *p, void *stream) { (void)hipFreeAsync(p, static_cast<hipStream_t>(stream)); }
