@@ -302,6 +302,8 @@ def test_gemv_gemm_and_generator(emu, oracle):
             Ds = copy_in(Cs, np.float32)
             rc = emu.emu_gemm_f16_f32(Asi.ctypes.data, Bsi.ctypes.data, Ds.ctypes.data, Ds.ctypes.data, Ms, Ns, Ks, 0.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(Ds.reshape(Ms, Ns).astype(np.float64), refs), ("split tail", Ms, Ns, Ks)
+            if Ms == Ns:
+                continue  # fp16 outputs once is enough: the two cases differ in the tile mapping only
             Chs = copy_in(Cs.astype(np.float16).view(np.uint16))
             Dhs = aligned(Ms * Ns, np.uint16, 0x7e00)
             rc = emu.emu_gemm_f16_f16(Asi.ctypes.data, Bsi.ctypes.data, Chs.ctypes.data, Dhs.ctypes.data, Ms, Ns, Ks, 0.5, 2.0, V_BLOCK)
