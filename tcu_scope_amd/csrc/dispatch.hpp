@@ -343,6 +343,11 @@ inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t nu
     g_log2 = 1;
     while (g_log2 < 6 && ((size_t)8 << g_log2) < expected) g_log2++;
   }
+  // 128 to 512 halves expected: half as many lanes (at most 16), so that a segment takes two to four rounds and a
+  // lane has as many loads in flight, while a round still reads 128 or 256 contiguous bytes (N = 2^28, S = 128 /
+  // 256 / 512: 82 / 79 / 78 us against 104 / 102 / 102 with one chunk per lane; with 4 or 2 lanes, S = 64 / 32,
+  // a round reads half a cache line per segment and the time goes up to 151 / 157 us from 105 / 108)
+  if (expected >= 128 && expected <= 512) g_log2 = g_log2 - 1 < 4 ? g_log2 - 1 : 4;
   // one chunk per lane in flight is too little (120 us at N = 2^28): up to 1024 halves expected, a block takes two
   // runs of segments and has the first load of both in flight (107-111 us)
   const int passes = expected && expected <= 1024 ? 2 : 1;  // four passes measure worse (131 us: registers)
