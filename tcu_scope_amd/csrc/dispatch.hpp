@@ -337,6 +337,20 @@ inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t nu
     stream_free(partials, stream);
     return TCU_OK;
   }
+  // 4096 halves and more expected: a block per segment, about 32 halves per thread (128 to 512 threads, 1024 from 65536 halves on), the
+  // result written by the block itself.  N = 2^28 against a wave per segment: S = 4096 76 vs 78.5 us, 16384 77.4 vs
+  // 82.7, 65536 78.4 vs 89.5 (2^28 / S long-lived waves fill the chip unevenly); at 2048 the wave is faster (75.5 vs 88)
+  if (expected >= 4096) {
+    unsigned threads = 128;
+    while (threads < 512 && (size_t)threads * 32 < expected) threads *= 2;
+    if (expected >= 65536) threads = 1024;  // 1024 threads lose below that (S = 16384: 97 us)
+    if (num_segments > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_offsets_f16: grid exceeds the launch limit");
+    if (nt)
+      launch(seg_reduce_offsets_sliced_kernel<OFF, true, true>, (unsigned)num_segments, threads, stream, in, reinterpret_cast<float *>(out), begin, end, 1u, vector);
+    else
+      launch(seg_reduce_offsets_sliced_kernel<OFF, false, true>, (unsigned)num_segments, threads, stream, in, reinterpret_cast<float *>(out), begin, end, 1u, vector);
+    return TCU_OK;
+  }
   // lanes per segment: about one 128-bit chunk per lane for the expected length, a whole wave when unknown
   int g_log2 = 6;
   if (expected) {

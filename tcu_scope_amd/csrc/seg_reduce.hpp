@@ -391,7 +391,7 @@ __global__ __launch_bounds__(256) void seg_reduce_offsets_kernel(const uint16_t 
 // Long segments: `slices` blocks share a segment.  Block (segment j, slice p) adds the p-th of
 // `slices` equal parts of the segment (part length rounded up to whole 128-bit chunks) and
 // writes an fp32 partial to partial[j * slices + p]; a second kernel adds the partials.
-template <typename OFF, bool NT>
+template <typename OFF, bool NT, bool DIRECT = false>
 __global__ __launch_bounds__(kMaxBlock) void seg_reduce_offsets_sliced_kernel(const uint16_t *__restrict__ in, float *__restrict__ partial_out, const OFF *__restrict__ begin,
                                                                               const OFF *__restrict__ end, unsigned slices, int vector) {
   __shared__ float partial[kMaxWaves];
@@ -415,7 +415,10 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_offsets_sliced_kernel(co
   if (threadIdx.x == 0) {
     float s = 0.0f;
     for (unsigned w = 0; w < (blockDim.x >> 6); w++) s += partial[w];
-    partial_out[blockIdx.x] = s;
+    if constexpr (DIRECT)  // one block per segment: partial_out is the fp16 result array
+      reinterpret_cast<uint16_t *>(partial_out)[blockIdx.x] = f16_bits(s);
+    else
+      partial_out[blockIdx.x] = s;
   }
 }
 

@@ -353,7 +353,7 @@ def test_segmented_reduction_over_offsets(tcu, oracle):
         exact = np.abs(want_grid).max() < 4096 and max_len <= 20000
         for dtype in (torch.int32, torch.int64):
             bd, ed = torch.from_numpy(begin).to(dtype).cuda(), torch.from_numpy(end).to(dtype).cuda()
-            for expected in (0, 16, 100, 512, 1 << 16, 1 << 17, 1 << 20):
+            for expected in (0, 16, 100, 512, 4096, 20000, 1 << 16, 1 << 17, 1 << 20):
                 got = to_host(tcu.seg_reduce_offsets(xd, bd, ed, expected_segment_size=expected)).view(np.float16).astype(np.float64)
                 allow = 2 * np.maximum(np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64), 2.0 ** -24) + 1e-3 * np.sqrt(length)
                 bad = np.abs(got - ref) > allow
