@@ -534,6 +534,9 @@ inline int seg_scan_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_
     g_log2 = 1;
     while (g_log2 < 4 && ((size_t)8 << g_log2) < expected) g_log2++;
   }
+  // 65 to 128 halves expected: 8 lanes and two rounds instead of 16 and one (N = 2^28, S = 128: 168 vs 174 us;
+  // fewer lanes lose at every other length: half a cache line per segment and round, or too many rounds)
+  if (expected > 64 && expected <= 128) g_log2 = 3;
   const size_t threads = num_segments << g_log2;
   const size_t grid = (threads + 255) / 256;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_offsets_f16: grid exceeds the launch limit");
