@@ -497,18 +497,19 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
 
 template <typename OFF>
 inline int seg_scan_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_segments, const OFF *begin, const OFF *end, size_t expected, void *stream) {
-  // expected length of 2048 halves and more: a block per run of at most about 65536 halves of one
-  // segment, one 128-bit chunk per thread and round (256 ... 1024 threads); with more than one run
+  // expected length of 1024 halves and more: a block per run of at most about 65536 halves of one
+  // segment, one 128-bit chunk per thread and round (64 ... 1024 threads); with more than one run
   // per segment the runs' sums are taken first (fp32, stream-ordered temporary memory) and turned
   // into carry-ins.  (Groups of 16 lanes walking a segment: 226-313 us for 2048 ... 32768 at
   // N = 2^28 and milliseconds beyond, against 175-200 and 290 us this way.)
-  if (expected >= 2048) {
+  if (expected >= 1024) {
     const int vec = aligned16(in) && aligned16(out) ? 1 : 0;
     const bool ntl = options().nontemporal;
     size_t slices = (expected + 65535) / 65536;
     if (slices > 4096) slices = 4096;
-    unsigned threads = 256;
-    while (threads < 1024 && (size_t)threads * 16 < expected) threads *= 2;  // two rounds per block measure better than one
+    // two to four rounds per block measure best (N = 2^28: S = 1024 with 64 threads 165 us, 180 with groups of 16
+    // lanes; S = 2048 with 128 threads 164, with 256 184; S = 4096 with 128 threads 167.5, with 256 173)
+    const unsigned threads = expected < 2048 ? 64 : expected < 8192 ? 128 : expected <= 8192 ? 512 : 1024;
     const size_t blocks = num_segments * slices;
     if (blocks > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_offsets_f16: grid exceeds the launch limit");
     float *sums = nullptr;

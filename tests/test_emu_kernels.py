@@ -166,7 +166,7 @@ def test_segmented_scan_over_offsets(emu, oracle):
     n = 40000
     x = oracle.generate_f16(n, 10, oracle.DIST_GRID)  # exact partial sums: results are fixed bit for bit
     xi = copy_in(x)
-    for nseg, expected, bits in ((1500, 16, 32), (1500, 0, 64), (300, 64, 32), (300, 100, 64), (40, 1000, 64), (7, 0, 32), (5, 1 << 16, 32), (4, 3 << 16, 64), (3, 1 << 19, 32)):
+    for nseg, expected, bits in ((1500, 16, 32), (1500, 0, 64), (300, 64, 32), (300, 100, 64), (40, 1000, 64), (40, 1500, 32), (40, 3000, 64), (7, 0, 32), (5, 1 << 16, 32), (4, 3 << 16, 64), (3, 1 << 19, 32)):
         begin, end = disjoint_offsets(rng, n, nseg)
         w64 = oracle.seg_scan_offsets_f64(x, begin, end)
         inside = ~np.isnan(w64)
