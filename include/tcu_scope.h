@@ -12,9 +12,17 @@
  * become run-time arguments.
  *
  * Conventions
- *   - every pointer named d_* is DEVICE memory owned by the caller; nothing here
- *     allocates, frees or retains it.  Reduction/scan inputs and outputs must be
- *     16-byte aligned unless the variant is TCU_VARIANT_AUTO.
+ *   - every pointer named d_* is DEVICE memory owned by the caller; nothing here frees or
+ *     retains it.  Reduction/scan inputs and outputs must be 16-byte aligned unless the
+ *     variant is TCU_VARIANT_AUTO.
+ *   - temporary device memory: the kernels of the common sizes need none.  A few paths take
+ *     some in stream order from a memory pool the library keeps per device (it is given back
+ *     to the pool when the enqueued work has run, and the pool keeps it for the next call):
+ *     tcu_seg_reduce_f16 with segments of 2^20 halves and more and tcu_seg_scan_f16 from 2^21
+ *     (4 or 8 bytes per 65536 input halves), the *_offsets_f16 entry points with expected
+ *     segment lengths of 2^17 and more (4 bytes per 65536 halves), and tcu_gemm_* when the
+ *     last round of output tiles is sparsely filled (up to 128 MiB).  The full-array entry
+ *     points work in the caller's workspace.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
  *     enqueue work; they do not synchronise.
  *   - the return value is a tcu_status; on failure tcu_last_error() describes it (per
@@ -64,7 +72,10 @@ typedef enum {
   TCU_FULL_AUTO = 0,
   TCU_FULL_SINGLE_PASS = 1, /* one kernel: atomic ticket + carry (reduce), decoupled look-back (scan);
                                replaces reference *_ATOMIC_W_BLOCK_SYNC / _ATOMIC_BALLOT / _CG */
-  TCU_FULL_MULTI_KERNEL = 2 /* reference "2 kernels" (reduce) / "3 kernels" (scan) sequences */
+  TCU_FULL_MULTI_KERNEL = 2, /* reference "2 kernels" (reduce) / "3 kernels" (scan) sequences */
+  TCU_FULL_MFMA = 0x100     /* flag, OR-ed onto a strategy: the single-pass kernels add (reduce: D += A * ones) and scan
+                               (U * X + carry) on the matrix unit, as the reference's *_CG / *_ATOMIC_* kernels do on
+                               WMMA fragments; without it the DPP flavour runs.  AUTO | MFMA runs SINGLE_PASS | MFMA */
 } tcu_full_strategy;
 
 typedef enum {
@@ -103,6 +114,13 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *   "compute_units"   blocks of the big-tile GEMM kernel the device runs at a time (set by tcu_init; for tests)
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
+ *   "lookback_poll_limit"  default 2^20 (negative restores it): how often a block of a single-pass full-array
+ *                     kernel (and of the look-back path of tcu_seg_scan_f16 for segments of 2^21 halves and more)
+ *                     looks again for a value another block has not published yet before it gives up.  Giving up
+ *                     never yields a finite wrong number: the reduction's result, or the scan's outputs from the
+ *                     waiting partition to the end of the array (or segment), become NaN
+ *   "test_mute_partition"  default 0; p > 0: partition p - 1 of those kernels publishes nothing, so every wait
+ *                     for it expires (for tests of the rule above; all kernels still run to their end)
  * Unknown names return TCU_ERR_INVALID_ARG. */
 int tcu_set_option(const char *name, int value);
 
@@ -232,7 +250,7 @@ int tcu_stream_probe(void *d_dst, const void *d_src, size_t bytes, int mode, int
 int tcu_time_next_launch(void *start_event, void *stop_event);
 /* Runs every cross-lane primitive the kernels rely on (MFMA 16x16x32 / 32x32x16 operand
  * layouts, DPP controls, lane swaps) on lane-indexed inputs and writes the raw results
- * to d_out (fp32 / u32 words; see tcu_scope_amd/csrc/probe.hpp for the record layout).
+ * to d_out (fp32 / u32 words; lane_probe_kernel in tcu_scope_amd/csrc/util_kernels.hpp has the record layout).
  * *out_words receives the number of 32-bit words (call with d_out == NULL to query). */
 int tcu_lane_probe(void *d_out, size_t *out_words, void *stream);
 

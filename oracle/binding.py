@@ -47,6 +47,7 @@ def lib():
         L.tcu_oracle_generate_f16.argtypes = [u16p, sz, c.c_uint64, c.c_int]
         L.tcu_oracle_generate_f16_range.argtypes = [u16p, sz, sz, c.c_uint64, c.c_int]
         L.tcu_oracle_fill_f16.argtypes = [u16p, c.c_float, sz]
+        L.tcu_oracle_convert_f32_to_f16.argtypes = [u16p, f32p, sz]
         for name in ("seg_reduce_ref", "seg_scan_ref"):
             getattr(L, "tcu_oracle_" + name).argtypes = [u16p, u16p, sz, sz]
             getattr(L, "tcu_oracle_" + name + "_mt").argtypes = [u16p, u16p, sz, sz, c.c_int]
@@ -86,6 +87,14 @@ def f16_to_f32(h):
 
 def f32_to_f16(f):
     return lib().tcu_oracle_f32_to_f16(float(np.float32(f)))
+
+
+def f32_to_f16_array(values):
+    """Element-wise float32 -> fp16 bit patterns (the reference's convertFp32ToFp16)."""
+    a = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty(a.shape, dtype=np.uint16)
+    lib().tcu_oracle_convert_f32_to_f16(_p(out, ctypes.c_uint16), _p(a, ctypes.c_float), a.size)
+    return out
 
 
 def f64_to_f16(d):

@@ -165,6 +165,10 @@ void tcu_oracle_fill_f16(uint16_t *out, float value, size_t n) {
   for (size_t i = 0; i < n; i++) out[i] = h;
 }
 
+void tcu_oracle_convert_f32_to_f16(uint16_t *out, const float *in, size_t n) {
+  for (size_t i = 0; i < n; i++) out[i] = tcu_oracle_f32_to_f16(in[i]);
+}
+
 /* ------------------------------------------------------------------------------------ */
 /* reference CPU path: fp32 sequential running sum, fp16 out                             */
 /* ------------------------------------------------------------------------------------ */

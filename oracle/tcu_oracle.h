@@ -67,6 +67,9 @@ void tcu_oracle_generate_f16_range(uint16_t *out, size_t first, size_t n, uint64
 /* Constant fill with a float -> half cast: reference cuda_memory_set / setFP16,
  * src/utils/cuda_helpers.cuh:123-181. */
 void tcu_oracle_fill_f16(uint16_t *out, float value, size_t n);
+/* Element-wise float -> half cast (round to nearest even): reference convertFp32ToFp16,
+ * src/utils/cuda_helpers.cuh:116-121. */
+void tcu_oracle_convert_f32_to_f16(uint16_t *out, const float *in, size_t n);
 
 /* ---- reference CPU path (fp32 sequential, fp16 out) ------------------------------- */
 /* reference src/reduction/seg_wmma_16.cu:77-104, seg_wmma_256n.cu:85-121 */

@@ -11,6 +11,7 @@ from .binding import (  # noqa: F401
     VARIANTS,
     Variant,
     FullStrategy,
+    FULL_MFMA,
     Dist,
     add_partial_sums,
     build,

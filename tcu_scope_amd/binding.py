@@ -38,6 +38,10 @@ class FullStrategy(enum.IntEnum):
     MULTI_KERNEL = 2
 
 
+# flag OR-ed onto a FullStrategy: the single-pass full-array kernels work on the matrix unit
+FULL_MFMA = 0x100
+
+
 class Dist(enum.IntEnum):
     UNIFORM = 0
     GRID = 1

@@ -26,6 +26,9 @@ int runtime_error(const char *what, hipError_t e) { return tcu::fail(TCU_ERR_RUN
 // Kernel launches are asynchronous; what can be caught here is a launch that the runtime
 // rejected (bad configuration, no code object for the device).
 int after_launch(const char *what, unsigned long launches_before, int rc) {
+  // events armed by tcu_time_next_launch belong to this call: if it launched nothing (a rejected
+  // argument, an empty input) they must not ride on some later, unrelated launch
+  tcu::next_launch_events() = tcu::LaunchEvents{};
   if (rc != TCU_OK || tcu::launch_count() == launches_before) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return runtime_error(what, e);

@@ -42,6 +42,8 @@ struct Options {
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
   int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
   int gemm_split_tail = 1;     // spread the K steps of the tiles of a last, partly filled round of the GEMM grid over all compute units: 0 never, 1 where it pays, 2 always
+  unsigned lookback_poll_limit = kDefaultPollLimit;  // polls of an unpublished value before a single-pass kernel gives up (results become NaN)
+  unsigned test_mute_partition = 0;                  // tests only: partition test_mute_partition - 1 of a single-pass kernel publishes nothing
 };
 inline Options &options() {
   static Options o;
@@ -63,9 +65,13 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
   else if (n == "compute_units") o.compute_units = value < 1 ? 1 : value;
+  else if (n == "lookback_poll_limit") o.lookback_poll_limit = value < 0 ? kDefaultPollLimit : (unsigned)value;
+  else if (n == "test_mute_partition") o.test_mute_partition = value < 0 ? 0u : (unsigned)value;
   else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
   return TCU_OK;
 }
+
+inline WaitPolicy wait_policy() { return WaitPolicy{options().lookback_poll_limit, options().test_mute_partition}; }
 
 inline bool is_pow2(size_t x) { return x && !(x & (x - 1)); }
 inline int ilog2(size_t x) {
@@ -234,21 +240,34 @@ inline int seg_reduce_huge(const half8_t *in, uint16_t *out, size_t num_segments
   return TCU_OK;
 }
 
-inline int seg_scan_huge(const half8_t *in, uint4_t *out, uint16_t *totals, size_t num_segments, size_t S, bool nt, void *stream) {
-  const char *what = "tcu_seg_scan_f16";
+// Where the partition descriptors of seg_scan_huge live: in stream-ordered temporary memory
+// (words == nullptr) or in a buffer the caller of the dispatcher brings (capacity in 32-bit words).
+struct ScanScratch {
+  unsigned *words = nullptr;
+  size_t capacity = 0;
+};
+
+inline int seg_scan_huge(const char *what, const half8_t *in, uint4_t *out, uint16_t *totals, size_t num_segments, size_t S, bool nt, void *stream, ScanScratch scratch) {
   const size_t pps = S / kHugePartHalves, parts = num_segments * pps;
   if (parts > kMaxGrid || pps > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
   const size_t words = 64 + 2 * parts;  // ticket counter, then one 64-bit descriptor per partition
-  unsigned *ws = static_cast<unsigned *>(stream_alloc(words * sizeof(unsigned), stream));
-  if (!ws) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partition descriptors");
+  unsigned *ws = scratch.words;
+  if (ws) {
+    if (words > scratch.capacity)
+      return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": " + std::to_string(parts) + " partitions of 65536 halves exceed the built-in scratch buffer (at most " +
+                                           std::to_string((scratch.capacity - 64) / 2) + " partitions, i.e. " + std::to_string((scratch.capacity - 64) / 2 * kHugePartHalves) + " halves per call)");
+  } else {
+    ws = static_cast<unsigned *>(stream_alloc(words * sizeof(unsigned), stream));
+    if (!ws) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partition descriptors");
+  }
   const size_t n_chunks = num_segments * S / 8;
   launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
   const int static_order = options().static_order ? 1 : 0;
   if (nt)
-    launch(full_scan_kernel<8, false, true>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals);
+    launch(full_scan_kernel<8, false, true>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy());
   else
-    launch(full_scan_kernel<8, false, false>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals);
-  stream_free(ws, stream);
+    launch(full_scan_kernel<8, false, false>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy());
+  if (!scratch.words) stream_free(ws, stream);
   return TCU_OK;
 }
 
@@ -435,10 +454,11 @@ inline void launch_scan_wave_s(int lps_log2, int u, bool nt, unsigned grid, unsi
   }
 }
 
-inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
+inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream,
+                             const char *what = "tcu_seg_scan_f16", ScanScratch scratch = ScanScratch{}) {
   SegArgs a{num_segments, segment_size, variant, tiles_per_wave, waves_per_block, false};
   bool generic = false;
-  if (int rc = validate_segmented("tcu_seg_scan_f16", d_in, d_out, a, &generic)) return rc;
+  if (int rc = validate_segmented(what, d_in, d_out, a, &generic)) return rc;
   if (num_segments == 0) return TCU_OK;
   const size_t S = segment_size, N = num_segments * S;
   const half8_t *in = static_cast<const half8_t *>(d_in);
@@ -449,11 +469,11 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   if (generic) {
     const int gw = waves_per_block ? waves_per_block : 4;
     const size_t grid = (num_segments + gw - 1) / gw;
-    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: grid exceeds the launch limit");
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     launch(seg_scan_generic_kernel, (unsigned)grid, (unsigned)gw * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), totals, num_segments, S);
     return TCU_OK;
   }
-  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeScanSegment) return seg_scan_huge(in, out, totals, num_segments, S, nt, stream);
+  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeScanSegment) return seg_scan_huge(what, in, out, totals, num_segments, S, nt, stream, scratch);
   const size_t n_chunks = N / 8;
   const Plan plan = auto_plan_scan(S);
   const bool use_block = variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant);
@@ -466,7 +486,7 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
     const size_t tiles_per_seg = S / kTileHalves;
     const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;
     const size_t grid = (num_segments + spb - 1) / spb;
-    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: grid exceeds the launch limit");
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     TCU_SWITCH_U_MFMA_NT(seg_scan_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, spb);
     return TCU_OK;
   }
@@ -480,12 +500,12 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
     tps_log2 = ilog2(S) - 9;
     const size_t tiles_per_seg = (size_t)1 << tps_log2;
     iters = tiles_per_seg > (size_t)u ? tiles_per_seg / u : 1;
-    if (iters > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: segment too long for the wave-per-segment kernel; use a block variant");
+    if (iters > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment too long for the wave-per-segment kernel; use a block variant");
   }
   const size_t per_wave = iters * u;
   const size_t waves = (tiles + per_wave - 1) / per_wave;
   const size_t grid = (waves + wpb - 1) / wpb;
-  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_f16: grid exceeds the launch limit");
+  if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
   if (a.mfma)
     launch_scan_wave_s<true>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters);
   else
@@ -621,10 +641,12 @@ inline int plan_full(const char *what, size_t segment_size, int waves_per_block,
 inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d_ws, size_t *ws_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream) {
   const char *what = "tcu_full_reduce_f16";
   if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
+  const bool mfma = (strategy & TCU_FULL_MFMA) != 0;
+  strategy &= ~TCU_FULL_MFMA;
   if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
   // AUTO with the default partition: partition sums, then one small block adds them (measured
   // 90 us at 2^28 against 96 us for the single kernel, whose workspace must be zeroed first)
-  const bool two_level = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0;
+  const bool two_level = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && !mfma;
   if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {
@@ -662,7 +684,7 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
     }
     unsigned *ws = static_cast<unsigned *>(d_ws);
     launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
-    TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, false, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws);
+    TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, mfma, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws, wait_policy());
     return TCU_OK;
   }
   // the reference's two-kernel sequence: segmented reduction into fp16 totals, then a sum of the totals
@@ -677,7 +699,7 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
   }
   if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
   if (!d_out || (n && !d_in)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
-  if (int rc = seg_reduce_dispatch(d_in, d_ws, nseg, S, S == 16 ? TCU_VARIANT_MFMA_16 : TCU_VARIANT_MFMA_16N, 0, waves_per_block, stream)) return rc;
+  if (int rc = seg_reduce_dispatch(d_in, d_ws, nseg, S, S == 16 ? TCU_VARIANT_MFMA_16 : TCU_VARIANT_MFMA_16N, 0, waves_per_block, stream)) return rc;  // the reference's sequence is built on its WMMA kernels
   launch(sum_f16_kernel, 1u, 1024u, stream, static_cast<const uint16_t *>(d_ws), static_cast<uint16_t *>(d_out), nseg);
   return TCU_OK;
 }
@@ -685,9 +707,11 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
 inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_ws, size_t *ws_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream) {
   const char *what = "tcu_full_scan_f16";
   if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
+  const bool mfma = (strategy & TCU_FULL_MFMA) != 0;
+  strategy &= ~TCU_FULL_MFMA;
   if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
   // AUTO with the default partition: the kernel that parks 4 more tiles per wave in LDS
-  const bool lds_held = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && options().scan_lds_tiles;
+  const bool lds_held = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && options().scan_lds_tiles && !mfma;
   if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {
@@ -721,12 +745,12 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
     if (lds_held) {  // partitions of 16 x 12 tiles: fewer than `parts`, same workspace layout
       const size_t big_parts = (n_tiles + 16 * 12 - 1) / (16 * 12);
       if (nt)
-        launch(full_scan_lds_kernel<8, 4, true>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0);
+        launch(full_scan_lds_kernel<8, 4, true>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy());
       else
-        launch(full_scan_lds_kernel<8, 4, false>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0);
+        launch(full_scan_lds_kernel<8, 4, false>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy());
       return TCU_OK;
     }
-    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, false, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr));
+    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, mfma, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr), wait_policy());
     return TCU_OK;
   }
   // the reference's three-kernel sequence: segmented scan + totals, exclusive scan of the totals, add

@@ -51,16 +51,26 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned *words, size_t
 // aligned) u64 partial[blocks], u64 group_sum[groups]; all zeroed before the launch.
 constexpr unsigned kFullReduceGroup = 64;
 constexpr unsigned long long kPublished = 1ull << 32;
-constexpr unsigned kPublishPollLimit = 1u << 22;
+
+// What bounds the waits of the single-pass kernels.  poll_limit: how often a wave looks again
+// for a value that has not been published yet before it gives up; giving up makes the results
+// that depend on the missing value NaN, never a finite wrong number.  mute_partition (tests
+// only, 0 = none): partition mute_partition - 1 computes its own results but publishes
+// nothing, which makes every wait for it expire while all kernels still run to their end.
+struct WaitPolicy {
+  unsigned poll_limit;
+  unsigned mute_partition;
+};
+constexpr unsigned kDefaultPollLimit = 1u << 20;
 
 // sum over lanes of the published values at p[lane], lane < count (count <= 64); false if a
 // value never showed up
-TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, int lane, float *sum) {
+TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, int lane, float *sum, unsigned poll_limit) {
   unsigned long long d = kPublished;
   for (unsigned polls = 0;; polls++) {
     if ((unsigned)lane < count) d = atomic_load_u64(p + lane);
     if (ballot((d >> 32) == 1ull) == ~0ull) break;
-    if (polls > kPublishPollLimit) return false;
+    if (polls >= poll_limit) return false;
     spin_pause();
   }
   const float v = (unsigned)lane < count ? __uint_as_float((unsigned)d) : 0.0f;
@@ -69,7 +79,7 @@ TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, in
 }
 
 template <int U, bool MFMA, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, unsigned *ws) {
+__global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, unsigned *ws, WaitPolicy wait) {
   __shared__ float partial[kMaxWaves];
   __shared__ unsigned ticket;
   const int lane = lane_id();
@@ -102,7 +112,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   if (threadIdx.x == 0) {
     float s = 0.0f;
     for (int w = 0; w < WPB; w++) s += partial[w];
-    atomic_store_u64(partials + blockIdx.x, kPublished | __float_as_uint(s));
+    if (blockIdx.x + 1 != wait.mute_partition) atomic_store_u64(partials + blockIdx.x, kPublished | __float_as_uint(s));
     ticket = atomic_add_u32(group_counter + g, 1u);
   }
   __syncthreads();
@@ -112,7 +122,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   if (wave != 0) return;
   const uint16_t failed = 0x7e00u;  // NaN: a published value never became visible
   float s;
-  if (!gather_published(partials + first, members, lane, &s)) {
+  if (!gather_published(partials + first, members, lane, &s, wait.poll_limit)) {
     if (lane == 0) out[0] = failed;
     return;
   }
@@ -127,7 +137,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   for (unsigned base = 0; base < n_groups; base += 64) {
     const unsigned count = n_groups - base < 64 ? n_groups - base : 64;
     float part;
-    if (!gather_published(group_sum + base, count, lane, &part)) {
+    if (!gather_published(group_sum + base, count, lane, &part, wait.poll_limit)) {
       if (lane == 0) out[0] = failed;
       return;
     }
@@ -136,13 +146,45 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   if (lane == 0) out[0] = f16_bits(t);
 }
 
+// Decoupled look-back of partition `part` over the descriptors desc[floor .. part): wave 0 reads
+// 64 descriptors per round (lane l takes desc[base - l]), adds the aggregates down to the
+// nearest published inclusive prefix and returns the sum in every lane.  A descriptor that stays
+// empty for more than wait.poll_limit polls ends the look-back with NaN: the partition's own
+// results and, through the prefix it then publishes, those of every later partition of the scan
+// become NaN instead of a plausible wrong number.  Every lane of the wave takes the same path.
+TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long long floor, int lane, WaitPolicy wait) {
+  float prefix = 0.0f;
+  long long base = part - 1;
+  unsigned polls = 0;
+  while (true) {
+    const long long idx = base - lane;
+    const unsigned long long d = idx >= floor ? atomic_load_u64(desc + idx) : kFlagPrefix;
+    const unsigned flag = (unsigned)(d >> 32);
+    const unsigned long long is_prefix = ballot(flag == 2u);
+    const unsigned long long is_empty = ballot(flag == 0u);
+    const int first_prefix = is_prefix ? __builtin_ctzll(is_prefix) : 64;
+    const unsigned long long needed = first_prefix >= 63 ? ~0ull : ((2ull << first_prefix) - 1ull);
+    if (is_empty & needed) {
+      if (polls++ >= wait.poll_limit) return __builtin_nanf("");  // never spin without bound
+      spin_pause();
+      continue;
+    }
+    float val = lane <= first_prefix ? __uint_as_float((unsigned)d) : 0.0f;
+    val = lane_group_sum<6>(val);
+    prefix += readlane(val, 63);
+    if (first_prefix < 64) return prefix;
+    base -= 64;
+  }
+}
+
 // One partition (blockDim/64 * U tiles) per block.  workspace: ticket counter at word 0,
 // descriptors (64-bit: flag << 32 | float bits) from byte 256.
 // parts_per_segment = 0: one scan over the whole array.  Otherwise the array is a sequence of
 // segments of parts_per_segment whole partitions each, scanned independently (segments far
 // larger than what one block can walk), and `totals`, if given, receives every segment's sum.
 template <int U, bool MFMA, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order, unsigned parts_per_segment, uint16_t *totals) {
+__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order, unsigned parts_per_segment, uint16_t *totals,
+                                                               WaitPolicy wait) {
   __shared__ float wave_total[kMaxWaves];
   __shared__ unsigned s_part;
   __shared__ float s_prefix;
@@ -177,35 +219,13 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
     // and nobody looks back past it
     const unsigned in_segment = parts_per_segment ? part % parts_per_segment : part;
     const long long floor = (long long)part - in_segment;
+    const bool muted = part + 1 == wait.mute_partition;
     if (in_segment == 0) {
-      if (lane == 0) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(aggregate));
     } else {
-      if (lane == 0) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
-      long long base = (long long)part - 1;
-      unsigned polls = 0;
-      while (true) {  // every lane of wave 0 takes the same path
-        const long long idx = base - lane;
-        unsigned long long d = idx >= floor ? atomic_load_u64(desc + idx) : kFlagPrefix;
-        const unsigned flag = (unsigned)(d >> 32);
-        const unsigned long long is_prefix = ballot(flag == 2u);
-        const unsigned long long is_empty = ballot(flag == 0u);
-        const int first_prefix = is_prefix ? __builtin_ctzll(is_prefix) : 64;
-        const unsigned long long needed = first_prefix >= 63 ? ~0ull : ((2ull << first_prefix) - 1ull);
-        if (is_empty & needed) {
-          if (++polls > (1u << 20)) {  // give up: never spin without bound
-            if (lane == 0) atomic_add_u32(ws + 1, 1u);
-            break;
-          }
-          spin_pause();
-          continue;
-        }
-        float val = lane <= first_prefix ? __uint_as_float((unsigned)d) : 0.0f;
-        val = lane_group_sum<6>(val);
-        prefix += readlane(val, 63);
-        if (first_prefix < 64) break;
-        base -= 64;
-      }
-      if (lane == 0) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
+      prefix = look_back(desc, (long long)part, floor, lane, wait);
+      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
     }
     if (totals && parts_per_segment && in_segment == parts_per_segment - 1 && lane == 0) totals[part / parts_per_segment] = f16_bits(prefix + aggregate);
     if (lane == 0) s_prefix = prefix;
@@ -229,7 +249,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
 // per block, still two blocks per CU.  Tiles U .. U+ULDS-1 of a wave follow its register
 // tiles in memory and in scan order.  Same workspace and descriptors as full_scan_kernel.
 template <int U, int ULDS, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order) {
+__global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order, WaitPolicy wait) {
   __shared__ __attribute__((aligned(1024))) half_t held[kMaxWaves * ULDS * kTileHalves];
   __shared__ float wave_total[kMaxWaves];
   __shared__ unsigned s_part;
@@ -273,35 +293,13 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t 
     float aggregate = 0.0f;
     for (int w = 0; w < WPB; w++) aggregate += wave_total[w];
     float prefix = 0.0f;
+    const bool muted = part + 1 == wait.mute_partition;
     if (part == 0) {
-      if (lane == 0) atomic_store_u64(desc, kFlagPrefix | __float_as_uint(aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(desc, kFlagPrefix | __float_as_uint(aggregate));
     } else {
-      if (lane == 0) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
-      long long base = (long long)part - 1;
-      unsigned polls = 0;
-      while (true) {  // every lane of wave 0 takes the same path
-        const long long idx = base - lane;
-        unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : kFlagPrefix;
-        const unsigned flag = (unsigned)(d >> 32);
-        const unsigned long long is_prefix = ballot(flag == 2u);
-        const unsigned long long is_empty = ballot(flag == 0u);
-        const int first_prefix = is_prefix ? __builtin_ctzll(is_prefix) : 64;
-        const unsigned long long needed = first_prefix >= 63 ? ~0ull : ((2ull << first_prefix) - 1ull);
-        if (is_empty & needed) {
-          if (++polls > (1u << 20)) {  // give up: never spin without bound
-            if (lane == 0) atomic_add_u32(ws + 1, 1u);
-            break;
-          }
-          spin_pause();
-          continue;
-        }
-        float val = lane <= first_prefix ? __uint_as_float((unsigned)d) : 0.0f;
-        val = lane_group_sum<6>(val);
-        prefix += readlane(val, 63);
-        if (first_prefix < 64) break;
-        base -= 64;
-      }
-      if (lane == 0) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
+      prefix = look_back(desc, (long long)part, 0, lane, wait);
+      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
     }
     if (lane == 0) s_prefix = prefix;
   }

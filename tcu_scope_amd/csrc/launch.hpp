@@ -6,6 +6,8 @@
 #include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 namespace tcu {
 
 // number of kernels this host thread has enqueued (lets callers tell "nothing was
@@ -41,12 +43,15 @@ inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void
 // The pool keeps what it has handed out once (release threshold at its maximum): the default
 // pool gives unused memory back to the driver at every synchronisation, which turns the next
 // request into a real allocation of a millisecond or more.  The block may be used by work
-// enqueued on `stream` between stream_alloc and stream_free.
+// enqueued on `stream` between stream_alloc and stream_free.  The pool is that of the current
+// device, which must be the device of `stream` (as for every launch made through this library).
 inline void *stream_alloc(size_t bytes, void *stream) {
   constexpr int kMaxDevices = 64;
   static hipMemPool_t pools[kMaxDevices] = {};
+  static std::mutex pools_mutex;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(pools_mutex);
   if (!pools[dev]) {
     hipMemPoolProps props = {};
     props.allocType = hipMemAllocationTypePinned;

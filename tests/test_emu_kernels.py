@@ -217,7 +217,8 @@ def test_full_array_kernels(emu, oracle):
         x = oracle.generate_f16(n, 5, oracle.DIST_GRID)
         w64 = oracle.seg_scan_f64(x, 1, n)
         xi = copy_in(x)
-        for strategy, seg, wpb in ((0, 0, 0), (1, 2048, 4), (1, 1024, 1), (2, 0, 0), (2, 256, 2)):
+        # 0x100 = TCU_FULL_MFMA: the single-pass kernels on the matrix unit
+        for strategy, seg, wpb in ((0, 0, 0), (1, 2048, 4), (1, 1024, 1), (2, 0, 0), (2, 256, 2), (0x100, 0, 0), (0x101, 2048, 4), (0x101, 512, 1)):
             for op, fn in (("reduce", emu.emu_full_reduce_f16), ("scan", emu.emu_full_scan_f16)):
                 need = sz(0)
                 rc = fn(xi.ctypes.data, None, n, None, ctypes.byref(need), strategy, seg, wpb)
@@ -233,6 +234,43 @@ def test_full_array_kernels(emu, oracle):
                     assert np.array_equal(out, ref.astype(np.float16).view(np.uint16)), (op, n, strategy, seg, wpb)
                 else:  # per-segment totals are rounded to fp16 on the way, as in the reference
                     assert oracle.check_f16(out, ref, n)[0] == 0, (op, n, strategy, seg, wpb)
+
+
+def test_a_wait_that_expires_gives_nan(emu, oracle):
+    """A partition that publishes nothing (test option) with a small poll limit: the scan is right up to and
+    including that partition and NaN after it, the reduction's result is NaN, every kernel returns."""
+    sz = ctypes.c_size_t
+    n = 8 * 2048 + 1024
+    x = oracle.generate_f16(n, 5, oracle.DIST_GRID)
+    want = oracle.seg_scan_f64(x, 1, n).astype(np.float16).view(np.uint16)
+    xi = copy_in(x)
+    mute = 3  # partition index 2
+    try:
+        assert emu.emu_set_option(b"lookback_poll_limit", 4) == 0
+        assert emu.emu_set_option(b"test_mute_partition", mute) == 0
+        for strategy in (1, 0x101):
+            need = sz(0)
+            assert emu.emu_full_scan_f16(xi.ctypes.data, None, n, None, ctypes.byref(need), strategy, 2048, 4) == 0
+            ws = aligned(need.value, np.uint8, 0xAB)
+            out = aligned(n, np.uint16, 0xFFFF)
+            assert emu.emu_full_scan_f16(xi.ctypes.data, out.ctypes.data, n, ws.ctypes.data, ctypes.byref(need), strategy, 2048, 4) == 0, emu.emu_last_error()
+            good = mute * 2048
+            assert np.array_equal(out[:good], want[:good])
+            assert np.isnan(out[good:].view(np.float16)).all()
+            assert emu.emu_full_reduce_f16(xi.ctypes.data, None, n, None, ctypes.byref(need), strategy, 2048, 4) == 0
+            ws = aligned(need.value, np.uint8, 0xAB)
+            red = aligned(1, np.uint16, 0x1234)
+            assert emu.emu_full_reduce_f16(xi.ctypes.data, red.ctypes.data, n, ws.ctypes.data, ctypes.byref(need), strategy, 2048, 4) == 0, emu.emu_last_error()
+            assert np.isnan(red.view(np.float16)).all()
+    finally:
+        assert emu.emu_set_option(b"test_mute_partition", 0) == 0
+        assert emu.emu_set_option(b"lookback_poll_limit", -1) == 0
+    need = sz(0)
+    assert emu.emu_full_scan_f16(xi.ctypes.data, None, n, None, ctypes.byref(need), 1, 2048, 4) == 0
+    ws = aligned(need.value, np.uint8, 0xAB)
+    out = aligned(n, np.uint16, 0xFFFF)
+    assert emu.emu_full_scan_f16(xi.ctypes.data, out.ctypes.data, n, ws.ctypes.data, ctypes.byref(need), 1, 2048, 4) == 0
+    assert np.array_equal(out, want)
 
 
 def test_gemv_gemm_and_generator(emu, oracle):

@@ -21,15 +21,17 @@ def test_full_reduce_and_scan(tcu, oracle, n):
     x = oracle.generate_f16(n, 4, oracle.DIST_UNIFORM)
     ref = oracle.seg_scan_f64(x, 1, n)
     xd = to_dev(x)
-    for strategy, seg, w in [(S.AUTO, 0, 0), (S.SINGLE_PASS, 2048, 4), (S.SINGLE_PASS, 1024, 1), (S.SINGLE_PASS, 65536, 8), (S.MULTI_KERNEL, 0, 0), (S.MULTI_KERNEL, 256, 2)]:
+    M = tcu.FULL_MFMA  # flag: the single-pass kernels add and scan on the matrix unit
+    for strategy, seg, w in [(S.AUTO, 0, 0), (S.SINGLE_PASS, 2048, 4), (S.SINGLE_PASS, 1024, 1), (S.SINGLE_PASS, 65536, 8), (S.MULTI_KERNEL, 0, 0), (S.MULTI_KERNEL, 256, 2),
+                             (S.AUTO | M, 0, 0), (S.SINGLE_PASS | M, 4096, 2), (S.SINGLE_PASS | M, 512, 1), (S.SINGLE_PASS | M, 65536, 16)]:
         try:
             red = to_host(tcu.full_reduce(xd, strategy, seg, w))
             sc = to_host(tcu.full_scan(xd, strategy, seg, w))
         except tcu.TcuError as e:
             assert e.status == 2 and strategy == S.MULTI_KERNEL and n % (seg or 2048) != 0, (strategy, seg, str(e))
             continue
-        expect_ok(oracle, red, ref[-1:], n, f"full reduce n={n} {strategy.name} seg={seg}")
-        expect_ok(oracle, sc, ref, n, f"full scan n={n} {strategy.name} seg={seg}")
+        expect_ok(oracle, red, ref[-1:], n, f"full reduce n={n} strategy={int(strategy):#x} seg={seg}")
+        expect_ok(oracle, sc, ref, n, f"full scan n={n} strategy={int(strategy):#x} seg={seg}")
 
 
 def test_full_exact_grid_bitwise_and_repeatable(tcu, oracle):
@@ -57,15 +59,16 @@ def test_full_exact_grid_bitwise_and_repeatable(tcu, oracle):
 
 
 def test_full_size_2p30(tcu, oracle):
-    """N = 2^30: reduction against the fp64 sum; scan through its last element, windows at
-    both ends and the overflow rule (fp16 saturates to inf only where the fp64 prefix does)."""
+    """N = 2^30, every single-kernel form beside AUTO: the reduction against the fp64 sum; the scan
+    through its element at the end of every 2^26 piece, whole windows at both ends and the
+    overflow rule (fp16 saturates to inf only where the fp64 prefix does)."""
+    S = tcu.FullStrategy
     n = 1 << 30
     xd = tcu.generate(n, 1, tcu.Dist.UNIFORM)
-    red = to_host(tcu.full_reduce(xd))
-    out = tcu.full_scan(xd)
-    # fp64 prefix at chunk boundaries, streamed on the host in 2^26 pieces
+    # fp64 prefix at the end of every piece, streamed on the host in 2^26 pieces
     piece = 1 << 26
     carry = 0.0
+    ends = []
     first_ref = last_ref = None
     for p in range(n // piece):
         xp = oracle.generate_f16(piece, 1, oracle.DIST_UNIFORM, first=p * piece)
@@ -74,12 +77,92 @@ def test_full_size_2p30(tcu, oracle):
             first_ref = sc.copy()
         if p == n // piece - 1:
             last_ref = sc.copy()
-        got = to_host(out[p * piece + piece - 1:p * piece + piece])
-        expect_ok(oracle, got, sc[-1:], n, f"2^30 scan at element {p * piece + piece - 1}")
         carry = sc[-1]
-    expect_ok(oracle, red, np.array([carry]), n, "2^30 full reduce")
-    expect_ok(oracle, to_host(out[:piece]), first_ref, n, "2^30 scan first window")
-    expect_ok(oracle, to_host(out[n - piece:]), last_ref, n, "2^30 scan last window")
+        ends.append(carry)
+    ends = np.array(ends)
+    out = None
+    for strategy in (S.AUTO, S.SINGLE_PASS, S.SINGLE_PASS | tcu.FULL_MFMA):
+        what = f"2^30 strategy={int(strategy):#x}"
+        red = to_host(tcu.full_reduce(xd, strategy))
+        expect_ok(oracle, red, ends[-1:], n, what + " full reduce")
+        out = tcu.full_scan(xd, strategy, out=out)
+        got_ends = to_host(out[piece - 1::piece].contiguous())
+        expect_ok(oracle, got_ends, ends, n, what + " scan at the end of every 2^26 piece")
+        expect_ok(oracle, to_host(out[:piece]), first_ref, n, what + " scan first window")
+        expect_ok(oracle, to_host(out[n - piece:]), last_ref, n, what + " scan last window")
+        out.zero_()
+
+
+def test_a_wait_that_expires_gives_nan_not_wrong_numbers(tcu, oracle):
+    """A block of a single-pass kernel that waits in vain for a value another block should have
+    published must not return finite, plausible, wrong data.  The condition is forced from the
+    host: one partition is told to publish nothing and the poll limit is made tiny, so the waits
+    for it expire while every kernel still runs to its end.  Expected: everything up to and
+    including the silent partition is right, everything that depends on it is NaN."""
+    import torch
+
+    S = tcu.FullStrategy
+    n = 1 << 22
+    x = oracle.generate_f16(n, 9, oracle.DIST_UNIFORM)
+    ref = oracle.seg_scan_f64(x, 1, n)
+    xd = to_dev(x)
+    mute = 5  # partition index 4 is silent
+    try:
+        tcu.set_option("lookback_poll_limit", 16)
+        tcu.set_option("test_mute_partition", mute)
+        # (strategy, segment_size, waves) -> halves per partition
+        for strategy, seg, w, part in [(S.SINGLE_PASS, 0, 0, 65536), (S.SINGLE_PASS, 8192, 4, 8192), (S.AUTO, 0, 0, 98304), (S.SINGLE_PASS | tcu.FULL_MFMA, 0, 0, 65536)]:
+            got = to_host(tcu.full_scan(xd, strategy, seg, w))
+            good = mute * part
+            expect_ok(oracle, got[:good], ref[:good], n, f"scan strategy={int(strategy):#x}: partitions before the silent one")
+            assert np.isnan(got[good:].view(np.float16)).all(), f"scan strategy={int(strategy):#x}: data after a wait that expired must be NaN"
+            red = to_host(tcu.full_reduce(xd, S.SINGLE_PASS | (strategy & tcu.FULL_MFMA), seg, w))
+            assert np.isnan(red.view(np.float16)).all(), f"reduce strategy={int(strategy):#x}: the result of a wait that expired must be NaN"
+        # the look-back path of the segmented scan (segments of 2^21 halves = 32 partitions): only the silent
+        # partition's segment is affected
+        seg = 1 << 21
+        refs = oracle.seg_scan_f64(x, n // seg, seg)
+        tot = torch.zeros(n // seg, dtype=torch.float16, device="cuda")
+        got = to_host(tcu.seg_scan(xd, seg, totals=tot))
+        good = mute * 65536
+        expect_ok(oracle, got[:good], refs[:good], seg, "segmented look-back scan: before the silent partition")
+        assert np.isnan(got[good:seg].view(np.float16)).all()
+        expect_ok(oracle, got[seg:], refs[seg:], seg, "segmented look-back scan: the other segment")
+        th = to_host(tot)
+        assert np.isnan(th[:1].view(np.float16)).all()
+        expect_ok(oracle, th[1:], refs[-1:], seg, "segmented look-back scan: total of the other segment")
+    finally:
+        tcu.set_option("test_mute_partition", 0)
+        tcu.set_option("lookback_poll_limit", -1)
+    # and with the defaults restored the same calls are right again
+    expect_ok(oracle, to_host(tcu.full_scan(xd, S.SINGLE_PASS)), ref, n, "scan after the options were reset")
+    expect_ok(oracle, to_host(tcu.full_reduce(xd, S.SINGLE_PASS)), ref[-1:], n, "reduce after the options were reset")
+
+
+def test_convert_f32_to_f16_bit_exact(tcu, oracle):
+    """tcu_convert_f32_to_f16 (the reference's convertFp32ToFp16, src/utils/cuda_helpers.cuh:116-121) against the
+    oracle's round-to-nearest-even conversion: random bit patterns of every exponent, dense samples around the
+    subnormal / normal / overflow boundaries, every exact tie between neighbouring halves, +-65520, +-0, infinities."""
+    import torch
+
+    rng = np.random.default_rng(21)
+    raw = rng.integers(0, 1 << 32, size=1 << 18, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    near = np.concatenate([rng.uniform(-70000, 70000, 1 << 16), rng.uniform(-1e-4, 1e-4, 1 << 16), rng.uniform(-2, 2, 1 << 16)]).astype(np.float32)
+    halves = np.arange(0x7C00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    ties = ((halves[:-1] + halves[1:]) / 2).astype(np.float32)
+    edge = np.float32([65520.0, -65520.0, 65519.996, -65519.996, 65504.0, 2.0 ** -25, -(2.0 ** -25), 2.0 ** -24, 2.0 ** -14, 6.0975552e-05, 0.0, -0.0, np.inf, -np.inf, 0.001])
+    vals = np.concatenate([raw, near, ties, -ties, np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)), edge])
+    vals = vals[~np.isnan(vals)]
+    want = oracle.f32_to_f16_array(vals)
+    got = to_host(tcu.convert_f32_to_f16(torch.from_numpy(vals).cuda()))
+    assert got.shape == want.shape
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, f"{bad.size} conversions differ, first: {vals[bad[0]]!r} -> {got[bad[0]]:#06x}, oracle {want[bad[0]]:#06x}"
+    # NaN in, NaN out
+    nan = to_host(tcu.convert_f32_to_f16(torch.tensor([float("nan")], device="cuda")))
+    assert (nan[0] & 0x7C00) == 0x7C00 and (nan[0] & 0x03FF) != 0
+    # empty input: nothing is launched, nothing fails
+    tcu.convert_f32_to_f16(torch.empty(0, dtype=torch.float32, device="cuda"))
 
 
 def test_add_partial_sums(tcu, oracle):

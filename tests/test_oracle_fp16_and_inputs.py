@@ -44,6 +44,25 @@ def test_f32_to_f16_matches_numpy_rne(oracle):
     assert np.array_equal(got, want)
 
 
+def test_convert_f32_to_f16_array_matches_numpy_rne(oracle):
+    """The element-wise conversion (the reference's convertFp32ToFp16, src/utils/cuda_helpers.cuh:116-121)
+    against numpy's IEEE round-to-nearest-even cast, NaNs by class."""
+    rng = np.random.default_rng(8)
+    raw = rng.integers(0, 1 << 32, size=1 << 18, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    halves = np.arange(0x7C00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    ties = ((halves[:-1] + halves[1:]) / 2).astype(np.float32)
+    vals = np.concatenate([raw, ties, -ties, np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)),
+                           np.float32([65520.0, -65520.0, 65519.996, 65504.0, 2.0 ** -25, 2.0 ** -24, 0.0, -0.0, np.inf, -np.inf, 0.001])])
+    got = oracle.f32_to_f16_array(vals)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    nan = np.isnan(vals)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert ((got[nan] & 0x7C00) == 0x7C00).all() and ((got[nan] & 0x03FF) != 0).all()
+    assert oracle.f32_to_f16_array(np.float32([0.001]))[0] == 0x1419  # the reference's fill value
+    assert oracle.f32_to_f16_array(np.empty(0, np.float32)).size == 0
+
+
 def test_f64_to_f16_single_rounding(oracle):
     rng = np.random.default_rng(11)
     vals = np.concatenate([rng.uniform(-70000, 70000, 20000), rng.uniform(-1e-4, 1e-4, 20000), rng.uniform(-4, 4, 20000)])
