@@ -22,7 +22,7 @@
  *     (4 or 8 bytes per 65536 input halves), the *_offsets_f16 entry points with expected
  *     segment lengths of 2^17 and more (4 bytes per 65536 halves), and tcu_gemm_* when the
  *     last round of output tiles is sparsely filled (up to 128 MiB).  The full-array entry
- *     points work in the caller's workspace.
+ *     points work in the caller's workspace; tcu_seg_scan_f16_noalloc never allocates.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
  *     enqueue work; they do not synchronise.
  *   - the return value is a tcu_status; on failure tcu_last_error() describes it (per
@@ -154,6 +154,19 @@ int tcu_seg_reduce_offsets_f16(const void *d_in, void *d_out, size_t num_segment
  * compute_cub_{warp,block}_segmented_prefixsum (src/prefixsum/seg_cub_warp.cu:17-27,
  * seg_cub_block.cu:13-51).  In-place (d_out == d_in) is allowed. */
 int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
+
+/* tcu_seg_scan_f16 for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc): same arguments, same kernels, same
+ * results, but the partition descriptors of the look-back path (TCU_VARIANT_AUTO with segments of
+ * 2^21 halves and more, the only path of tcu_seg_scan_f16 that takes temporary memory) live in a
+ * 512.25 KiB array that is part of the library's device code, so this entry point never calls
+ * an allocating routine.  Limit: num_segments * segment_size <= 2^32 halves on that path (65536
+ * partitions of 65536 halves; larger calls return TCU_ERR_UNSUPPORTED).  Each GPU holds one such
+ * array: calls of this entry point that overlap in time on one GPU (different streams or
+ * threads) race on it and must be serialised by the caller; calls on the same stream are fine.
+ * The array is cleared by a kernel at the start of every call.  No counterpart in the reference,
+ * whose kernels take no temporary memory. */
+int tcu_seg_scan_f16_noalloc(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
 
 /* Segments given by offsets (conventions of tcu_seg_reduce_offsets_f16; segments must not
  * overlap): d_out[i] = fp16( d_in[begin[j]] + ... + d_in[i] ) for i in [begin[j], end[j]);

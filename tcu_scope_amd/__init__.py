@@ -31,6 +31,7 @@ from .binding import (  # noqa: F401
     seg_reduce_offsets,
     seg_scan_offsets,
     seg_scan,
+    seg_scan_noalloc,
     set_option,
     stream_probe,
     time_next_launch,

@@ -11,7 +11,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 
 EXPORTS = [
     "tcu_abi_version", "tcu_last_error", "tcu_init", "tcu_device_info", "tcu_set_option",
-    "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_offsets_f16", "tcu_add_partial_sums_f16",
+    "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_f16_noalloc", "tcu_seg_scan_offsets_f16", "tcu_add_partial_sums_f16",
     "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32", "tcu_gemv_f16_f16", "tcu_gemm_f16_f16",
     "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_time_next_launch", "tcu_lane_probe",
 ]
@@ -88,6 +88,7 @@ def lib():
         L.tcu_seg_reduce_f16.argtypes = [vp, vp, sz, sz, ci, ci, ci, vp]
         L.tcu_seg_reduce_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz, vp]
         L.tcu_seg_scan_f16.argtypes = [vp, vp, vp, sz, sz, ci, ci, ci, vp]
+        L.tcu_seg_scan_f16_noalloc.argtypes = [vp, vp, vp, sz, sz, ci, ci, ci, vp]
         L.tcu_seg_scan_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz, vp]
         L.tcu_add_partial_sums_f16.argtypes = [vp, vp, sz, sz, vp]
         L.tcu_full_reduce_f16.argtypes = [vp, vp, sz, vp, c.POINTER(sz), ci, sz, ci, vp]
@@ -187,6 +188,16 @@ def seg_scan(x, segment_size, variant=Variant.AUTO, tiles_per_wave=0, waves_per_
     if out is None:
         out = torch.empty(nseg * max(segment_size, 0), dtype=torch.float16, device=x.device)
     _check(lib().tcu_seg_scan_f16(_ptr(x), _ptr(out), _ptr(totals), nseg, segment_size, int(variant), tiles_per_wave, waves_per_block, _stream(stream)))
+    return out
+
+
+def seg_scan_noalloc(x, segment_size, out, variant=Variant.AUTO, tiles_per_wave=0, waves_per_block=0, totals=None, num_segments=None, stream=None):
+    """seg_scan through tcu_seg_scan_f16_noalloc: the caller brings `out`, nothing is allocated on the way
+    (the look-back path keeps its partition descriptors in an array inside the library's device code)."""
+    _need_f16(x, "x")
+    _need_f16(out, "out")
+    nseg = (x.numel() // segment_size if segment_size > 0 else 1) if num_segments is None else num_segments
+    _check(lib().tcu_seg_scan_f16_noalloc(_ptr(x), _ptr(out), _ptr(totals), nseg, segment_size, int(variant), tiles_per_wave, waves_per_block, _stream(stream)))
     return out
 
 

@@ -3,10 +3,43 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <mutex>
 
 #include "dispatch.hpp"
 
+// Partition descriptors of tcu_seg_scan_f16_noalloc: a ticket counter (64 words) and one 64-bit
+// descriptor for each of at most 65536 partitions of 65536 halves.  Every device the library's
+// code is loaded on holds its own copy of the array, at its own address, until the process ends;
+// `scratch` itself is only the host-side handle of the symbol, never a device address.
+constexpr size_t kScratchMaxPartitions = 65536;
+constexpr size_t kScratchWords = 64 + 2 * kScratchMaxPartitions;
+static __device__ __align__(256) unsigned scratch[kScratchWords];
+
 namespace {
+
+// The address of `scratch` on the current device, resolved once per device (tcu_init does it
+// for the device it selects; otherwise the first call that needs it).
+int scratch_on_current_device(const char *what, unsigned **out) {
+  constexpr int kMaxDevices = 64;
+  static unsigned *address[kMaxDevices] = {};
+  static std::mutex address_mutex;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return tcu::fail(TCU_ERR_RUNTIME, std::string(what) + ": hipGetDevice: " + hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return tcu::fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": device ordinal beyond what the library keeps scratch addresses for");
+  std::lock_guard<std::mutex> lock(address_mutex);
+  if (!address[dev]) {
+    unsigned *p = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return tcu::fail(TCU_ERR_RUNTIME, std::string(what) + ": hipGetSymbolAddress(scratch): " + hipGetErrorString(e));
+    }
+    address[dev] = p;
+  }
+  *out = address[dev];
+  return TCU_OK;
+}
 
 struct DeviceState {
   bool initialised = false;
@@ -63,7 +96,8 @@ int tcu_init(int device_id) {
   s.initialised = true;
   if (s.compute_units > 0) tcu::options().compute_units = s.compute_units;
   if (!s.gfx950) return tcu::fail(TCU_ERR_UNSUPPORTED, std::string("tcu_init: this library is built for gfx950 only, device is ") + prop.gcnArchName);
-  return TCU_OK;
+  unsigned *scratch_address = nullptr;
+  return scratch_on_current_device("tcu_init", &scratch_address);
 }
 
 int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int *is_gfx950) {
@@ -94,6 +128,15 @@ int tcu_seg_reduce_offsets_f16(const void *d_in, void *d_out, size_t num_segment
 int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
   const unsigned long before = tcu::launch_count();
   return after_launch("tcu_seg_scan_f16", before, tcu::seg_scan_dispatch(d_in, d_out, d_totals, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, stream));
+}
+
+int tcu_seg_scan_f16_noalloc(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
+  const char *what = "tcu_seg_scan_f16_noalloc";
+  tcu::ScanScratch s;
+  if (int rc = scratch_on_current_device(what, &s.words)) return rc;
+  s.capacity = kScratchWords;
+  const unsigned long before = tcu::launch_count();
+  return after_launch(what, before, tcu::seg_scan_dispatch(d_in, d_out, d_totals, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, stream, what, s));
 }
 
 int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments, const void *d_begin_offsets, const void *d_end_offsets, int offset_bits, size_t expected_segment_size, void *stream) {

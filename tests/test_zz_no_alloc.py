@@ -1,0 +1,90 @@
+"""tcu_seg_scan_f16_noalloc (the entry point for callers that cannot allocate device memory) against
+tcu_seg_scan_f16, through the C ABI: two calls in a row on the look-back path (segments of 2^21 halves and
+more, whose partition descriptors live in the library's built-in scratch array), the second with a smaller
+input, so that what the first call left in the array must not matter; then the paths that need no scratch,
+and the size limit.  Bar: inputs on the k/2048 grid (exact fp32 partial sums) bit for bit equal to the
+existing entry point and to the rounded fp64 prefix; uniform inputs within 2 ulp_fp16 + 1e-3*sqrt(segment
+size) of the fp64 prefix for both entry points (the look-back's fp32 carry depends on timing in its last bit,
+so two calls of either entry point need not agree bit for bit on such inputs)."""
+import numpy as np
+import pytest
+
+from gpu_common import expect_ok, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tcu():
+    import tcu_scope_amd as t
+
+    t.init(0)
+    return t
+
+
+def _both(tcu, oracle, x16, seg, what, exact):
+    import torch
+
+    n = x16.size
+    nseg = n // seg
+    xd = to_dev(x16)
+    ref = oracle.seg_scan_f64(x16, nseg, seg)
+    tot_a = torch.zeros(nseg, dtype=torch.float16, device="cuda")
+    tot_b = torch.zeros(nseg, dtype=torch.float16, device="cuda")
+    out_b = torch.full((n,), float("nan"), dtype=torch.float16, device="cuda")
+    got_a = to_host(tcu.seg_scan(xd, seg, totals=tot_a))
+    got_b = to_host(tcu.seg_scan_noalloc(xd, seg, out_b, totals=tot_b))
+    ref_tot = ref.reshape(nseg, seg)[:, -1]
+    if exact:
+        want = ref.astype(np.float16).view(np.uint16)
+        assert np.array_equal(got_a, want), what + ": tcu_seg_scan_f16 vs rounded fp64 prefix"
+        assert np.array_equal(got_b, got_a), what + ": tcu_seg_scan_f16_noalloc differs from tcu_seg_scan_f16"
+        assert np.array_equal(to_host(tot_b), to_host(tot_a)), what + ": totals differ"
+        assert np.array_equal(to_host(tot_b), want.reshape(nseg, seg)[:, -1]), what + ": totals vs rounded fp64 sums"
+    else:
+        expect_ok(oracle, got_a, ref, seg, what + ": tcu_seg_scan_f16")
+        expect_ok(oracle, got_b, ref, seg, what + ": tcu_seg_scan_f16_noalloc")
+        expect_ok(oracle, to_host(tot_b), ref_tot, seg, what + ": tcu_seg_scan_f16_noalloc totals")
+        # the two entry points against each other: both are within the bound of the same fp64 prefix, so
+        # they are within twice the bound of each other
+        a = got_a.view(np.float16).astype(np.float64)
+        b = got_b.view(np.float16).astype(np.float64)
+        bound = 2 * (2 * np.maximum(np.spacing(np.abs(a).astype(np.float16)).astype(np.float64), 2.0 ** -24) + 1e-3 * np.sqrt(seg))
+        assert (np.abs(a - b) <= bound).all(), what + ": the two entry points disagree beyond the tolerance"
+
+
+def test_noalloc_matches_seg_scan_on_two_calls_in_a_row(tcu, oracle):
+    # first call: 2^24 halves in 4 segments of 2^22 (256 partitions); second call: 2^22 halves in 2 segments of
+    # 2^21 (64 partitions) - fewer descriptors than the first call left behind
+    for call, (n_log2, seg_log2) in enumerate([(24, 22), (22, 21)]):
+        n, seg = 1 << n_log2, 1 << seg_log2
+        g = oracle.generate_f16(n, 40 + call, oracle.DIST_GRID)
+        assert np.abs(oracle.seg_scan_f64(g, n // seg, seg)).max() < 8192  # every fp32 partial sum is exact
+        _both(tcu, oracle, g, seg, f"call {call} grid inputs n=2^{n_log2} seg=2^{seg_log2}", exact=True)
+    for call, (n_log2, seg_log2) in enumerate([(24, 23), (21, 21)]):
+        n, seg = 1 << n_log2, 1 << seg_log2
+        x = oracle.generate_f16(n, 50 + call, oracle.DIST_UNIFORM)
+        _both(tcu, oracle, x, seg, f"call {call} uniform inputs n=2^{n_log2} seg=2^{seg_log2}", exact=False)
+
+
+def test_noalloc_other_paths_and_limit(tcu, oracle):
+    import torch
+
+    # sizes and variants that need no scratch run the same kernels: bit for bit on any input
+    x = oracle.generate_f16(1 << 20, 60, oracle.DIST_UNIFORM)
+    xd = to_dev(x)
+    for seg, variant in [(16, tcu.Variant.AUTO), (256, tcu.Variant.MFMA_256), (2048, tcu.Variant.AUTO), (16384, tcu.Variant.BLOCK_LDS), (24, tcu.Variant.AUTO)]:
+        nseg = x.size // seg
+        xs = xd[:nseg * seg]
+        out = torch.zeros(nseg * seg, dtype=torch.float16, device="cuda")
+        tcu.seg_scan_noalloc(xs, seg, out, variant=variant)
+        assert torch.equal(out, tcu.seg_scan(xs, seg, variant=variant)), (seg, variant.name)
+    # empty input
+    tcu.seg_scan_noalloc(xd[:0], 1 << 21, xd[:0])
+    # beyond the built-in array: 65537 partitions of 65536 halves.  Rejected on the host before anything is
+    # launched, so the (far too small) buffers are never touched
+    small = torch.zeros(1 << 21, dtype=torch.float16, device="cuda")
+    with pytest.raises(tcu.TcuError) as e:
+        tcu.seg_scan_noalloc(small, 1 << 21, small, num_segments=(1 << 11) + 1)
+    assert e.value.status == 2 and "scratch" in str(e.value)
+    # exactly at the limit the host side accepts the size; not launched here (that would need 16 GiB)
