@@ -114,6 +114,11 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *   "compute_units"   blocks of the big-tile GEMM kernel the device runs at a time (set by tcu_init; for tests)
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
+ *   "xcd_run"         -1/0/C, default -1: consecutive blocks of a launch run on different XCDs (block b on XCD
+ *                     b % 8); with C > 0 the segmented kernels renumber their blocks inside groups of 8 * C so that
+ *                     every XCD works on C consecutive pieces of the array (a piece = what one block takes) while
+ *                     the launch still sweeps the array front to back; 0 = no renumbering; -1 = the value measured
+ *                     best for the segment size and launch shape
  *   "lookback_poll_limit"  default 2^20 (negative restores it): how often a block of a single-pass full-array
  *                     kernel (and of the look-back path of tcu_seg_scan_f16 for segments of 2^21 halves and more)
  *                     looks again for a value another block has not published yet before it gives up.  Giving up

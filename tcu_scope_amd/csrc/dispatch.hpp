@@ -42,6 +42,7 @@ struct Options {
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
   int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
   int gemm_split_tail = 1;     // spread the K steps of the tiles of a last, partly filled round of the GEMM grid over all compute units: 0 never, 1 where it pays, 2 always
+  int xcd_run = -1;            // consecutive pieces of work per XCD (xcd_run_piece): -1 = the measured value for the size, 0 = none, C > 0 = C
   unsigned lookback_poll_limit = kDefaultPollLimit;  // polls of an unpublished value before a single-pass kernel gives up (results become NaN)
   unsigned test_mute_partition = 0;                  // tests only: partition test_mute_partition - 1 of a single-pass kernel publishes nothing
 };
@@ -65,6 +66,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
   else if (n == "compute_units") o.compute_units = value < 1 ? 1 : value;
+  else if (n == "xcd_run") o.xcd_run = value < 0 ? -1 : value;
   else if (n == "lookback_poll_limit") o.lookback_poll_limit = value < 0 ? kDefaultPollLimit : (unsigned)value;
   else if (n == "test_mute_partition") o.test_mute_partition = value < 0 ? 0u : (unsigned)value;
   else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
@@ -138,26 +140,32 @@ inline int validate_segmented(const char *what, const void *in, const void *out,
 struct Plan {
   bool block;  // block-per-segment kernel
   int u, w;
+  unsigned c = 0;  // consecutive blocks per XCD (xcd_run_piece)
 };
+// the run length a launch uses: the option when set, else the plan's (only when the plan's shape is the one launched)
+inline unsigned xcd_run_for(const Plan &plan, bool plan_shape) {
+  if (options().xcd_run >= 0) return (unsigned)options().xcd_run;
+  return plan_shape ? plan.c : 0u;
+}
 inline Plan auto_plan_reduce(size_t S) {
-  if (S <= 32) return {false, 2, 1};
-  if (S <= 512) return {false, 2, 4};
-  if (S == 1024) return {false, 4, 4};
-  if (S == 2048) return {false, 1, 1};
-  if (S == 4096) return {true, 2, 4};
-  if (S == 8192) return {true, 4, 8};
-  if (S >= 262144) return {true, 2, 8};
-  return {true, 1, 8};
+  if (S <= 512) return {false, 2, 1, 512};
+  if (S == 1024) return {true, 2, 1, 64};
+  if (S == 2048) return {false, 1, 1, 0};
+  if (S == 4096) return {true, 2, 4, 64};
+  if (S == 8192) return {true, 2, 8, 64};
+  if (S == 16384) return {true, 2, 8, 64};
+  if (S >= 262144) return {true, 2, 8, 0};
+  return {true, 1, 8, 0};
 }
 inline Plan auto_plan_scan(size_t S) {
-  if (S <= 512) return {false, 1, 1};
-  if (S == 1024) return {false, 1, 2};
-  if (S == 2048) return {true, 4, 2};
-  if (S == 4096) return {true, 1, 2};
-  if (S == 8192) return {true, 4, 8};
-  if (S == 16384) return {true, 8, 4};
-  if (S == 32768) return {true, 8, 8};
-  return {true, 8, 16};
+  if (S <= 512) return {false, 2, 1, 256};
+  if (S == 1024) return {false, 1, 1, 64};
+  if (S == 2048) return {true, 2, 2, 256};
+  if (S == 4096) return {true, 2, 4, 128};
+  if (S == 8192) return {true, 2, 8, 0};
+  if (S == 16384) return {true, 4, 8, 8};
+  if (S == 32768) return {true, 8, 8, 4};
+  return {true, 8, 16, 0};
 }
 
 inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || v == TCU_VARIANT_MFMA_256N_BLOCK || v == TCU_VARIANT_BLOCK_LDS; }
@@ -165,30 +173,30 @@ inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || 
 // ----- segmented reduction ----------------------------------------------------------------
 
 template <int LPS_LOG2, int U, bool MFMA>
-inline void launch_reduce_small(unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg) {
+inline void launch_reduce_small(unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg, unsigned run) {
   if (options().nontemporal)
-    launch(seg_reduce_small_kernel<LPS_LOG2, U, MFMA, true>, grid, block, stream, in, out, n_chunks, nseg);
+    launch(seg_reduce_small_kernel<LPS_LOG2, U, MFMA, true>, grid, block, stream, in, out, n_chunks, nseg, run);
   else
-    launch(seg_reduce_small_kernel<LPS_LOG2, U, MFMA, false>, grid, block, stream, in, out, n_chunks, nseg);
+    launch(seg_reduce_small_kernel<LPS_LOG2, U, MFMA, false>, grid, block, stream, in, out, n_chunks, nseg, run);
 }
 template <int LPS_LOG2, bool MFMA>
-inline void launch_reduce_small_u(int u, unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg) {
+inline void launch_reduce_small_u(int u, unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg, unsigned run) {
   switch (u) {
-    case 1: return launch_reduce_small<LPS_LOG2, 1, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
-    case 2: return launch_reduce_small<LPS_LOG2, 2, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
-    case 4: return launch_reduce_small<LPS_LOG2, 4, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
-    default: return launch_reduce_small<LPS_LOG2, 8, MFMA>(grid, block, stream, in, out, n_chunks, nseg);
+    case 1: return launch_reduce_small<LPS_LOG2, 1, MFMA>(grid, block, stream, in, out, n_chunks, nseg, run);
+    case 2: return launch_reduce_small<LPS_LOG2, 2, MFMA>(grid, block, stream, in, out, n_chunks, nseg, run);
+    case 4: return launch_reduce_small<LPS_LOG2, 4, MFMA>(grid, block, stream, in, out, n_chunks, nseg, run);
+    default: return launch_reduce_small<LPS_LOG2, 8, MFMA>(grid, block, stream, in, out, n_chunks, nseg, run);
   }
 }
 template <bool MFMA>
-inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg) {
+inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned block, void *stream, const half8_t *in, uint16_t *out, size_t n_chunks, size_t nseg, unsigned run) {
   switch (lps_log2) {
-    case 1: return launch_reduce_small_u<1, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
-    case 2: return launch_reduce_small_u<2, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
-    case 3: return launch_reduce_small_u<3, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
-    case 4: return launch_reduce_small_u<4, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
-    case 5: return launch_reduce_small_u<5, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
-    default: return launch_reduce_small_u<6, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg);
+    case 1: return launch_reduce_small_u<1, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg, run);
+    case 2: return launch_reduce_small_u<2, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg, run);
+    case 3: return launch_reduce_small_u<3, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg, run);
+    case 4: return launch_reduce_small_u<4, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg, run);
+    case 5: return launch_reduce_small_u<5, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg, run);
+    default: return launch_reduce_small_u<6, MFMA>(u, grid, block, stream, in, out, n_chunks, nseg, run);
   }
 }
 
@@ -224,6 +232,9 @@ inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned b
 // few bytes per partition of temporary device memory, taken in stream order.
 constexpr size_t kHugeReduceSegment = (size_t)1 << 20, kHugeScanSegment = (size_t)1 << 21, kHugePartHalves = 65536;
 
+// partitions of 65536 halves per XCD in the partition-sum launches (xcd_run_piece)
+inline unsigned partition_sums_run() { return options().xcd_run >= 0 ? (unsigned)options().xcd_run : 0u; }
+
 inline int seg_reduce_huge(const half8_t *in, uint16_t *out, size_t num_segments, size_t S, bool nt, void *stream) {
   const char *what = "tcu_seg_reduce_f16";
   const size_t pps = S / kHugePartHalves, parts = num_segments * pps;
@@ -232,9 +243,9 @@ inline int seg_reduce_huge(const half8_t *in, uint16_t *out, size_t num_segments
   if (!partials) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partition sums");
   const size_t n_chunks = num_segments * S / 8;
   if (nt)
-    launch(partition_sums_kernel<8, true>, (unsigned)parts, 1024u, stream, in, partials, n_chunks);
+    launch(partition_sums_kernel<8, true>, (unsigned)parts, 1024u, stream, in, partials, n_chunks, partition_sums_run());
   else
-    launch(partition_sums_kernel<8, false>, (unsigned)parts, 1024u, stream, in, partials, n_chunks);
+    launch(partition_sums_kernel<8, false>, (unsigned)parts, 1024u, stream, in, partials, n_chunks, partition_sums_run());
   launch(segment_of_partials_kernel, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(partials), out, pps);
   stream_free(partials, stream);
   return TCU_OK;
@@ -297,13 +308,14 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
   const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 2 : 4));
   const int wpb = waves_per_block ? waves_per_block : (plan_fits ? plan.w : (use_block ? 8 : 4));
   const unsigned block = (unsigned)wpb * 64u;
+  const unsigned run = xcd_run_for(plan, plan_fits && u == plan.u && wpb == plan.w);
 
   if (use_block) {
     const size_t tiles_per_seg = S / kTileHalves;
     const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;  // the reference's 16n_block owns 16 segments per block
     const size_t grid = (num_segments + spb - 1) / spb;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
-    TCU_SWITCH_U_MFMA_NT(seg_reduce_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tiles_per_seg, spb);
+    TCU_SWITCH_U_MFMA_NT(seg_reduce_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tiles_per_seg, spb, run);
     return TCU_OK;
   }
   if (S <= 512) {
@@ -313,9 +325,9 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
     const int lps_log2 = ilog2(S) - 3;
     if (a.mfma)
-      launch_reduce_small_s<true>(lps_log2, u, (unsigned)grid, block, stream, in, out, n_chunks, num_segments);
+      launch_reduce_small_s<true>(lps_log2, u, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, run);
     else
-      launch_reduce_small_s<false>(lps_log2, u, (unsigned)grid, block, stream, in, out, n_chunks, num_segments);
+      launch_reduce_small_s<false>(lps_log2, u, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, run);
     return TCU_OK;
   }
   // S >= 1024: each wave walks max(S, u tiles) of data
@@ -328,7 +340,7 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
   const size_t waves = (tiles + tiles_per_wave_total - 1) / tiles_per_wave_total;
   const size_t grid = (waves + wpb - 1) / wpb;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
-  TCU_SWITCH_U_MFMA_NT(seg_reduce_long_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tps_log2, (unsigned)iters);
+  TCU_SWITCH_U_MFMA_NT(seg_reduce_long_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tps_log2, (unsigned)iters, run);
   return TCU_OK;
 }
 
@@ -426,12 +438,12 @@ inline int seg_reduce_offsets_dispatch(const void *d_in, void *d_out, size_t num
 
 template <int LPS_LOG2, bool MFMA>
 inline void launch_scan_wave_u(int u, bool nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg, int tps_log2,
-                               unsigned iters) {
-#define TCU_SCAN_CASE(UU)                                                                                                          \
-  if (nt)                                                                                                                          \
-    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, true>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters); \
-  else                                                                                                                             \
-    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, false>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters); \
+                               unsigned iters, unsigned run) {
+#define TCU_SCAN_CASE(UU)                                                                                                               \
+  if (nt)                                                                                                                               \
+    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, true>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run); \
+  else                                                                                                                                  \
+    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, false>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run); \
   return
   switch (u) {
     case 1: TCU_SCAN_CASE(1);
@@ -443,14 +455,14 @@ inline void launch_scan_wave_u(int u, bool nt, unsigned grid, unsigned block, vo
 }
 template <bool MFMA>
 inline void launch_scan_wave_s(int lps_log2, int u, bool nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg,
-                               int tps_log2, unsigned iters) {
+                               int tps_log2, unsigned iters, unsigned run) {
   switch (lps_log2) {
-    case 1: return launch_scan_wave_u<1, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
-    case 2: return launch_scan_wave_u<2, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
-    case 3: return launch_scan_wave_u<3, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
-    case 4: return launch_scan_wave_u<4, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
-    case 5: return launch_scan_wave_u<5, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
-    default: return launch_scan_wave_u<6, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters);
+    case 1: return launch_scan_wave_u<1, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);
+    case 2: return launch_scan_wave_u<2, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);
+    case 3: return launch_scan_wave_u<3, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);
+    case 4: return launch_scan_wave_u<4, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);
+    case 5: return launch_scan_wave_u<5, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);
+    default: return launch_scan_wave_u<6, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);
   }
 }
 
@@ -481,13 +493,14 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 4 : 4));
   const int wpb = waves_per_block ? waves_per_block : (plan_fits ? plan.w : (use_block ? 4 : 1));
   const unsigned block = (unsigned)wpb * 64u;
+  const unsigned run = xcd_run_for(plan, plan_fits && u == plan.u && wpb == plan.w);
 
   if (use_block) {
     const size_t tiles_per_seg = S / kTileHalves;
     const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;
     const size_t grid = (num_segments + spb - 1) / spb;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    TCU_SWITCH_U_MFMA_NT(seg_scan_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, spb);
+    TCU_SWITCH_U_MFMA_NT(seg_scan_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, spb, run);
     return TCU_OK;
   }
   int lps_log2, tps_log2 = 0;
@@ -507,9 +520,9 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   const size_t grid = (waves + wpb - 1) / wpb;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
   if (a.mfma)
-    launch_scan_wave_s<true>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters);
+    launch_scan_wave_s<true>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters, run);
   else
-    launch_scan_wave_s<false>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters);
+    launch_scan_wave_s<false>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters, run);
   return TCU_OK;
 }
 
@@ -676,9 +689,9 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
     if (two_level) {  // p is 16 waves of 8 tiles; the workspace (sized for the single kernel) holds one float per partition
       float *partials = static_cast<float *>(d_ws);
       if (nt)
-        launch(partition_sums_kernel<8, true>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks);
+        launch(partition_sums_kernel<8, true>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks, partition_sums_run());
       else
-        launch(partition_sums_kernel<8, false>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks);
+        launch(partition_sums_kernel<8, false>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks, partition_sums_run());
       launch(segment_of_partials_kernel, 1u, 1024u, stream, static_cast<const float *>(partials), static_cast<uint16_t *>(d_out), grid);
       return TCU_OK;
     }

@@ -324,12 +324,13 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t 
 // Segments far larger than one block's reach, first level: block b adds its partition
 // (blockDim/64 * U tiles) and writes the fp32 partial to partial[b].
 template <int U, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void partition_sums_kernel(const half8_t *__restrict__ in, float *__restrict__ partial_out, size_t n_chunks) {
+__global__ __launch_bounds__(kMaxBlock) void partition_sums_kernel(const half8_t *__restrict__ in, float *__restrict__ partial_out, size_t n_chunks, unsigned xcd_run) {
   __shared__ float partial[kMaxWaves];
   const int lane = lane_id(), wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
+  const size_t part = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run);
   half8_t v[U];
-  load_tiles<U, NT>(v, in, ((size_t)blockIdx.x * WPB + wave) * U * kTileChunks, n_chunks, lane);
+  load_tiles<U, NT>(v, in, (part * WPB + wave) * U * kTileChunks, n_chunks, lane);
   float accs[2] = {0.0f, 0.0f};
 #pragma unroll
   for (int j = 0; j < U; j++) accs[j & 1] = sum8(v[j], accs[j & 1]);
@@ -339,7 +340,7 @@ __global__ __launch_bounds__(kMaxBlock) void partition_sums_kernel(const half8_t
   if (threadIdx.x == 0) {
     float s = 0.0f;
     for (int w = 0; w < WPB; w++) s += partial[w];
-    partial_out[blockIdx.x] = s;
+    partial_out[part] = s;
   }
 }
 // second level: block j (1024 threads) adds the parts_per_segment partials of segment j in a

@@ -47,6 +47,22 @@ TCU_DEVICE void load_tiles(half8_t (&v)[U], const half8_t *__restrict__ in, size
   }
 }
 
+// Which piece of work the block with index b of a grid of `grid` blocks takes.  Consecutive
+// blocks of a launch are dealt round-robin to the 8 XCDs (block b runs on XCD b % 8).  With
+// run = 0 block b takes piece b, so neighbouring pieces of the array are worked on by different
+// XCDs.  With run = C > 0 the blocks are renumbered inside groups of 8 * C so that every XCD
+// takes C consecutive pieces (XCD x of a group: pieces x * C .. x * C + C - 1) while the
+// launch as a whole still sweeps the array front to back; a last, incomplete group keeps its
+// own numbering.  What this changes is the order in which the memory channels see the
+// requests of one XCD; the best C per segment size is measured (dispatch.hpp).
+TCU_DEVICE size_t xcd_run_piece(size_t b, size_t grid, unsigned run) {
+  if (run == 0) return b;
+  const size_t group = (size_t)8 * run;
+  const size_t first = b / group * group;
+  if (first + group > grid) return b;
+  return first + (b & 7) * run + ((b - first) >> 3);
+}
+
 // Sum over groups of 2^LOG2 adjacent lanes.  For LOG2 <= 4 every lane of a group ends
 // up with the group's sum; for LOG2 = 5 only lanes 16..31 / 48..63 do, for LOG2 = 6
 // only lanes 48..63.
@@ -69,13 +85,13 @@ TCU_DEVICE half8_t column_select_operand(int lane, int slot) { return splat8((la
 // S = 16 .. 512
 // ---------------------------------------------------------------------------------------
 template <int LPS_LOG2, int U, bool MFMA, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void seg_reduce_small_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, size_t num_segments) {
+__global__ __launch_bounds__(kMaxBlock) void seg_reduce_small_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, size_t num_segments, unsigned xcd_run) {
   constexpr int LPS = 1 << LPS_LOG2;  // lanes (chunks) per segment
   constexpr int R = 64 / LPS;         // segments per tile
   constexpr int RW = R * U;           // segments per wave
   const int lane = lane_id();
   const int wave = wave_in_block();
-  const size_t gw = (size_t)blockIdx.x * (blockDim.x >> 6) + wave;
+  const size_t gw = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave;
   const size_t chunk0 = gw * (size_t)(U * kTileChunks);
   if (chunk0 >= n_chunks) return;  // wave-uniform
   const size_t seg0 = gw * (size_t)RW;
@@ -159,9 +175,9 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_small_kernel(const half8
 // i.e. iters*U/tiles_per_seg whole segments (the host picks iters so that this is >= 1).
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void seg_reduce_long_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, size_t num_segments, int tiles_per_seg_log2,
-                                                                     unsigned iters) {
+                                                                     unsigned iters, unsigned xcd_run) {
   const int lane = lane_id();
-  const size_t gw = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  const size_t gw = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave_in_block();
   const size_t tile0 = gw * (size_t)iters * U;
   if (tile0 * kTileChunks >= n_chunks) return;
   const size_t tmask = ((size_t)1 << tiles_per_seg_log2) - 1;
@@ -202,14 +218,15 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_long_kernel(const half8_
 // ---------------------------------------------------------------------------------------
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void seg_reduce_block_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, size_t num_segments, size_t tiles_per_seg,
-                                                                      unsigned segs_per_block) {
+                                                                      unsigned segs_per_block, unsigned xcd_run) {
   __shared__ float partial[kMaxWaves];
   const int lane = lane_id();
   const int wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
   const half8_t ones = splat8(1.0f);
+  const size_t piece = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run);
   for (unsigned sb = 0; sb < segs_per_block; sb++) {
-    const size_t seg = (size_t)blockIdx.x * segs_per_block + sb;
+    const size_t seg = piece * segs_per_block + sb;
     if (seg >= num_segments) break;  // block-uniform
     const size_t tile_base = seg * tiles_per_seg;
     float accs = 0.0f;

@@ -202,9 +202,10 @@ TCU_DEVICE void scan_tile(half8_t v, float carry, const ScanOperands &ops, int l
 // Each wave owns iters*U consecutive tiles.
 // ---------------------------------------------------------------------------------------
 template <int LPS_LOG2, int U, bool MFMA, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, int tiles_per_seg_log2, unsigned iters) {
+__global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, int tiles_per_seg_log2, unsigned iters,
+                                                                   unsigned xcd_run) {
   const int lane = lane_id();
-  const size_t gw = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  const size_t gw = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave_in_block();
   const size_t tile0 = gw * (size_t)iters * U;
   if (tile0 * kTileChunks >= n_chunks) return;
   const size_t tmask = ((size_t)1 << tiles_per_seg_log2) - 1;
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t 
 // ---------------------------------------------------------------------------------------
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, size_t tiles_per_seg,
-                                                                    unsigned segs_per_block) {
+                                                                    unsigned segs_per_block, unsigned xcd_run) {
   __shared__ float wave_total[2][kMaxWaves];
   const int lane = lane_id();
   const int wave = wave_in_block();
@@ -248,8 +249,9 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
   ScanOperands ops;
   if constexpr (MFMA) ops = make_scan_operands(lane);
   unsigned parity = 0;
+  const size_t piece = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run);
   for (unsigned sb = 0; sb < segs_per_block; sb++) {
-    const size_t seg = (size_t)blockIdx.x * segs_per_block + sb;
+    const size_t seg = piece * segs_per_block + sb;
     if (seg >= num_segments) break;  // block-uniform
     const size_t tile_base = seg * tiles_per_seg;
     size_t lim = (tile_base + tiles_per_seg) * kTileChunks;
