@@ -59,13 +59,16 @@ typedef enum {
   TCU_VARIANT_AUTO = 0,            /* fastest measured family for the size; any segment size >= 1 */
   TCU_VARIANT_MFMA_16 = 1,         /* segment size 16      (reference *_16)          */
   TCU_VARIANT_MFMA_16N = 2,        /* power of two >= 16   (reference *_16N, _16N_OPT) */
-  TCU_VARIANT_MFMA_16N_BLOCK = 3,  /* >= 512, 16 segments per block (reference *_16N_BLOCK) */
+  TCU_VARIANT_MFMA_16N_BLOCK = 3,  /* power of two >= 16, 16 segments per block (reference *_16N_BLOCK) */
   TCU_VARIANT_MFMA_256 = 4,        /* segment size 256     (reference *_256)         */
   TCU_VARIANT_MFMA_256N = 5,       /* power of two >= 256  (reference *_256N)        */
-  TCU_VARIANT_MFMA_256N_BLOCK = 6, /* >= 512, block per segment (reference *_256N_BLOCK) */
+  TCU_VARIANT_MFMA_256N_BLOCK = 6, /* power of two >= 256, block per segment (reference *_256N_BLOCK) */
   TCU_VARIANT_WAVE_SHUFFLE = 7,    /* DPP wavefront collectives (reference CUB_WARP_*) */
-  TCU_VARIANT_BLOCK_LDS = 8        /* >= 512, block collectives through LDS (reference CUB_BLOCK_*) */
+  TCU_VARIANT_BLOCK_LDS = 8        /* power of two >= 16, block collectives through LDS (reference CUB_BLOCK_*) */
 } tcu_variant;
+/* The three block families share a segment among the waves of a block from 512 halves (one 1 KiB tile) on.  A
+ * shorter segment lies inside one wave's tile, so there the same launch shape (waves per block x tiles per wave)
+ * runs the kernels whose waves take whole tiles: no wave of the block has anything to tell another. */
 
 /* Strategies of the full-array entry points. */
 typedef enum {

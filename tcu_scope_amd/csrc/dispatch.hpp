@@ -118,13 +118,12 @@ inline int validate_segmented(const char *what, const void *in, const void *out,
       if (S != 256) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment size must be 256");
       break;
     case TCU_VARIANT_MFMA_256N:
+    case TCU_VARIANT_MFMA_256N_BLOCK:  // the reference registers *_256N_BLOCK from 256 on (src/reduction/seg_wmma_256n_block.cu:242-248)
       if (!is_pow2(S) || S < 256) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment size must be a power-of-two multiple of 256");
       break;
-    case TCU_VARIANT_MFMA_16N_BLOCK:
-    case TCU_VARIANT_MFMA_256N_BLOCK:
-    case TCU_VARIANT_BLOCK_LDS:
-      if (!is_pow2(S) || S < 512) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": block-per-segment variants need a power-of-two segment size >= 512");
-      break;
+    // MFMA_16N_BLOCK (reference *_16N_BLOCK, 16 ... 1024: src/reduction/seg_wmma_16n_block.cu:229-235) and BLOCK_LDS
+    // (reference cub::Block*, THREADS * ITEMS from 32 on: src/reduction/seg_cub_block.cu:145-288) take every power
+    // of two from 16 on, like the wave families
     default:
       if (!is_pow2(S) || S < 16) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment size must be a power of two >= 16");
   }
@@ -169,6 +168,16 @@ inline Plan auto_plan_scan(size_t S) {
 }
 
 inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || v == TCU_VARIANT_MFMA_256N_BLOCK || v == TCU_VARIANT_BLOCK_LDS; }
+// Default tiles per wave of a wave-kernel launch (segments shorter than a tile).  The reference's *_16N_BLOCK kernels
+// give a block 16 segments (src/reduction/kernel.cuh:176-236): here the block's waves then cover at least 16
+// segments, i.e. 16 * S / 512 tiles (rounded up to a whole tile per wave, at most 8).
+inline int block_family_tiles(int variant, size_t S, int wpb, int otherwise) {
+  if (variant != TCU_VARIANT_MFMA_16N_BLOCK) return otherwise;
+  const size_t tiles = (16 * S + kTileHalves - 1) / kTileHalves;
+  int u = 1;
+  while (u < 8 && (size_t)u * wpb < tiles) u *= 2;
+  return u;
+}
 
 // ----- segmented reduction ----------------------------------------------------------------
 
@@ -302,11 +311,13 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
   if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeReduceSegment) return seg_reduce_huge(in, out, num_segments, S, nt, stream);
   const size_t n_chunks = N / 8;
   const Plan plan = auto_plan_reduce(S);
-  const bool use_block = variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant);
+  // A segment shorter than a tile cannot be shared by the waves of a block: below 512 halves the block families
+  // run the kernels whose waves take whole tiles, at the block's launch shape (waves per block x tiles per wave)
+  const bool use_block = S >= kTileHalves && (variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant));
   // explicit families keep their own tuned shape; AUTO and matching families use the plan
   const bool plan_fits = variant == TCU_VARIANT_AUTO || plan.block == use_block;
-  const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 2 : 4));
   const int wpb = waves_per_block ? waves_per_block : (plan_fits ? plan.w : (use_block ? 8 : 4));
+  const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 2 : block_family_tiles(variant, S, wpb, 4)));
   const unsigned block = (unsigned)wpb * 64u;
   const unsigned run = xcd_run_for(plan, plan_fits && u == plan.u && wpb == plan.w);
 
@@ -488,10 +499,10 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeScanSegment) return seg_scan_huge(what, in, out, totals, num_segments, S, nt, stream, scratch);
   const size_t n_chunks = N / 8;
   const Plan plan = auto_plan_scan(S);
-  const bool use_block = variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant);
+  const bool use_block = S >= kTileHalves && (variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant));  // as in the reduction
   const bool plan_fits = variant == TCU_VARIANT_AUTO || plan.block == use_block;
-  const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 4 : 4));
   const int wpb = waves_per_block ? waves_per_block : (plan_fits ? plan.w : (use_block ? 4 : 1));
+  const int u = tiles_per_wave ? tiles_per_wave : (plan_fits ? plan.u : (use_block ? 4 : block_family_tiles(variant, S, wpb, 4)));
   const unsigned block = (unsigned)wpb * 64u;
   const unsigned run = xcd_run_for(plan, plan_fits && u == plan.u && wpb == plan.w);
 

@@ -58,6 +58,102 @@ static inline int64_t two_power_i(int64_t p) { return argspace::pow2(p); }
 #define SEG_8192_ARGS() TCU_SEG_ARGS(8192)
 #define SEG_16384_ARGS() TCU_SEG_ARGS(16384)
 
+// One registration per WARPS_PER_BLOCK of the reference's lists (1, 2, 4, 8, 16), and the reference's two lists of
+// segment sizes: 16 ... 1024 for the *_16N* families (e.g. src/reduction/seg_wmma_16n.cu:215-221) and 256 ... 16384
+// for the *_256N* families (src/reduction/seg_wmma_256n.cu:223-229)
+#define RUN_WPB(NAME, ARGS_MACRO)                             \
+  BENCHMARK_TEMPLATE(NAME, 1)->ARGS_MACRO()->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 2)->ARGS_MACRO()->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 4)->ARGS_MACRO()->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 8)->ARGS_MACRO()->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 16)->ARGS_MACRO()->UseManualTime()
+#define RUN_WPB_APPLY(NAME, FN)                            \
+  BENCHMARK_TEMPLATE(NAME, 1)->Apply(FN)->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 2)->Apply(FN)->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 4)->Apply(FN)->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 8)->Apply(FN)->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 16)->Apply(FN)->UseManualTime()
+#define RUN_WPB_SEG_16_TO_1024(NAME) \
+  RUN_WPB(NAME, SEG_16_ARGS);        \
+  RUN_WPB(NAME, SEG_32_ARGS);        \
+  RUN_WPB(NAME, SEG_64_ARGS);        \
+  RUN_WPB(NAME, SEG_128_ARGS);       \
+  RUN_WPB(NAME, SEG_256_ARGS);       \
+  RUN_WPB(NAME, SEG_512_ARGS);       \
+  RUN_WPB(NAME, SEG_1024_ARGS)
+#define RUN_WPB_SEG_256_TO_16384(NAME) \
+  RUN_WPB(NAME, SEG_256_ARGS);         \
+  RUN_WPB(NAME, SEG_512_ARGS);         \
+  RUN_WPB(NAME, SEG_1024_ARGS);        \
+  RUN_WPB(NAME, SEG_2048_ARGS);        \
+  RUN_WPB(NAME, SEG_4096_ARGS);        \
+  RUN_WPB(NAME, SEG_8192_ARGS);        \
+  RUN_WPB(NAME, SEG_16384_ARGS)
+// The reference's cub::Block* registrations: every (THREADS_PER_BLOCK, ITEMS_PER_THREAD) with 32 ... 1024 threads whose
+// product is a segment size from 32 to 16384 (src/reduction/seg_cub_block.cu:145-288, src/prefixsum/seg_cub_block.cu:159-302)
+#define RUN_CUB_BLOCK(NAME, ALG)                                                       \
+  BENCHMARK_TEMPLATE(NAME, 32, 1, ALG)->SEG_32_ARGS()->UseManualTime();                \
+  BENCHMARK_TEMPLATE(NAME, 32, 2, ALG)->SEG_64_ARGS()->UseManualTime();                \
+  BENCHMARK_TEMPLATE(NAME, 64, 1, ALG)->SEG_64_ARGS()->UseManualTime();                \
+  BENCHMARK_TEMPLATE(NAME, 32, 4, ALG)->SEG_128_ARGS()->UseManualTime();               \
+  BENCHMARK_TEMPLATE(NAME, 64, 2, ALG)->SEG_128_ARGS()->UseManualTime();               \
+  BENCHMARK_TEMPLATE(NAME, 128, 1, ALG)->SEG_128_ARGS()->UseManualTime();              \
+  BENCHMARK_TEMPLATE(NAME, 32, 8, ALG)->SEG_256_ARGS()->UseManualTime();               \
+  BENCHMARK_TEMPLATE(NAME, 64, 4, ALG)->SEG_256_ARGS()->UseManualTime();               \
+  BENCHMARK_TEMPLATE(NAME, 128, 2, ALG)->SEG_256_ARGS()->UseManualTime();              \
+  BENCHMARK_TEMPLATE(NAME, 256, 1, ALG)->SEG_256_ARGS()->UseManualTime();              \
+  BENCHMARK_TEMPLATE(NAME, 32, 16, ALG)->SEG_512_ARGS()->UseManualTime();              \
+  BENCHMARK_TEMPLATE(NAME, 64, 8, ALG)->SEG_512_ARGS()->UseManualTime();               \
+  BENCHMARK_TEMPLATE(NAME, 128, 4, ALG)->SEG_512_ARGS()->UseManualTime();              \
+  BENCHMARK_TEMPLATE(NAME, 256, 2, ALG)->SEG_512_ARGS()->UseManualTime();              \
+  BENCHMARK_TEMPLATE(NAME, 512, 1, ALG)->SEG_512_ARGS()->UseManualTime();              \
+  BENCHMARK_TEMPLATE(NAME, 32, 32, ALG)->SEG_1024_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 64, 16, ALG)->SEG_1024_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 128, 8, ALG)->SEG_1024_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 256, 4, ALG)->SEG_1024_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 512, 2, ALG)->SEG_1024_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 1024, 1, ALG)->SEG_1024_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 32, 64, ALG)->SEG_2048_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 64, 32, ALG)->SEG_2048_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 128, 16, ALG)->SEG_2048_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 256, 8, ALG)->SEG_2048_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 512, 4, ALG)->SEG_2048_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 1024, 2, ALG)->SEG_2048_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 32, 128, ALG)->SEG_4096_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 64, 64, ALG)->SEG_4096_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 128, 32, ALG)->SEG_4096_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 256, 16, ALG)->SEG_4096_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 512, 8, ALG)->SEG_4096_ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, 1024, 4, ALG)->SEG_4096_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 32, 256, ALG)->SEG_8192_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 64, 128, ALG)->SEG_8192_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 128, 64, ALG)->SEG_8192_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 256, 32, ALG)->SEG_8192_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 512, 16, ALG)->SEG_8192_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 1024, 8, ALG)->SEG_8192_ARGS()->UseManualTime();            \
+  BENCHMARK_TEMPLATE(NAME, 32, 512, ALG)->SEG_16384_ARGS()->UseManualTime();           \
+  BENCHMARK_TEMPLATE(NAME, 64, 256, ALG)->SEG_16384_ARGS()->UseManualTime();           \
+  BENCHMARK_TEMPLATE(NAME, 128, 128, ALG)->SEG_16384_ARGS()->UseManualTime();          \
+  BENCHMARK_TEMPLATE(NAME, 256, 64, ALG)->SEG_16384_ARGS()->UseManualTime();           \
+  BENCHMARK_TEMPLATE(NAME, 512, 32, ALG)->SEG_16384_ARGS()->UseManualTime();           \
+  BENCHMARK_TEMPLATE(NAME, 1024, 16, ALG)->SEG_16384_ARGS()->UseManualTime()
+// cub::Warp*: 32 ... 1024 threads per block, logical warps of 16 and 32 (src/reduction/seg_cub_warp.cu:145-161)
+#define RUN_CUB_WARP(NAME)                                        \
+  BENCHMARK_TEMPLATE(NAME, 32, 16)->SEG_16_ARGS()->UseManualTime();   \
+  BENCHMARK_TEMPLATE(NAME, 64, 16)->SEG_16_ARGS()->UseManualTime();   \
+  BENCHMARK_TEMPLATE(NAME, 128, 16)->SEG_16_ARGS()->UseManualTime();  \
+  BENCHMARK_TEMPLATE(NAME, 256, 16)->SEG_16_ARGS()->UseManualTime();  \
+  BENCHMARK_TEMPLATE(NAME, 512, 16)->SEG_16_ARGS()->UseManualTime();  \
+  BENCHMARK_TEMPLATE(NAME, 1024, 16)->SEG_16_ARGS()->UseManualTime(); \
+  BENCHMARK_TEMPLATE(NAME, 32, 32)->SEG_32_ARGS()->UseManualTime();   \
+  BENCHMARK_TEMPLATE(NAME, 64, 32)->SEG_32_ARGS()->UseManualTime();   \
+  BENCHMARK_TEMPLATE(NAME, 128, 32)->SEG_32_ARGS()->UseManualTime();  \
+  BENCHMARK_TEMPLATE(NAME, 256, 32)->SEG_32_ARGS()->UseManualTime();  \
+  BENCHMARK_TEMPLATE(NAME, 512, 32)->SEG_32_ARGS()->UseManualTime();  \
+  BENCHMARK_TEMPLATE(NAME, 1024, 32)->SEG_32_ARGS()->UseManualTime()
+
+constexpr auto Tuning16_x_14 = argspace::with_growing_segments<16, 14>;
+constexpr auto Tuning16_x_18 = argspace::with_growing_segments<16, 18>;
 constexpr auto Tuning16_x_22 = argspace::with_growing_segments<16, 22>;
 constexpr auto Tuning256_x_22 = argspace::with_growing_segments<256, 22>;
 constexpr auto Tuning16_x_26 = argspace::with_growing_segments<16, 26>;

@@ -90,6 +90,13 @@ void run_seg_reduce(benchmark::State &state, int variant, int tiles_per_wave, in
 void run_seg_reduce_offsets(benchmark::State &state, bool pass_expected_size, const char *name);
 void run_seg_scan_offsets(benchmark::State &state, const char *name);
 void run_seg_scan(benchmark::State &state, int variant, int tiles_per_wave, int waves_per_block, bool with_totals, const char *name);
+// Halves per block of the single-pass full-array kernels for the reference's template pair (SEGMENT_SIZE per warp
+// and step, WARPS_PER_BLOCK): their product, capped at what a block of this build holds in registers (8 tiles of 512
+// halves per wave); the reference's kernels loop over larger values, these do not need to
+inline size_t single_pass_partition(size_t segment_size, int waves_per_block) {
+  const size_t want = segment_size * (size_t)waves_per_block, most = (size_t)waves_per_block * 8 * 512;
+  return want < most ? want : most;
+}
 void run_full_reduce(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
 void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
 // half_out: y (GEMV) or C and D (GEMM) in fp16, the reference's H* benchmarks

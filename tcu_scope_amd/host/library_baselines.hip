@@ -170,7 +170,15 @@ BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_2048_ARGS()->UseManualTime();
 BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_4096_ARGS()->UseManualTime();
 BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_8192_ARGS()->UseManualTime();
 BENCHMARK(CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_16384_ARGS()->UseManualTime();
+// the reference registers the sweeps over 2^22 and 2^30 elements (src/reduction/seg_cub_device.cu:153-155) and its
+// figure specifications also ask for 2^14, 2^18 and 2^26 (figures/spec/tune_segmented_reduction*.yml); 2^28 is what
+// this build's measurements are quoted on
+BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_14)->UseManualTime();
+BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_18)->UseManualTime();
+BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_22)->UseManualTime();
+BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_26)->UseManualTime();
 BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
+BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_30)->UseManualTime();
 
 // ---- rocBLAS ------------------------------------------------------------------------------------
 namespace {
@@ -218,28 +226,43 @@ static void blas_gemm(benchmark::State &state, bool half_out) {
 }
 static void CUBLAS_WMMA_GEMM(benchmark::State &state) { blas_gemm(state, false); }
 static void CUBLAS_WMMA_HGEMM(benchmark::State &state) { blas_gemm(state, true); }
-BENCHMARK(CUBLAS_WMMA_HGEMM)->Apply(GemmArgs)->UseManualTime();
+// The reference times every product twice, with tensor-core math switched on (CUBLAS_WMMA_*) and off (CUBLAS_GEMM,
+// CUBLAS_HGEMM), and the fp16-output product also through cublasGemmEx (src/gemm/cublas.cu:618-627).  rocBLAS has no
+// such switch and one entry point for these types, so the names below time the same library call as their twins.
+static void CUBLAS_GEMM(benchmark::State &state) { blas_gemm(state, false); }
+static void CUBLAS_HGEMM(benchmark::State &state) { blas_gemm(state, true); }
+static void CUBLAS_WMMA_HGEMM_GemmEx(benchmark::State &state) { blas_gemm(state, true); }
+static void CUBLAS_HGEMM_GemmEx(benchmark::State &state) { blas_gemm(state, true); }
+BENCHMARK(CUBLAS_GEMM)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUBLAS_WMMA_GEMM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUBLAS_HGEMM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUBLAS_WMMA_HGEMM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUBLAS_WMMA_HGEMM_GemmEx)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(CUBLAS_HGEMM_GemmEx)->Apply(GemmArgs)->UseManualTime();
 
-// y (M) = alpha * A (M x K row-major) x + beta * y as a one-column GEMM (fp16 in, fp32 out)
-static void CUBLAS_GEMV(benchmark::State &state) {
+// y (M) = alpha * A (M x K row-major) x + beta * y as a one-column GEMM (fp16 in, fp32 accumulate; y in fp32 or fp16):
+// what the reference's CUDA_WMMA_GEMV_CUBLAS / CUDA_WMMA_HGEMV_CUBLAS do with cuBLAS (src/gemv/wmma_cublas.cu:245-246) and,
+// in fp32, its CUBLAS_GEMV (src/gemv/cublas.cu:88)
+static void blas_gemv(benchmark::State &state, bool half_out) {
   guarded(state, [&] {
     const size_t M = state.range(0), K = state.range(1);
     const float alpha = 1.0f, beta = 0.0f;
-    DeviceBuffer A(M * K * 2), x(K * 2), y(M * 4);
+    const size_t out_size = half_out ? 2 : 4;
+    const rocblas_datatype out_type = half_out ? rocblas_datatype_f16_r : rocblas_datatype_f32_r;
+    DeviceBuffer A(M * K * 2), x(K * 2), y(M * out_size);
     TCU_CHECK(tcu_generate_f16(A.get(), M * K, harness::flags().seed, TCU_DIST_NORMAL, 0, nullptr));
     TCU_CHECK(tcu_generate_f16(x.get(), K, harness::flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
-    PRINT_IF_ERROR(hipMemset(y.get(), 0, M * 4));
+    PRINT_IF_ERROR(hipMemset(y.get(), 0, M * out_size));
     auto run = [&] {
       check_blas(rocblas_gemm_ex(blas(), rocblas_operation_transpose, rocblas_operation_none, (rocblas_int)M, 1, (rocblas_int)K, &alpha, A.get(), rocblas_datatype_f16_r, (rocblas_int)K, x.get(),
-                                 rocblas_datatype_f16_r, (rocblas_int)K, &beta, y.get(), rocblas_datatype_f32_r, (rocblas_int)M, y.get(), rocblas_datatype_f32_r, (rocblas_int)M, rocblas_datatype_f32_r,
+                                 rocblas_datatype_f16_r, (rocblas_int)K, &beta, y.get(), out_type, (rocblas_int)M, y.get(), out_type, (rocblas_int)M, rocblas_datatype_f32_r,
                                  rocblas_gemm_algo_standard, 0, 0),
                  "rocblas_gemm_ex");
     };
     run();
     PRINT_IF_ERROR(hipDeviceSynchronize());
     timed_loop(state, [&](size_t) { run(); });
-    const double bytes = 2.0 * M * K + 2.0 * K + 4.0 * M;
+    const double bytes = 2.0 * M * K + 2.0 * K + (double)out_size * M;
     state.counters.insert({{"M", (double)M},
                            {"N", (double)K},
                            {"flops", {state.iterations() * 2.0 * M * K, benchmark::Counter::kAvgThreadsRate}},
@@ -247,4 +270,9 @@ static void CUBLAS_GEMV(benchmark::State &state) {
                            {"hbm_peak_fraction", {state.iterations() * bytes / 8e12, benchmark::Counter::kAvgThreadsRate}}});
   });
 }
+static void CUBLAS_GEMV(benchmark::State &state) { blas_gemv(state, false); }
+static void CUDA_WMMA_GEMV_CUBLAS(benchmark::State &state) { blas_gemv(state, false); }
+static void CUDA_WMMA_HGEMV_CUBLAS(benchmark::State &state) { blas_gemv(state, true); }
 BENCHMARK(CUBLAS_GEMV)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_GEMV_CUBLAS)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(CUDA_WMMA_HGEMV_CUBLAS)->Apply(GemvArgs)->UseManualTime();

@@ -56,45 +56,20 @@ RUN_256(1);
 RUN_256(2);
 RUN_256(4);
 RUN_256(8);
-#define RUN_WPB(NAME, ARGS_MACRO)                                   \
-  BENCHMARK_TEMPLATE(NAME, 1)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 2)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 4)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 8)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 16)->ARGS_MACRO()->UseManualTime()
-#define RUN_WPB_APPLY(NAME, FN)                                     \
-  BENCHMARK_TEMPLATE(NAME, 1)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 2)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 4)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 8)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 16)->Apply(FN)->UseManualTime()
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N, SEG_16_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N, SEG_32_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N, SEG_64_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N, SEG_128_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N, SEG_256_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N_OPT, SEG_16_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N_OPT, SEG_256_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N_BLOCK, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N_BLOCK, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N, SEG_256_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N, SEG_2048_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N, SEG_4096_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N, SEG_8192_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N, SEG_16384_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK, SEG_2048_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK, SEG_4096_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK, SEG_8192_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK, SEG_16384_ARGS);
+// the reference's lists (src/prefixsum/seg_wmma_16n.cu:217-223, seg_wmma_16n_opt.cu:217-223, seg_wmma_16n_block.cu:232-238,
+// seg_wmma_256n.cu:216-222, seg_wmma_256n_block.cu:227-233; tuning sweeps :208 / :205-208 of the same files), plus the
+// sweeps over 2^28 elements that the measurements of this build are quoted on
+RUN_WPB_SEG_16_TO_1024(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N);
+RUN_WPB_SEG_16_TO_1024(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N_OPT);
+RUN_WPB_SEG_16_TO_1024(CUDA_WMMA_SEGMENTED_PREFIXSUM_16N_BLOCK);
+RUN_WPB_SEG_256_TO_16384(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N);
+RUN_WPB_SEG_256_TO_16384(CUDA_WMMA_SEGMENTED_PREFIXSUM_256N_BLOCK);
 RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_PREFIXSUM_16N, Tuning16_x_28);
+RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_PREFIXSUM_16N, Tuning16_x_30);
+RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_PREFIXSUM_256N, Tuning256_x_22);
 RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_PREFIXSUM_256N, Tuning256_x_28);
 RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_PREFIXSUM_256N, Tuning256_x_30);
+RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_PREFIXSUM_256N_BLOCK, Tuning256_x_22);
 RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_PREFIXSUM_256N_BLOCK, Tuning256_x_30);
 BENCHMARK(TCU_AUTO_SEGMENTED_PREFIXSUM)->SEG_16_ARGS()->UseManualTime();
 BENCHMARK(TCU_AUTO_SEGMENTED_PREFIXSUM)->SEG_256_ARGS()->UseManualTime();
@@ -108,7 +83,8 @@ static void CUB_WARP_SEGMENTED_PREFIXSUM(benchmark::State &state) {
     state.SkipWithError("segment size must equal the logical warp size");
     return;
   }
-  run_seg_scan(state, TCU_VARIANT_WAVE_SHUFFLE, 0, THREADS_PER_BLOCK / 64, false, "CUB_WARP_SEGMENTED_PREFIXSUM");
+  // a block of 32 threads is half a wave here: it runs as one wave
+  run_seg_scan(state, TCU_VARIANT_WAVE_SHUFFLE, 0, THREADS_PER_BLOCK >= 64 ? THREADS_PER_BLOCK / 64 : 1, false, "CUB_WARP_SEGMENTED_PREFIXSUM");
 }
 enum { BLOCK_SCAN_RAKING = 0 };
 template <int THREADS_PER_BLOCK, int ITEMS_PER_THREAD, int ALGORITHM>
@@ -117,28 +93,12 @@ static void CUB_BLOCK_SEGMENTED_PREFIXSUM(benchmark::State &state) {
     state.SkipWithError("segment size must equal THREADS_PER_BLOCK * ITEMS_PER_THREAD");
     return;
   }
+  // as in the reduction: ITEMS_PER_THREAD / 8 loads in flight per lane; below 512 halves the block is a launch shape
   const int tiles = ITEMS_PER_THREAD >= 64 ? 8 : ITEMS_PER_THREAD >= 32 ? 4 : ITEMS_PER_THREAD >= 16 ? 2 : 1;
-  run_seg_scan(state, TCU_VARIANT_BLOCK_LDS, tiles, THREADS_PER_BLOCK / 64, false, "CUB_BLOCK_SEGMENTED_PREFIXSUM");
+  run_seg_scan(state, TCU_VARIANT_BLOCK_LDS, tiles, THREADS_PER_BLOCK >= 64 ? THREADS_PER_BLOCK / 64 : 1, false, "CUB_BLOCK_SEGMENTED_PREFIXSUM");
 }
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 64, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 128, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 256, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 512, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 1024, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 64, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 256, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_PREFIXSUM, 1024, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 64, 8, BLOCK_SCAN_RAKING)->SEG_512_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 128, 8, BLOCK_SCAN_RAKING)->SEG_1024_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 256, 8, BLOCK_SCAN_RAKING)->SEG_2048_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 128, 16, BLOCK_SCAN_RAKING)->SEG_2048_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 512, 8, BLOCK_SCAN_RAKING)->SEG_4096_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 128, 32, BLOCK_SCAN_RAKING)->SEG_4096_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 512, 16, BLOCK_SCAN_RAKING)->SEG_8192_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 256, 32, BLOCK_SCAN_RAKING)->SEG_8192_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 1024, 16, BLOCK_SCAN_RAKING)->SEG_16384_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 512, 32, BLOCK_SCAN_RAKING)->SEG_16384_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_PREFIXSUM, 256, 64, BLOCK_SCAN_RAKING)->SEG_16384_ARGS()->UseManualTime();
+RUN_CUB_WARP(CUB_WARP_SEGMENTED_PREFIXSUM);
+RUN_CUB_BLOCK(CUB_BLOCK_SEGMENTED_PREFIXSUM, BLOCK_SCAN_RAKING);
 
 // ---- full-array prefix sum -----------------------------------------------------------------
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>
@@ -153,27 +113,44 @@ static void CUDA_WMMA_FULL_PREFIXSUM_3KERS_BLOCK(benchmark::State &state) {
 // upstream; the decoupled look-back kernel takes their place)
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>
 static void CUDA_WMMA_FULL_PREFIXSUM_CG(benchmark::State &state) {
-  run_full_scan(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, (size_t)SEGMENT_SIZE * WARPS_PER_BLOCK, WARPS_PER_BLOCK, "CUDA_WMMA_FULL_PREFIXSUM_CG");
+  run_full_scan(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, harness::single_pass_partition(SEGMENT_SIZE, WARPS_PER_BLOCK), WARPS_PER_BLOCK, "CUDA_WMMA_FULL_PREFIXSUM_CG");
 }
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>
 static void CUDA_WMMA_FULL_PREFIXSUM_ATOMIC_W_ATOMIC_BALLOT(benchmark::State &state) {
-  run_full_scan(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, (size_t)SEGMENT_SIZE * WARPS_PER_BLOCK, WARPS_PER_BLOCK, "CUDA_WMMA_FULL_PREFIXSUM_ATOMIC_W_ATOMIC_BALLOT");
+  run_full_scan(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, harness::single_pass_partition(SEGMENT_SIZE, WARPS_PER_BLOCK), WARPS_PER_BLOCK, "CUDA_WMMA_FULL_PREFIXSUM_ATOMIC_W_ATOMIC_BALLOT");
 }
 static void TCU_AUTO_FULL_PREFIXSUM(benchmark::State &state) { run_full_scan(state, TCU_FULL_AUTO, 0, 0, "TCU_AUTO_FULL_PREFIXSUM"); }
 
-#define BENCHMARK_PRIFIXSUM0(SEGMENT_SIZE, WARPS_PER_BLOCK)                                                                 \
-  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_PREFIXSUM_3KERS, SEGMENT_SIZE, WARPS_PER_BLOCK)->ARGS()->UseManualTime();              \
-  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_PREFIXSUM_3KERS_BLOCK, SEGMENT_SIZE, WARPS_PER_BLOCK)->ARGS()->UseManualTime();        \
-  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_PREFIXSUM_CG, SEGMENT_SIZE, WARPS_PER_BLOCK)->ARGS()->UseManualTime();                 \
-  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_PREFIXSUM_ATOMIC_W_ATOMIC_BALLOT, SEGMENT_SIZE, WARPS_PER_BLOCK)->ARGS()->UseManualTime()
-#define BENCHMARK_PRIFIXSUM(SEGMENT_SIZE) \
-  BENCHMARK_PRIFIXSUM0(SEGMENT_SIZE, 1);  \
-  BENCHMARK_PRIFIXSUM0(SEGMENT_SIZE, 2);  \
-  BENCHMARK_PRIFIXSUM0(SEGMENT_SIZE, 4);  \
-  BENCHMARK_PRIFIXSUM0(SEGMENT_SIZE, 8);  \
-  BENCHMARK_PRIFIXSUM0(SEGMENT_SIZE, 16)
+// the reference's lists: SEGMENT_SIZE 256 ... 16 * 256 for the three-kernel family (src/prefixsum/wmma_3kers.cu:173-177),
+// up to 256 * 256 for its block form (wmma_3kers_block.cu:175-183), up to 1024 * 256 for the single-kernel forms
+// (wmma_cg.cu:196-207, wmma_atomic.cu:190-200)
+#define BENCHMARK_FULL_SCAN(NAME, SEGMENT_SIZE)                                   \
+  BENCHMARK_TEMPLATE(NAME, SEGMENT_SIZE, 1)->ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, SEGMENT_SIZE, 2)->ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, SEGMENT_SIZE, 4)->ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, SEGMENT_SIZE, 8)->ARGS()->UseManualTime();             \
+  BENCHMARK_TEMPLATE(NAME, SEGMENT_SIZE, 16)->ARGS()->UseManualTime()
+#define BENCHMARK_PRIFIXSUM(SEGMENT_SIZE)                                         \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_3KERS, SEGMENT_SIZE);              \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_3KERS_BLOCK, SEGMENT_SIZE);        \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_CG, SEGMENT_SIZE);                 \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_ATOMIC_W_ATOMIC_BALLOT, SEGMENT_SIZE)
+#define BENCHMARK_PRIFIXSUM_LARGE(SEGMENT_SIZE)                                   \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_3KERS_BLOCK, SEGMENT_SIZE);        \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_CG, SEGMENT_SIZE);                 \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_ATOMIC_W_ATOMIC_BALLOT, SEGMENT_SIZE)
+#define BENCHMARK_PRIFIXSUM_LARGEST(SEGMENT_SIZE)                                 \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_CG, SEGMENT_SIZE);                 \
+  BENCHMARK_FULL_SCAN(CUDA_WMMA_FULL_PREFIXSUM_ATOMIC_W_ATOMIC_BALLOT, SEGMENT_SIZE)
+BENCHMARK_PRIFIXSUM(256);
 BENCHMARK_PRIFIXSUM(2 * 256);
 BENCHMARK_PRIFIXSUM(4 * 256);
 BENCHMARK_PRIFIXSUM(8 * 256);
 BENCHMARK_PRIFIXSUM(16 * 256);
+BENCHMARK_PRIFIXSUM_LARGE(32 * 256);
+BENCHMARK_PRIFIXSUM_LARGE(64 * 256);
+BENCHMARK_PRIFIXSUM_LARGE(128 * 256);
+BENCHMARK_PRIFIXSUM_LARGE(256 * 256);
+BENCHMARK_PRIFIXSUM_LARGEST(512 * 256);
+BENCHMARK_PRIFIXSUM_LARGEST(1024 * 256);
 BENCHMARK(TCU_AUTO_FULL_PREFIXSUM)->ARGS()->UseManualTime();

@@ -61,44 +61,14 @@ RUN_256(2);
 RUN_256(4);
 RUN_256(8);
 
-#define RUN_WPB(NAME, ARGS_MACRO)                                   \
-  BENCHMARK_TEMPLATE(NAME, 1)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 2)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 4)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 8)->ARGS_MACRO()->UseManualTime();       \
-  BENCHMARK_TEMPLATE(NAME, 16)->ARGS_MACRO()->UseManualTime()
-#define RUN_WPB_APPLY(NAME, FN)                                     \
-  BENCHMARK_TEMPLATE(NAME, 1)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 2)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 4)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 8)->Apply(FN)->UseManualTime();          \
-  BENCHMARK_TEMPLATE(NAME, 16)->Apply(FN)->UseManualTime()
-
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N, SEG_16_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N, SEG_32_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N, SEG_64_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N, SEG_128_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N, SEG_256_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N_OPT, SEG_16_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N_OPT, SEG_256_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N_OPT, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N_BLOCK, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_16N_BLOCK, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N, SEG_256_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N, SEG_2048_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N, SEG_4096_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N, SEG_8192_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N, SEG_16384_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK, SEG_512_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK, SEG_1024_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK, SEG_2048_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK, SEG_4096_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK, SEG_8192_ARGS);
-RUN_WPB(CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK, SEG_16384_ARGS);
+// the reference's lists (src/reduction/seg_wmma_16n.cu:215-221, seg_wmma_16n_opt.cu:215-221, seg_wmma_16n_block.cu:229-235,
+// seg_wmma_256n.cu:223-229, seg_wmma_256n_block.cu:242-248; tuning sweeps :206 / :212-214 of the same files), plus the
+// sweeps over 2^28 elements that the measurements of this build are quoted on
+RUN_WPB_SEG_16_TO_1024(CUDA_WMMA_SEGMENTED_REDUCTION_16N);
+RUN_WPB_SEG_16_TO_1024(CUDA_WMMA_SEGMENTED_REDUCTION_16N_OPT);
+RUN_WPB_SEG_16_TO_1024(CUDA_WMMA_SEGMENTED_REDUCTION_16N_BLOCK);
+RUN_WPB_SEG_256_TO_16384(CUDA_WMMA_SEGMENTED_REDUCTION_256N);
+RUN_WPB_SEG_256_TO_16384(CUDA_WMMA_SEGMENTED_REDUCTION_256N_BLOCK);
 RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_REDUCTION_16N, Tuning16_x_28);
 RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_REDUCTION_16N, Tuning16_x_30);
 RUN_WPB_APPLY(CUDA_WMMA_TUNE_SEGMENTED_REDUCTION_16N_BLOCK, Tuning16_x_30);
@@ -123,7 +93,8 @@ static void CUB_WARP_SEGMENTED_REDUCTION(benchmark::State &state) {
     state.SkipWithError("segment size must equal the logical warp size");
     return;
   }
-  run_seg_reduce(state, TCU_VARIANT_WAVE_SHUFFLE, 0, THREADS_PER_BLOCK / 64, "CUB_WARP_SEGMENTED_REDUCTION");
+  // a block of 32 threads is half a wave here: it runs as one wave
+  run_seg_reduce(state, TCU_VARIANT_WAVE_SHUFFLE, 0, THREADS_PER_BLOCK >= 64 ? THREADS_PER_BLOCK / 64 : 1, "CUB_WARP_SEGMENTED_REDUCTION");
 }
 enum { BLOCK_REDUCE_RAKING = 0 };
 template <int THREADS_PER_BLOCK, int ITEMS_PER_THREAD, int ALGORITHM>
@@ -132,34 +103,13 @@ static void CUB_BLOCK_SEGMENTED_REDUCTION(benchmark::State &state) {
     state.SkipWithError("segment size must equal THREADS_PER_BLOCK * ITEMS_PER_THREAD");
     return;
   }
-  // a lane takes 8 items per 128-bit load; ITEMS_PER_THREAD / 8 such loads stay in flight
+  // a lane takes 8 items per 128-bit load; ITEMS_PER_THREAD / 8 such loads stay in flight (at most 8); segments
+  // below 512 halves lie inside one wave's tile and the block is a launch shape of the wave kernel
   const int tiles = ITEMS_PER_THREAD >= 64 ? 8 : ITEMS_PER_THREAD >= 32 ? 4 : ITEMS_PER_THREAD >= 16 ? 2 : 1;
-  run_seg_reduce(state, TCU_VARIANT_BLOCK_LDS, tiles, THREADS_PER_BLOCK / 64, "CUB_BLOCK_SEGMENTED_REDUCTION");
+  run_seg_reduce(state, TCU_VARIANT_BLOCK_LDS, tiles, THREADS_PER_BLOCK >= 64 ? THREADS_PER_BLOCK / 64 : 1, "CUB_BLOCK_SEGMENTED_REDUCTION");
 }
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 64, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 128, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 256, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 512, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 1024, 16)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 64, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 128, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 256, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 512, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_WARP_SEGMENTED_REDUCTION, 1024, 32)->SEG_32_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 64, 8, BLOCK_REDUCE_RAKING)->SEG_512_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 128, 8, BLOCK_REDUCE_RAKING)->SEG_1024_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 64, 16, BLOCK_REDUCE_RAKING)->SEG_1024_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 256, 8, BLOCK_REDUCE_RAKING)->SEG_2048_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 128, 16, BLOCK_REDUCE_RAKING)->SEG_2048_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 512, 8, BLOCK_REDUCE_RAKING)->SEG_4096_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 256, 16, BLOCK_REDUCE_RAKING)->SEG_4096_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 128, 32, BLOCK_REDUCE_RAKING)->SEG_4096_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 1024, 8, BLOCK_REDUCE_RAKING)->SEG_8192_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 512, 16, BLOCK_REDUCE_RAKING)->SEG_8192_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 256, 32, BLOCK_REDUCE_RAKING)->SEG_8192_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 1024, 16, BLOCK_REDUCE_RAKING)->SEG_16384_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 512, 32, BLOCK_REDUCE_RAKING)->SEG_16384_ARGS()->UseManualTime();
-BENCHMARK_TEMPLATE(CUB_BLOCK_SEGMENTED_REDUCTION, 256, 64, BLOCK_REDUCE_RAKING)->SEG_16384_ARGS()->UseManualTime();
+RUN_CUB_WARP(CUB_WARP_SEGMENTED_REDUCTION);
+RUN_CUB_BLOCK(CUB_BLOCK_SEGMENTED_REDUCTION, BLOCK_REDUCE_RAKING);
 
 // ---- full-array reduction --------------------------------------------------------------------
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>
@@ -173,20 +123,24 @@ static void CUDA_WMMA_FULL_REDUCTION_2KERS_BASE_256(benchmark::State &state) {
 // single kernel with an atomic carry: the reference's atomic (block-sync / atomic-ballot) and
 // cooperative-groups variants differ only in how a block agrees on its partial; here a block
 // always combines through LDS, so the three names run the same kernel
+// SEGMENT_SIZE is what a warp takes per step in the reference; a block of this build holds its whole partition in
+// registers, at most 8 tiles (4096 halves) per wave: larger template arguments run with that partition
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>
 static void CUDA_WMMA_FULL_REDUCTION_ATOMIC_W_BLOCK_SYNC(benchmark::State &state) {
-  run_full_reduce(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, SEGMENT_SIZE * WARPS_PER_BLOCK, WARPS_PER_BLOCK, "CUDA_WMMA_FULL_REDUCTION_ATOMIC_W_BLOCK_SYNC");
+  run_full_reduce(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, harness::single_pass_partition(SEGMENT_SIZE, WARPS_PER_BLOCK), WARPS_PER_BLOCK, "CUDA_WMMA_FULL_REDUCTION_ATOMIC_W_BLOCK_SYNC");
 }
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>
 static void CUDA_WMMA_FULL_REDUCTION_ATOMIC_W_ATOMIC_BALLOT(benchmark::State &state) {
-  run_full_reduce(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, SEGMENT_SIZE * WARPS_PER_BLOCK, WARPS_PER_BLOCK, "CUDA_WMMA_FULL_REDUCTION_ATOMIC_W_ATOMIC_BALLOT");
+  run_full_reduce(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, harness::single_pass_partition(SEGMENT_SIZE, WARPS_PER_BLOCK), WARPS_PER_BLOCK, "CUDA_WMMA_FULL_REDUCTION_ATOMIC_W_ATOMIC_BALLOT");
 }
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>
 static void CUDA_WMMA_FULL_REDUCTION_CG(benchmark::State &state) {
-  run_full_reduce(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, SEGMENT_SIZE * WARPS_PER_BLOCK, WARPS_PER_BLOCK, "CUDA_WMMA_FULL_REDUCTION_CG");
+  run_full_reduce(state, TCU_FULL_SINGLE_PASS | TCU_FULL_MFMA, harness::single_pass_partition(SEGMENT_SIZE, WARPS_PER_BLOCK), WARPS_PER_BLOCK, "CUDA_WMMA_FULL_REDUCTION_CG");
 }
 static void TCU_AUTO_FULL_REDUCTION(benchmark::State &state) { run_full_reduce(state, TCU_FULL_AUTO, 0, 0, "TCU_AUTO_FULL_REDUCTION"); }
 
+// the reference's lists: SEGMENT_SIZE 256 ... 16 * 256 for the two-kernel and atomic families
+// (src/reduction/wmma_2kers.cu:189-193, wmma_atomic.cu:181-185), up to 1024 * 256 for the cooperative-groups one (wmma_cg.cu:184-195)
 #define BENCHMARK_REDUCTION0(SEGMENT_SIZE, WARPS_PER_BLOCK)                                                                        \
   BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_REDUCTION_2KERS_BASE_16, SEGMENT_SIZE, WARPS_PER_BLOCK)->ARGS()->UseManualTime();              \
   BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_REDUCTION_2KERS_BASE_256, SEGMENT_SIZE, WARPS_PER_BLOCK)->ARGS()->UseManualTime();             \
@@ -199,8 +153,21 @@ static void TCU_AUTO_FULL_REDUCTION(benchmark::State &state) { run_full_reduce(s
   BENCHMARK_REDUCTION0(SEGMENT_SIZE, 4);  \
   BENCHMARK_REDUCTION0(SEGMENT_SIZE, 8);  \
   BENCHMARK_REDUCTION0(SEGMENT_SIZE, 16)
+#define BENCHMARK_REDUCTION_CG(SEGMENT_SIZE)                                                          \
+  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_REDUCTION_CG, SEGMENT_SIZE, 1)->ARGS()->UseManualTime();          \
+  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_REDUCTION_CG, SEGMENT_SIZE, 2)->ARGS()->UseManualTime();          \
+  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_REDUCTION_CG, SEGMENT_SIZE, 4)->ARGS()->UseManualTime();          \
+  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_REDUCTION_CG, SEGMENT_SIZE, 8)->ARGS()->UseManualTime();          \
+  BENCHMARK_TEMPLATE(CUDA_WMMA_FULL_REDUCTION_CG, SEGMENT_SIZE, 16)->ARGS()->UseManualTime()
+BENCHMARK_REDUCTION(256);
 BENCHMARK_REDUCTION(2 * 256);
 BENCHMARK_REDUCTION(4 * 256);
 BENCHMARK_REDUCTION(8 * 256);
 BENCHMARK_REDUCTION(16 * 256);
+BENCHMARK_REDUCTION_CG(32 * 256);
+BENCHMARK_REDUCTION_CG(64 * 256);
+BENCHMARK_REDUCTION_CG(128 * 256);
+BENCHMARK_REDUCTION_CG(256 * 256);
+BENCHMARK_REDUCTION_CG(512 * 256);
+BENCHMARK_REDUCTION_CG(1024 * 256);
 BENCHMARK(TCU_AUTO_FULL_REDUCTION)->ARGS()->UseManualTime();

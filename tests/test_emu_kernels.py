@@ -62,9 +62,9 @@ def copy_in(x, dtype=np.uint16):
 
 
 CASES = [  # (segment size, variants, (tiles per wave, waves per block) list, segment counts)
-    (16, (V_WAVE, V_MFMA_16, V_MFMA_16N, V_AUTO), ((8, 2), (1, 1)), (96, 1027)),
-    (64, (V_WAVE, V_MFMA_16N), ((4, 1),), (37,)),
-    (256, (V_WAVE, V_MFMA_256, V_MFMA_256N), ((2, 2), (8, 1)), (19,)),
+    (16, (V_WAVE, V_MFMA_16, V_MFMA_16N, V_AUTO, V_MFMA_16N_BLOCK, V_BLOCK), ((8, 2), (1, 1), (0, 4)), (96, 1027)),
+    (64, (V_WAVE, V_MFMA_16N, V_BLOCK), ((4, 1), (0, 0)), (37,)),
+    (256, (V_WAVE, V_MFMA_256, V_MFMA_256N, V_MFMA_256N_BLOCK, V_MFMA_16N_BLOCK), ((2, 2), (8, 1), (0, 2)), (19,)),
     (512, (V_WAVE, V_MFMA_16N, V_BLOCK, V_MFMA_256N_BLOCK), ((2, 1),), (9,)),
     (2048, (V_WAVE, V_MFMA_256N, V_BLOCK, V_MFMA_16N_BLOCK, V_AUTO), ((2, 2), (8, 1)), (5,)),
     (8192, (V_WAVE, V_MFMA_16N, V_MFMA_256N_BLOCK), ((4, 2),), (3,)),
@@ -208,7 +208,8 @@ def test_generic_segment_sizes_and_preconditions(emu, oracle):
         assert emu.emu_seg_reduce_f16(xi.ctypes.data, red.ctypes.data, nseg, seg, V_WAVE, 0, 0) == 2
     xi = copy_in(np.zeros(512, np.uint16))
     assert emu.emu_seg_reduce_f16(xi.ctypes.data, xi.ctypes.data, 4, 32, V_MFMA_16, 0, 0) == 2 and b"must be 16" in emu.emu_last_error()
-    assert emu.emu_seg_scan_f16(xi.ctypes.data, xi.ctypes.data, None, 2, 256, V_BLOCK, 0, 0) == 2
+    assert emu.emu_seg_scan_f16(xi.ctypes.data, xi.ctypes.data, None, 4, 128, V_MFMA_256N_BLOCK, 0, 0) == 2 and b"256" in emu.emu_last_error()
+    assert emu.emu_seg_scan_f16(xi.ctypes.data, xi.ctypes.data, None, 2, 24, V_BLOCK, 0, 0) == 2
 
 
 def test_full_array_kernels(emu, oracle):

@@ -21,15 +21,15 @@ def tcu():
 
 def variants_for(tcu, seg):
     V = tcu.Variant
-    out = [V.AUTO, V.WAVE_SHUFFLE, V.MFMA_16N]
+    # the block families take every size the reference registers them at (16 ... for *_16N_BLOCK and cub::Block*,
+    # 256 ... for *_256N_BLOCK); below 512 halves they are launch shapes of the wave kernels
+    out = [V.AUTO, V.WAVE_SHUFFLE, V.MFMA_16N, V.BLOCK_LDS, V.MFMA_16N_BLOCK]
     if seg == 16:
         out.append(V.MFMA_16)
     if seg == 256:
         out.append(V.MFMA_256)
     if seg >= 256:
-        out.append(V.MFMA_256N)
-    if seg >= 512:
-        out += [V.BLOCK_LDS, V.MFMA_256N_BLOCK, V.MFMA_16N_BLOCK]
+        out += [V.MFMA_256N, V.MFMA_256N_BLOCK]
     return out
 
 
@@ -201,7 +201,7 @@ def test_ragged_and_edge_cases(tcu, oracle):
     assert tcu.seg_reduce(empty, 16).numel() == 0 and tcu.seg_scan(empty, 16).numel() == 0
     # the reference's precondition failures map to "unsupported"
     x = to_dev(oracle.generate_f16(4096, 9, oracle.DIST_UNIFORM))
-    for v, seg in [(V.MFMA_16, 32), (V.MFMA_256, 16), (V.MFMA_256N, 128), (V.BLOCK_LDS, 256)]:
+    for v, seg in [(V.MFMA_16, 32), (V.MFMA_256, 16), (V.MFMA_256N, 128), (V.MFMA_256N_BLOCK, 128), (V.BLOCK_LDS, 24)]:
         with pytest.raises(tcu.TcuError) as e:
             tcu.seg_reduce(x, seg, variant=v)
         assert e.value.status == 2
