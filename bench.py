@@ -4,17 +4,28 @@ N = 2^28 elements, segment sizes 16..16384, on one MI355X.
 
 A step is one pass over the whole sweep: 5 segmented reductions (seg 16, 256, 1024, 4096,
 16384) and 4 segmented scans (seg 16, 256, 2048, 16384), each over 2^28 synthetic
-elements already resident in HBM.  `value` = elements processed per second over the
-timed steps (wall clock, synchronised on both sides).  The same steps then run once more
-with a pair of HIP events per launch on the launch stream, stamped by the kernel's own
-dispatch with its begin and end (tcu_time_next_launch); from those come the per-kernel
-bandwidths and the `roofline` object (algorithmic bytes / average kernel time / 8 TB/s).
-Two input buffers alternate between launches so that no launch finds its input in the
-256 MB Infinity Cache.
+elements already resident in HBM.  Order of the run:
+
+1. every launch of the sweep (and of `all_sizes`: both operations at every power of two from
+   16 to 16384) runs once and a window of 2^24 elements of its output is compared with the
+   fp64 sums of the same seeded inputs (CPU oracle, |err| <= 2 ulp_fp16 + 1e-3 * sqrt(segment
+   size)); a mismatch ends the run with a non-zero status.  Outside every timed region.
+2. warm-up steps, then the timed region: exactly `steps` steps, nothing on the stream but the
+   launches, wall clock, synchronised on both sides -> `value`.
+3. the same steps once more with a pair of HIP events per launch on the launch stream, stamped
+   by the kernel's own dispatch with its begin and end (tcu_time_next_launch): per-kernel
+   bandwidths and the `roofline` object (algorithmic bytes / average kernel time / 8 TB/s).
+4. `all_sizes`, timed like 3.
+5. the CPU baseline: the reference's CPU path (restated in oracle/) on the same sweep.
+
+Two input buffers alternate between launches so that no launch finds its input in the 256 MB
+Infinity Cache.
 """
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,15 +37,35 @@ HBM_PEAK_GBS = 8000.0
 N_LOG2 = 28
 REDUCE_SEGS = [16, 256, 1024, 4096, 16384]
 SCAN_SEGS = [16, 256, 2048, 16384]
+ALL_SIZES = [16 << i for i in range(11)]  # 16 ... 16384
+CHECK_WINDOW_LOG2 = 24
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "seg_reduce_scan_2p28_hbm_traffic.md")
+KERNEL_SOURCES = ["wave_ops.hpp", "seg_reduce.hpp", "seg_scan.hpp", "dispatch.hpp"]
 
 
-# HBM bytes per launch at N = 2^28 with the AUTO launch shapes, from rocprofv3 FETCH_SIZE /
-# WRITE_SIZE runs of this script, each counter scaled by what it reads for the plain copy
-# kernel of known size (profiles/seg_reduce_scan_2p28_hbm_traffic.md).
-MEASURED_TRAFFIC_2P28_AUTO = {
-    ("reduce", 16): 570417963, ("reduce", 256): 538966187, ("reduce", 1024): 537931269, ("reduce", 4096): 537925093, ("reduce", 16384): 537136897,
-    ("scan", 16): 1073728548, ("scan", 256): 1073787570, ("scan", 2048): 1073609230, ("scan", 16384): 1073637069,
-}
+def kernel_sources_digest():
+    """sha256 over the sources that decide what the segmented launches do (kernels and launch shapes)."""
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "tcu_scope_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic():
+    """HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE summary in profiles/, but only if that
+    summary was made from the kernel sources of this tree (it records their digest); otherwise nothing."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return {}
+    m = re.search(r"kernel sources digest: `([0-9a-f]+)`", text)
+    if not m or m.group(1) != kernel_sources_digest():
+        return {}
+    out = {}
+    for op, seg, by in re.findall(r"\|\s*(reduce|scan) seg=(\d+)\s*\|.*?\|\s*(\d+)\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*$", text, re.M):
+        out[(op, int(seg))] = int(by)
+    return out
 
 
 def algorithmic_bytes(kind, n, seg):
@@ -67,10 +98,12 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--n-log2", type=int, default=N_LOG2, help="log2 of the element count (28 = the benchmark configuration)")
-    ap.add_argument("--variant", default="AUTO", help="kernel family for every launch (AUTO, WAVE_SHUFFLE, MFMA_16N, ...)")
+    ap.add_argument("--variant", default="AUTO", help="kernel family for every launch (AUTO, WAVE_SHUFFLE, MFMA_16N, ...); sizes the family does not cover are reported as skipped, never substituted")
     ap.add_argument("--tiles-per-wave", type=int, default=0)
     ap.add_argument("--waves-per-block", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true", help="skip the comparison with the CPU oracle before timing (for profiler runs)")
+    ap.add_argument("--no-all-sizes", action="store_true", help="skip the second list (every power of two 16 ... 16384)")
     ap.add_argument("--with-copy-probe", action="store_true", help="also launch the plain copy kernel over 2^n_log2 halves before timing (calibrates hardware counters)")
     ap.add_argument("--cpu-n-log2", type=int, default=28, help="element count of the CPU-baseline sample")
     args = ap.parse_args()
@@ -78,6 +111,7 @@ def main():
         print("bench.py: this build runs on one GPU only (--gpus 1); segments are independent, so a multi-GPU run would be N copies of this one", file=sys.stderr)
         sys.exit(2)
 
+    import numpy as np
     import torch
 
     import tcu_scope_amd as tcu
@@ -88,30 +122,63 @@ def main():
     variant = tcu.Variant[args.variant]
     stream = torch.cuda.current_stream()
 
-    inputs = [tcu.generate(n, 1, tcu.Dist.UNIFORM), tcu.generate(n, 2, tcu.Dist.UNIFORM)]
+    seeds = (1, 2)
+    inputs = [tcu.generate(n, s, tcu.Dist.UNIFORM) for s in seeds]
     red_out = torch.empty(n // 16, dtype=torch.float16, device="cuda")
     scan_out = torch.empty(n, dtype=torch.float16, device="cuda")
     configs = [("reduce", s) for s in REDUCE_SEGS] + [("scan", s) for s in SCAN_SEGS]
-
-    def supported(kind, seg):
-        V = tcu.Variant
-        if variant in (V.BLOCK_LDS, V.MFMA_256N_BLOCK, V.MFMA_16N_BLOCK):
-            return seg >= 512
-        if variant == V.MFMA_16:
-            return seg == 16
-        if variant == V.MFMA_256:
-            return seg == 256
-        if variant == V.MFMA_256N:
-            return seg >= 256
-        return True
+    all_sizes = [] if args.no_all_sizes else [("reduce", s) for s in ALL_SIZES] + [("scan", s) for s in ALL_SIZES]
 
     def launch(i, kind, seg):
         x = inputs[i & 1]
-        v = variant if supported(kind, seg) else tcu.Variant.AUTO
         if kind == "reduce":
-            tcu.seg_reduce(x, seg, variant=v, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=red_out, stream=stream)
+            tcu.seg_reduce(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=red_out, stream=stream)
         else:
-            tcu.seg_scan(x, seg, variant=v, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=scan_out, stream=stream)
+            tcu.seg_scan(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=scan_out, stream=stream)
+
+    # families do not cover every size (MFMA_16 is 16 only, ...): such launches are left out and said so
+    skipped = []
+    for kind, seg in list(dict.fromkeys(configs + all_sizes)):
+        try:
+            launch(0, kind, seg)
+        except tcu.TcuError as e:
+            if e.status != 2:
+                raise
+            skipped.append({"op": kind, "segment_size": seg, "reason": str(e)})
+    torch.cuda.synchronize()
+    unsupported = {(s["op"], s["segment_size"]) for s in skipped}
+    configs = [c for c in configs if c not in unsupported]
+    all_sizes = [c for c in all_sizes if c not in unsupported]
+    if not configs:
+        print("bench.py: the chosen variant covers no launch of the sweep", file=sys.stderr)
+        sys.exit(2)
+
+    # 1. every launch once, a window of its output against the fp64 sums of the same inputs
+    checked = None
+    if not args.no_check:
+        from oracle import binding as oracle
+
+        w = min(n, 1 << CHECK_WINDOW_LOG2)
+        first = (n - w) // 2  # a window in the middle of the array (a multiple of every segment size)
+        x_host = oracle.generate_f16(w, seeds[0], oracle.DIST_UNIFORM, first=first)
+        worst_excess = 0.0
+        for kind, seg in list(dict.fromkeys(configs + all_sizes)):
+            launch(0, kind, seg)
+            torch.cuda.synchronize()
+            nseg = w // seg
+            if kind == "reduce":
+                got = red_out[first // seg:first // seg + nseg].cpu().numpy().view(np.uint16)
+                ref = oracle.seg_reduce_f64(x_host, nseg, seg)
+            else:
+                got = scan_out[first:first + w].cpu().numpy().view(np.uint16)
+                ref = oracle.seg_scan_f64(x_host, nseg, seg)
+            bad, worst, first_bad = oracle.check_f16(got, ref, seg, 2.0, 1e-3)
+            if bad:
+                print(f"bench.py: seg_{kind} segment_size={seg} disagrees with the CPU oracle: {bad} of {got.size} outside 2 ulp + 1e-3*sqrt(S), first at {first_bad}", file=sys.stderr)
+                sys.exit(1)
+            worst_excess = max(worst_excess, worst)
+        checked = {"launches": len(dict.fromkeys(configs + all_sizes)), "window_elements": w, "window_first": first,
+                   "tolerance": "2 ulp_fp16 + 1e-3*sqrt(segment_size) against the fp64 sum", "passed": True}
 
     if args.with_copy_probe:
         for i in range(4):  # 2*n bytes read + 2*n bytes written per launch, same launch shape as the scan kernels
@@ -125,7 +192,7 @@ def main():
             counter += 1
     torch.cuda.synchronize()
 
-    # the timed region: exactly `steps` steps, nothing but the launches on the stream
+    # 2. the timed region: exactly `steps` steps, nothing but the launches on the stream
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
@@ -135,41 +202,55 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
 
-    # the same steps once more with a pair of events per launch, carried by the kernel's own
+    # 3. the same steps once more with a pair of events per launch, carried by the kernel's own
     # dispatch (tcu_time_next_launch): the pair brackets the kernel and nothing else.  Kept out of
-    # the region above because a dispatch that reports its times costs the step about 4 %
-    # (1.09 against 1.05 ms; an event recorded before and after every launch 1.12).
-    events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in configs] for _ in range(args.steps)]
-    for step_events in events:
-        for a, b in step_events:  # a torch event gets its handle with its first record
-            a.record(stream)
-            b.record(stream)
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    for k in range(args.steps):
-        for c, (kind, seg) in enumerate(configs):
-            tcu.time_next_launch(*events[k][c])
+    # the region above because a dispatch that reports its times costs the step about 4 %.
+    def timed_with_events(launches, repeats):
+        nonlocal counter
+        events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches] for _ in range(repeats)]
+        for step_events in events:
+            for a, b in step_events:  # a torch event gets its handle with its first record
+                a.record(stream)
+                b.record(stream)
+        torch.cuda.synchronize()
+        ta = time.perf_counter()
+        for k in range(repeats):
+            for c, (kind, seg) in enumerate(launches):
+                tcu.time_next_launch(*events[k][c])
+                launch(counter, kind, seg)
+                counter += 1
+        torch.cuda.synchronize()
+        tb = time.perf_counter()
+        rows = []
+        for c, (kind, seg) in enumerate(launches):
+            ms = sorted(events[k][c][0].elapsed_time(events[k][c][1]) for k in range(repeats))
+            avg = sum(ms) / len(ms)
+            by = algorithmic_bytes(kind, n, seg)
+            rows.append({
+                "op": kind, "segment_size": seg, "avg_ms": round(avg, 5), "min_ms": round(ms[0], 5), "median_ms": round(ms[len(ms) // 2], 5),
+                "gelem_per_s": round(n / avg / 1e6, 1), "algorithmic_bytes": by, "gb_per_s": round(by / avg / 1e6, 1),
+                "frac_hbm_peak": round(by / avg / 1e6 / HBM_PEAK_GBS, 4),
+            })
+        return rows, (tb - ta) / repeats
+
+    per_config, step_with_events_s = timed_with_events(configs, args.steps)
+    default_shapes = args.n_log2 == 28 and variant == tcu.Variant.AUTO and args.tiles_per_wave == 0 and args.waves_per_block == 0
+    traffic = measured_traffic() if default_shapes else {}
+    for r in per_config:
+        r["traffic"] = traffic.get((r["op"], r["segment_size"]))
+
+    # 4. every power of two from 16 to 16384, both operations (not part of `value`)
+    all_rows = None
+    if all_sizes:
+        for kind, seg in all_sizes:  # warm
             launch(counter, kind, seg)
             counter += 1
-    torch.cuda.synchronize()
-    t3 = time.perf_counter()
+        all_rows, _ = timed_with_events(all_sizes, max(5, args.steps // 2))
 
     total_s = t1 - t0
     elems_per_step = len(configs) * n
     value = args.steps * elems_per_step / total_s / 1e9
 
-    measured_shapes = args.n_log2 == 28 and variant == tcu.Variant.AUTO and args.tiles_per_wave == 0 and args.waves_per_block == 0
-    per_config = []
-    for c, (kind, seg) in enumerate(configs):
-        ms = sorted(events[k][c][0].elapsed_time(events[k][c][1]) for k in range(args.steps))
-        avg = sum(ms) / len(ms)
-        by = algorithmic_bytes(kind, n, seg)
-        per_config.append({
-            "op": kind, "segment_size": seg, "avg_ms": round(avg, 5), "min_ms": round(ms[0], 5), "median_ms": round(ms[len(ms) // 2], 5),
-            "gelem_per_s": round(n / avg / 1e6, 1), "algorithmic_bytes": by, "gb_per_s": round(by / avg / 1e6, 1),
-            "frac_hbm_peak": round(by / avg / 1e6 / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_2P28_AUTO.get((kind, seg)) if measured_shapes else None,
-        })
     # the dominant kernel: the launch that takes the largest share of a step
     dom = max(per_config, key=lambda r: r["avg_ms"])
     roofline = {
@@ -177,18 +258,27 @@ def main():
         "frac": dom["frac_hbm_peak"], "traffic": dom["traffic"], "algorithmic_bytes_per_launch": dom["algorithmic_bytes"], "avg_launch_ms": dom["avg_ms"],
         "min_frac_over_sweep": min(r["frac_hbm_peak"] for r in per_config),
     }
+    if all_rows:
+        roofline["min_frac_all_sizes_16_to_16384"] = min(r["frac_hbm_peak"] for r in all_rows)
 
     result = {
         "metric": "fp16 segmented reduce+scan throughput, 2^%d elems, seg 16..16384" % args.n_log2,
         "value": round(value, 2), "unit": "Gelem/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(total_s / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 in/out, f32 accumulate", "data": "synthetic (uniform [-1,1) fp16 from a seeded counter-based generator)",
-        "config": {"workload": "segmented sum reduction (seg 16,256,1024,4096,16384) + segmented inclusive scan (seg 16,256,2048,16384), N=2^%d fp16 each" % args.n_log2,
-                   "variant": variant.name, "tiles_per_wave": args.tiles_per_wave, "waves_per_block": args.waves_per_block, "compute_units": info["compute_units"]},
+        "config": {"workload": "segmented sum reduction (seg %s) + segmented inclusive scan (seg %s), N=2^%d fp16 each" % (
+                       ",".join(str(s) for k, s in configs if k == "reduce"), ",".join(str(s) for k, s in configs if k == "scan"), args.n_log2),
+                   "variant": variant.name, "tiles_per_wave": args.tiles_per_wave, "waves_per_block": args.waves_per_block, "compute_units": info["compute_units"],
+                   "kernel_sources_digest": kernel_sources_digest()},
         "roofline": roofline,
-        "ms_per_step_with_kernel_events": round((t3 - t2) / args.steps * 1e3, 4),
+        "checked_against_cpu_oracle": checked,
+        "ms_per_step_with_kernel_events": round(step_with_events_s * 1e3, 4),
         "per_config": per_config,
     }
+    if skipped:
+        result["skipped"] = skipped
+    if all_rows:
+        result["all_sizes"] = all_rows
     if not args.no_cpu_baseline:
         cpu1, dt1 = cpu_baseline(args.cpu_n_log2, 1)
         threads = min(16, os.cpu_count() or 1)
