@@ -184,6 +184,24 @@ int tcu_seg_scan_f16_noalloc(const void *d_in, void *d_out, void *d_totals, size
  * described by an offsets array (src/reduction/seg_cub_device.cu:18-22). */
 int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments, const void *d_begin_offsets, const void *d_end_offsets, int offset_bits, size_t expected_segment_size, void *stream);
 
+/* Segments given by a key array: a segment is a run of equal consecutive keys (d_keys: n signed integers of
+ * key_bits = 32 or 64 bits in device memory; n < 2^32).  d_keys, d_in and the scan's d_out must be 16-byte
+ * aligned.  Workspace: the two-phase protocol of the full-array entry points below (8 or 16 bytes per 32768
+ * elements).  One pass over keys and values (decoupled look-back on (head flag, value) pairs).
+ *
+ * tcu_seg_scan_by_key_f16: d_out[i] = fp16( sum of d_in[j .. i] ), j = the first element of i's run.  In place
+ * (d_out == d_in) is allowed.  Hand-written counterpart of thrust::inclusive_scan_by_key(keys, keys + n, in, out)
+ * as the reference calls it (src/prefixsum/seg_thrust.cu:46-47).
+ *
+ * tcu_seg_reduce_by_key_f16: for the r-th run, d_out[r] = fp16(sum of the run) and, if d_keys_out is not NULL,
+ * d_keys_out[r] = its key; *d_num_runs (a 64-bit unsigned in device memory, may be NULL) receives the number of
+ * runs, which is what thrust::reduce_by_key(keys, keys + n, in, keys_out, out) returns as the end of its output
+ * (src/reduction/seg_thrust.cu:50-51).  d_out and d_keys_out need room for as many entries as there are runs
+ * (at most n) and must not overlap d_in or d_keys.  A look-back wait that expires (see "lookback_poll_limit")
+ * leaves ~0 in *d_num_runs and NaN in the sums that depended on it. */
+int tcu_seg_scan_by_key_f16(const void *d_keys, const void *d_in, void *d_out, size_t n, int key_bits, void *d_workspace, size_t *workspace_bytes, void *stream);
+int tcu_seg_reduce_by_key_f16(const void *d_keys, const void *d_in, void *d_keys_out, void *d_out, void *d_num_runs, size_t n, int key_bits, void *d_workspace, size_t *workspace_bytes, void *stream);
+
 /* d_out[s*S + i] += d_partial_sums[s]  (one fp16 addition per element).
  * Replaces add_partial_sums (reference src/prefixsum/kernel.cuh:31-43). */
 int tcu_add_partial_sums_f16(void *d_out, const void *d_partial_sums, size_t num_segments, size_t segment_size, void *stream);

@@ -61,6 +61,12 @@ def lib():
         L.tcu_oracle_seg_scan_offsets_ref.argtypes = [u16p, u16p, sz, i64p, i64p]
         L.tcu_oracle_seg_scan_offsets_f64.argtypes = [u16p, f64p, sz, i64p, i64p]
         L.tcu_oracle_seg_scan_f64.argtypes = [u16p, f64p, sz, sz]
+        L.tcu_oracle_seg_scan_by_key_ref.argtypes = [i64p, u16p, u16p, sz]
+        L.tcu_oracle_seg_scan_by_key_f64.argtypes = [i64p, u16p, f64p, sz]
+        L.tcu_oracle_seg_reduce_by_key_ref.restype = sz
+        L.tcu_oracle_seg_reduce_by_key_ref.argtypes = [i64p, u16p, i64p, u16p, sz]
+        L.tcu_oracle_seg_reduce_by_key_f64.restype = sz
+        L.tcu_oracle_seg_reduce_by_key_f64.argtypes = [i64p, u16p, i64p, f64p, sz]
         L.tcu_oracle_gemv_f64.argtypes = [u16p, u16p, f32p, f64p, sz, sz, c.c_double, c.c_double]
         L.tcu_oracle_gemm_f64.argtypes = [u16p, u16p, f32p, f64p, sz, sz, sz, c.c_double, c.c_double, sz, sz]
         L.tcu_oracle_check_f16.restype = sz
@@ -240,6 +246,40 @@ def seg_scan_offsets_f64(x, begin, end):
     out = np.full(x.size, np.nan, dtype=np.float64)
     lib().tcu_oracle_seg_scan_offsets_f64(_p(x, ctypes.c_uint16), _p(out, ctypes.c_double), begin.size, _p(begin, ctypes.c_int64), _p(end, ctypes.c_int64))
     return out
+
+
+def _keys64(keys):
+    return np.ascontiguousarray(keys, dtype=np.int64)
+
+
+def seg_scan_by_key_ref(keys, x):
+    """Inclusive prefix sums inside runs of equal consecutive keys: fp32 running sum, fp16 results (uint16 bit patterns)."""
+    k, x = _keys64(keys), _u16(x)
+    out = np.empty(x.size, dtype=np.uint16)
+    lib().tcu_oracle_seg_scan_by_key_ref(_p(k, ctypes.c_int64), _p(x, ctypes.c_uint16), _p(out, ctypes.c_uint16), x.size)
+    return out
+
+
+def seg_scan_by_key_f64(keys, x):
+    k, x = _keys64(keys), _u16(x)
+    out = np.empty(x.size, dtype=np.float64)
+    lib().tcu_oracle_seg_scan_by_key_f64(_p(k, ctypes.c_int64), _p(x, ctypes.c_uint16), _p(out, ctypes.c_double), x.size)
+    return out
+
+
+def seg_reduce_by_key_ref(keys, x):
+    """(keys of the runs, fp16 bit patterns of their sums): fp32 running sum per run."""
+    k, x = _keys64(keys), _u16(x)
+    ko, out = np.empty(max(x.size, 1), dtype=np.int64), np.empty(max(x.size, 1), dtype=np.uint16)
+    runs = lib().tcu_oracle_seg_reduce_by_key_ref(_p(k, ctypes.c_int64), _p(x, ctypes.c_uint16), _p(ko, ctypes.c_int64), _p(out, ctypes.c_uint16), x.size)
+    return ko[:runs].copy(), out[:runs].copy()
+
+
+def seg_reduce_by_key_f64(keys, x):
+    k, x = _keys64(keys), _u16(x)
+    ko, out = np.empty(max(x.size, 1), dtype=np.int64), np.empty(max(x.size, 1), dtype=np.float64)
+    runs = lib().tcu_oracle_seg_reduce_by_key_f64(_p(k, ctypes.c_int64), _p(x, ctypes.c_uint16), _p(ko, ctypes.c_int64), _p(out, ctypes.c_double), x.size)
+    return ko[:runs].copy(), out[:runs].copy()
 
 
 def seg_scan_f64(x, num_segments, segment_size):

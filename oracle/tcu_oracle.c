@@ -407,3 +407,55 @@ size_t tcu_oracle_check_f32_rel(const float *got, const double *ref, size_t n, d
   if (first_bad) *first_bad = fb;
   return bad;
 }
+
+/* ------------------------------------------------------------------------------------ */
+/* segments given by a key array: a segment is a run of equal consecutive keys            */
+/* ------------------------------------------------------------------------------------ */
+
+void tcu_oracle_seg_scan_by_key_ref(const int64_t *keys, const uint16_t *in, uint16_t *out, size_t n) {
+  float acc = 0.0f;
+  for (size_t i = 0; i < n; i++) {
+    if (i == 0 || keys[i] != keys[i - 1]) acc = 0.0f;
+    acc += tcu_oracle_f16_to_f32(in[i]);
+    out[i] = tcu_oracle_f32_to_f16(acc);
+  }
+}
+
+void tcu_oracle_seg_scan_by_key_f64(const int64_t *keys, const uint16_t *in, double *out, size_t n) {
+  double acc = 0.0;
+  for (size_t i = 0; i < n; i++) {
+    if (i == 0 || keys[i] != keys[i - 1]) acc = 0.0;
+    acc += (double)tcu_oracle_f16_to_f32(in[i]);
+    out[i] = acc;
+  }
+}
+
+size_t tcu_oracle_seg_reduce_by_key_ref(const int64_t *keys, const uint16_t *in, int64_t *keys_out, uint16_t *out, size_t n) {
+  size_t runs = 0;
+  float acc = 0.0f;
+  for (size_t i = 0; i < n; i++) {
+    acc += tcu_oracle_f16_to_f32(in[i]);
+    if (i + 1 == n || keys[i + 1] != keys[i]) {
+      keys_out[runs] = keys[i];
+      out[runs] = tcu_oracle_f32_to_f16(acc);
+      runs++;
+      acc = 0.0f;
+    }
+  }
+  return runs;
+}
+
+size_t tcu_oracle_seg_reduce_by_key_f64(const int64_t *keys, const uint16_t *in, int64_t *keys_out, double *out, size_t n) {
+  size_t runs = 0;
+  double acc = 0.0;
+  for (size_t i = 0; i < n; i++) {
+    acc += (double)tcu_oracle_f16_to_f32(in[i]);
+    if (i + 1 == n || keys[i + 1] != keys[i]) {
+      keys_out[runs] = keys[i];
+      out[runs] = acc;
+      runs++;
+      acc = 0.0;
+    }
+  }
+  return runs;
+}

@@ -103,6 +103,15 @@ void tcu_oracle_seg_scan_offsets_f64(const uint16_t *in, double *out, size_t num
 void tcu_oracle_seg_reduce_offsets_f64(const uint16_t *in, double *out, size_t num_segments, const int64_t *begin, const int64_t *end);
 void tcu_oracle_seg_reduce_f64(const uint16_t *in, double *out, size_t num_segments, size_t segment_size);
 void tcu_oracle_seg_scan_f64(const uint16_t *in, double *out, size_t num_segments, size_t segment_size);
+/* Segments as runs of equal consecutive keys: the semantics of thrust::inclusive_scan_by_key and
+ * thrust::reduce_by_key as the reference calls them (src/prefixsum/seg_thrust.cu:46-47,
+ * src/reduction/seg_thrust.cu:50-51).  _ref: fp32 running sum per run, fp16 results; _f64: the definition.
+ * The reductions return the number of runs and fill keys_out / out with one entry per run. */
+void tcu_oracle_seg_scan_by_key_ref(const int64_t *keys, const uint16_t *in, uint16_t *out, size_t n);
+void tcu_oracle_seg_scan_by_key_f64(const int64_t *keys, const uint16_t *in, double *out, size_t n);
+size_t tcu_oracle_seg_reduce_by_key_ref(const int64_t *keys, const uint16_t *in, int64_t *keys_out, uint16_t *out, size_t n);
+size_t tcu_oracle_seg_reduce_by_key_f64(const int64_t *keys, const uint16_t *in, int64_t *keys_out, double *out, size_t n);
+
 /* y = alpha*A*x + beta*y0; A is M x K row-major fp16, x fp16, y0 may be NULL when beta==0 */
 void tcu_oracle_gemv_f64(const uint16_t *A, const uint16_t *x, const float *y0, double *y, size_t M, size_t K, double alpha, double beta);
 /* D = alpha*A*B + beta*C; A M x K row-major, B K x N column-major (element (k,n) at

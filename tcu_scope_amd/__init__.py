@@ -32,6 +32,8 @@ from .binding import (  # noqa: F401
     seg_scan_offsets,
     seg_scan,
     seg_scan_noalloc,
+    seg_scan_by_key,
+    seg_reduce_by_key,
     set_option,
     stream_probe,
     time_next_launch,

@@ -11,7 +11,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 
 EXPORTS = [
     "tcu_abi_version", "tcu_last_error", "tcu_init", "tcu_device_info", "tcu_set_option",
-    "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_f16_noalloc", "tcu_seg_scan_offsets_f16", "tcu_add_partial_sums_f16",
+    "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_f16_noalloc", "tcu_seg_scan_offsets_f16", "tcu_seg_scan_by_key_f16", "tcu_seg_reduce_by_key_f16", "tcu_add_partial_sums_f16",
     "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32", "tcu_gemv_f16_f16", "tcu_gemm_f16_f16",
     "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_time_next_launch", "tcu_lane_probe",
 ]
@@ -90,6 +90,8 @@ def lib():
         L.tcu_seg_scan_f16.argtypes = [vp, vp, vp, sz, sz, ci, ci, ci, vp]
         L.tcu_seg_scan_f16_noalloc.argtypes = [vp, vp, vp, sz, sz, ci, ci, ci, vp]
         L.tcu_seg_scan_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz, vp]
+        L.tcu_seg_scan_by_key_f16.argtypes = [vp, vp, vp, sz, ci, vp, c.POINTER(sz), vp]
+        L.tcu_seg_reduce_by_key_f16.argtypes = [vp, vp, vp, vp, vp, sz, ci, vp, c.POINTER(sz), vp]
         L.tcu_add_partial_sums_f16.argtypes = [vp, vp, sz, sz, vp]
         L.tcu_full_reduce_f16.argtypes = [vp, vp, sz, vp, c.POINTER(sz), ci, sz, ci, vp]
         L.tcu_full_scan_f16.argtypes = [vp, vp, sz, vp, c.POINTER(sz), ci, sz, ci, vp]
@@ -214,6 +216,53 @@ def seg_scan_offsets(x, begin, end, expected_segment_size=0, out=None, stream=No
     bits = 32 if begin.dtype == torch.int32 else 64
     _check(lib().tcu_seg_scan_offsets_f16(_ptr(x), _ptr(out), begin.numel(), _ptr(begin), _ptr(end), bits, expected_segment_size, _stream(stream)))
     return out
+
+
+def _key_bits(keys):
+    torch = _torch()
+    if keys.dtype not in (torch.int32, torch.int64) or not keys.is_cuda or not keys.is_contiguous():
+        raise ValueError("keys must be a contiguous CUDA int32 or int64 tensor")
+    return 32 if keys.dtype == torch.int32 else 64
+
+
+def seg_scan_by_key(keys, x, out=None, workspace=None, stream=None):
+    """Inclusive prefix sums inside runs of equal consecutive keys (thrust::inclusive_scan_by_key)."""
+    torch = _torch()
+    _need_f16(x, "x")
+    bits = _key_bits(keys)
+    n = x.numel()
+    if keys.numel() != n:
+        raise ValueError("keys and x must have the same length")
+    if out is None:
+        out = torch.empty_like(x)
+    need = ctypes.c_size_t(0)
+    _check(lib().tcu_seg_scan_by_key_f16(None, None, None, n, bits, None, ctypes.byref(need), None))
+    if workspace is None:
+        workspace = torch.empty(max(need.value, 256), dtype=torch.uint8, device=x.device)
+    have = ctypes.c_size_t(workspace.numel())
+    _check(lib().tcu_seg_scan_by_key_f16(_ptr(keys), _ptr(x), _ptr(out), n, bits, _ptr(workspace), ctypes.byref(have), _stream(stream)))
+    return out
+
+
+def seg_reduce_by_key(keys, x, workspace=None, stream=None):
+    """One sum per run of equal consecutive keys (thrust::reduce_by_key): returns (keys_out, sums, num_runs tensor);
+    the first two have room for x.numel() entries, of which the first num_runs.item() are written."""
+    torch = _torch()
+    _need_f16(x, "x")
+    bits = _key_bits(keys)
+    n = x.numel()
+    if keys.numel() != n:
+        raise ValueError("keys and x must have the same length")
+    keys_out = torch.empty_like(keys)
+    out = torch.empty_like(x)
+    num_runs = torch.zeros(1, dtype=torch.int64, device=x.device)
+    need = ctypes.c_size_t(0)
+    _check(lib().tcu_seg_reduce_by_key_f16(None, None, None, None, None, n, bits, None, ctypes.byref(need), None))
+    if workspace is None:
+        workspace = torch.empty(max(need.value, 256), dtype=torch.uint8, device=x.device)
+    have = ctypes.c_size_t(workspace.numel())
+    _check(lib().tcu_seg_reduce_by_key_f16(_ptr(keys), _ptr(x), _ptr(keys_out), _ptr(out), _ptr(num_runs), n, bits, _ptr(workspace), ctypes.byref(have), _stream(stream)))
+    return keys_out, out, num_runs
 
 
 def add_partial_sums(out, partial_sums, segment_size, stream=None):

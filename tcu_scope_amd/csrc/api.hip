@@ -144,6 +144,16 @@ int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments,
   return after_launch("tcu_seg_scan_offsets_f16", before, tcu::seg_scan_offsets_dispatch(d_in, d_out, num_segments, d_begin_offsets, d_end_offsets, offset_bits, expected_segment_size, stream));
 }
 
+int tcu_seg_scan_by_key_f16(const void *d_keys, const void *d_in, void *d_out, size_t n, int key_bits, void *d_workspace, size_t *workspace_bytes, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_seg_scan_by_key_f16", before, tcu::seg_scan_by_key_dispatch(d_keys, d_in, d_out, n, key_bits, d_workspace, workspace_bytes, stream));
+}
+
+int tcu_seg_reduce_by_key_f16(const void *d_keys, const void *d_in, void *d_keys_out, void *d_out, void *d_num_runs, size_t n, int key_bits, void *d_workspace, size_t *workspace_bytes, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_seg_reduce_by_key_f16", before, tcu::seg_reduce_by_key_dispatch(d_keys, d_in, d_keys_out, d_out, d_num_runs, n, key_bits, d_workspace, workspace_bytes, stream));
+}
+
 int tcu_add_partial_sums_f16(void *d_out, const void *d_partial_sums, size_t num_segments, size_t segment_size, void *stream) {
   const unsigned long before = tcu::launch_count();
   return after_launch("tcu_add_partial_sums_f16", before, tcu::add_partial_sums_dispatch(d_out, d_partial_sums, num_segments, segment_size, stream));

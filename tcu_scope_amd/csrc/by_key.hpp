@@ -1,0 +1,355 @@
+// Segments given by a key array: a segment is a run of equal consecutive keys.  Inclusive prefix
+// sums inside every run (the reference's thrust::inclusive_scan_by_key baseline,
+// src/prefixsum/seg_thrust.cu:46-47) and one sum per run (thrust::reduce_by_key,
+// src/reduction/seg_thrust.cu:50-51), fp16 values, fp32 accumulation, one rounding to fp16.
+//
+// One pass over keys and values.  The scan operator on pairs (head flag, value)
+//     (f1, v1) (+) (f2, v2) = (f1 | f2, f2 ? v2 : v1 + v2)
+// is associative, so the whole array is scanned like the full-array prefix sum: a lane scans
+// its 8 elements serially, the 64 chunk summaries of a tile are scanned across the lanes with
+// DPP, tiles are chained in the wave, waves meet in LDS, blocks (partitions of
+// blockDim/64 * U tiles, handed out by a ticket) meet through decoupled look-back on 64-bit
+// descriptors {status + 4 * flag, fp32 value}: a predecessor whose aggregate carries a head
+// flag ends the look-back just as a published prefix does.  The reduction also counts the heads
+// (a second, integer look-back) to know where a run's sum goes, and writes a run's sum at the
+// head of the NEXT run (the value carried up to that head), so no element ever needs its
+// successor's key; the last run is written by the lane that holds the last element.
+//
+// Every wait is bounded (WaitPolicy): a look-back that gives up yields NaN sums (and, for the
+// reduction, counts of 0xffffffff that keep later partitions from writing anything).
+#pragma once
+
+#include "full_array.hpp"
+
+namespace tcu {
+
+constexpr unsigned kKeyStatusAggregate = 1u, kKeyStatusPrefix = 2u, kKeyFlagged = 4u;
+
+// (fl, vl) (+) (f, v) -> (f, v)
+TCU_DEVICE void seg_combine(unsigned fl, float vl, unsigned &f, float &v) {
+  v = f ? v : vl + v;
+  f |= fl;
+}
+
+// exclusive scan of (F, V) over the 64 lanes of a wave under the operator above
+TCU_DEVICE void wave_exclusive_seg_scan(unsigned F, float V, unsigned &Fe, float &Ve) {
+  unsigned f = dpp_u32<DPP_WAVE_SHR1>(0u, F);
+  float v = dpp<DPP_WAVE_SHR1>(0.0f, V);
+  seg_combine(dpp_u32<DPP_ROW_SHR0 + 1>(0u, f), dpp<DPP_ROW_SHR0 + 1>(0.0f, v), f, v);
+  seg_combine(dpp_u32<DPP_ROW_SHR0 + 2>(0u, f), dpp<DPP_ROW_SHR0 + 2>(0.0f, v), f, v);
+  seg_combine(dpp_u32<DPP_ROW_SHR0 + 4>(0u, f), dpp<DPP_ROW_SHR0 + 4>(0.0f, v), f, v);
+  seg_combine(dpp_u32<DPP_ROW_SHR0 + 8>(0u, f), dpp<DPP_ROW_SHR0 + 8>(0.0f, v), f, v);
+  seg_combine(dpp_u32<DPP_ROW_BCAST15, 0xA, 0xF, false>(0u, f), dpp<DPP_ROW_BCAST15, 0xA, 0xF, false>(0.0f, v), f, v);
+  seg_combine(dpp_u32<DPP_ROW_BCAST31, 0xC, 0xF, false>(0u, f), dpp<DPP_ROW_BCAST31, 0xC, 0xF, false>(0.0f, v), f, v);
+  Fe = f;
+  Ve = v;
+}
+// exclusive prefix sum of an unsigned over the 64 lanes
+TCU_DEVICE unsigned wave_exclusive_count(unsigned c) {
+  unsigned e = dpp_u32<DPP_WAVE_SHR1>(0u, c);
+  e += dpp_u32<DPP_ROW_SHR0 + 1>(0u, e);
+  e += dpp_u32<DPP_ROW_SHR0 + 2>(0u, e);
+  e += dpp_u32<DPP_ROW_SHR0 + 4>(0u, e);
+  e += dpp_u32<DPP_ROW_SHR0 + 8>(0u, e);
+  e += dpp_u32<DPP_ROW_BCAST15, 0xA, 0xF, false>(0u, e);
+  e += dpp_u32<DPP_ROW_BCAST31, 0xC, 0xF, false>(0u, e);
+  return e;
+}
+
+// Look-back over descriptors whose high word is status + 4 * flag: the walk ends at the nearest
+// predecessor that has published its inclusive prefix or whose aggregate carries a head flag.
+// Returns the value that precedes partition `part`; NaN when a wait expired.
+TCU_DEVICE float look_back_flagged(const unsigned long long *desc, long long part, int lane, WaitPolicy wait) {
+  float prefix = 0.0f;
+  long long base = part - 1;
+  unsigned polls = 0;
+  while (true) {
+    const long long idx = base - lane;
+    const unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : (unsigned long long)kKeyStatusPrefix << 32;
+    const unsigned hi = (unsigned)(d >> 32);
+    const unsigned long long is_stop = ballot(hi >= kKeyStatusPrefix);
+    const unsigned long long is_empty = ballot(hi == 0u);
+    const int first_stop = is_stop ? __builtin_ctzll(is_stop) : 64;
+    const unsigned long long needed = first_stop >= 63 ? ~0ull : ((2ull << first_stop) - 1ull);
+    if (is_empty & needed) {
+      if (polls++ >= wait.poll_limit) return __builtin_nanf("");
+      spin_pause();
+      continue;
+    }
+    float val = lane <= first_stop ? __uint_as_float((unsigned)d) : 0.0f;
+    val = lane_group_sum<6>(val);
+    prefix += readlane(val, 63);
+    if (first_stop < 64) return prefix;
+    base -= 64;
+  }
+}
+// The same walk over plain {status, count} descriptors (status 1 = aggregate, 2 = inclusive prefix).
+// 0xffffffff when a wait expired.
+TCU_DEVICE unsigned look_back_count(const unsigned long long *desc, long long part, int lane, WaitPolicy wait) {
+  unsigned prefix = 0;
+  long long base = part - 1;
+  unsigned polls = 0;
+  while (true) {
+    const long long idx = base - lane;
+    const unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : (unsigned long long)kKeyStatusPrefix << 32;
+    const unsigned hi = (unsigned)(d >> 32);
+    const unsigned long long is_stop = ballot(hi == kKeyStatusPrefix);
+    const unsigned long long is_empty = ballot(hi == 0u);
+    const int first_stop = is_stop ? __builtin_ctzll(is_stop) : 64;
+    const unsigned long long needed = first_stop >= 63 ? ~0ull : ((2ull << first_stop) - 1ull);
+    if (is_empty & needed) {
+      if (polls++ >= wait.poll_limit) return 0xffffffffu;
+      spin_pause();
+      continue;
+    }
+    unsigned val = lane <= first_stop ? (unsigned)d : 0u;
+    if (ballot(val == 0xffffffffu) != 0ull) return 0xffffffffu;  // a predecessor could not count either
+    val += wave_exclusive_count(val);  // inclusive in lane 63
+    prefix += readlane_u32(val, 63);
+    if (first_stop < 64) return prefix;
+    base -= 64;
+  }
+}
+
+// the key in lane l - 1 (lane 0: undefined, the caller replaces it)
+TCU_DEVICE int32_t key_of_previous_lane(int32_t k) { return (int32_t)dpp_u32<DPP_WAVE_SHR1>(0u, (unsigned)k); }
+TCU_DEVICE int64_t key_of_previous_lane(int64_t k) {
+  const unsigned lo = dpp_u32<DPP_WAVE_SHR1>(0u, (unsigned)(uint64_t)k), hi = dpp_u32<DPP_WAVE_SHR1>(0u, (unsigned)((uint64_t)k >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+TCU_DEVICE int32_t key_of_lane(int32_t k, int l) { return (int32_t)readlane_u32((unsigned)k, l); }
+TCU_DEVICE int64_t key_of_lane(int64_t k, int l) {
+  const unsigned lo = readlane_u32((unsigned)(uint64_t)k, l), hi = readlane_u32((unsigned)((uint64_t)k >> 32), l);
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// What a lane keeps of one chunk (8 elements) between the two passes.
+struct KeyChunk {
+  float p[8];     // inclusive prefix inside the chunk, restarted at every head, without any carry
+  unsigned heads; // bit i: element i starts a run
+  unsigned fe;    // exclusive scan over the tile's lanes: a head lies between the tile start and this chunk
+  float ve;       //   ... and the value carried from the tile start (or from that head) to this chunk
+  unsigned he;    // heads between the tile start and this chunk
+  int valid;      // elements of the chunk inside the array (0 ... 8)
+};
+
+// workspace words: [0] ticket, [64 ...) u64 value descriptors, then (REDUCE) u64 count descriptors
+template <typename KEY, int U, bool REDUCE, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict__ keys, const uint16_t *in, uint16_t *out, KEY *__restrict__ keys_out, unsigned long long *num_runs,
+                                                           size_t n, unsigned *ws, unsigned n_parts, int static_order, WaitPolicy wait) {
+  __shared__ float wave_v[kMaxWaves];
+  __shared__ unsigned wave_f[kMaxWaves], wave_h[kMaxWaves];
+  __shared__ unsigned s_part, s_count;
+  __shared__ float s_prefix;
+  const int lane = lane_id(), wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  unsigned long long *desc_v = reinterpret_cast<unsigned long long *>(ws + 64);
+  unsigned long long *desc_c = desc_v + n_parts;
+
+  if (!static_order) {
+    if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
+    __syncthreads();
+  }
+  const unsigned part = static_order ? blockIdx.x : s_part;
+  const size_t tile0 = ((size_t)part * WPB + wave) * U;
+
+  // ---- pass 1: load, flags, chunk scans, tile scans --------------------------------------
+  KeyChunk ch[U];
+  KEY k7_prev_tile = 0;
+  unsigned wf = 0, wh = 0;  // wave totals under the operator / head count
+  float wv = 0.0f;
+  unsigned tile_f[U], tile_h[U];
+  float tile_v[U];
+#pragma unroll
+  for (int j = 0; j < U; j++) {
+    const size_t e0 = ((tile0 + j) * kTileChunks + lane) * 8;  // first element of this lane's chunk
+    const int valid = e0 >= n ? 0 : (n - e0 >= 8 ? 8 : (int)(n - e0));
+    KEY k[8];
+    float x[8];
+    if (valid == 8) {
+      const half8_t v = load_chunk<NT>(reinterpret_cast<const half8_t *>(in + e0));
+#pragma unroll
+      for (int i = 0; i < 8; i++) x[i] = (float)v[i];
+      if constexpr (sizeof(KEY) == 4) {
+        const uint4_t a = *reinterpret_cast<const uint4_t *>(keys + e0), b = *reinterpret_cast<const uint4_t *>(keys + e0 + 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          k[i] = (KEY)a[i];
+          k[4 + i] = (KEY)b[i];
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const uint4_t a = *reinterpret_cast<const uint4_t *>(keys + e0 + 2 * q);
+          k[2 * q] = (KEY)(((uint64_t)a[1] << 32) | a[0]);
+          k[2 * q + 1] = (KEY)(((uint64_t)a[3] << 32) | a[2]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const bool ok = i < valid;
+        x[i] = ok ? (float)__builtin_bit_cast(half_t, in[e0 + i]) : 0.0f;
+        k[i] = ok ? keys[e0 + i] : (KEY)0;
+      }
+    }
+    // the key before the chunk: the previous lane's last key; lane 0 takes it from the wave's previous tile or from memory
+    KEY pk = key_of_previous_lane(k[7]);
+    if (lane == 0) {
+      if (j > 0)
+        pk = k7_prev_tile;
+      else if (e0 > 0 && e0 < n)
+        pk = keys[e0 - 1];
+    }
+    k7_prev_tile = key_of_lane(k[7], 63);
+    unsigned heads = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const KEY before = i ? k[i - 1] : pk;
+      if (i < valid && (k[i] != before || e0 + i == 0)) heads |= 1u << i;
+    }
+    float run = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      run = ((heads >> i) & 1u) ? x[i] : run + x[i];
+      ch[j].p[i] = run;
+    }
+    ch[j].heads = heads;
+    ch[j].valid = valid;
+    // chunk summary, its exclusive scan over the lanes, and the tile's summary (lane 63's inclusive value)
+    const unsigned F = heads ? 1u : 0u;
+    wave_exclusive_seg_scan(F, run, ch[j].fe, ch[j].ve);
+    unsigned fi = F;
+    float vi = run;
+    seg_combine(ch[j].fe, ch[j].ve, fi, vi);
+    unsigned tf = readlane_u32(fi, 63);
+    float tv = readlane(vi, 63);
+    unsigned th = 0;
+    ch[j].he = 0;
+    if constexpr (REDUCE) {
+      const unsigned hc = (unsigned)__builtin_popcount(heads);
+      ch[j].he = wave_exclusive_count(hc);
+      th = readlane_u32(ch[j].he + hc, 63);
+    }
+    // what the wave's earlier tiles carry into this one, then the wave's running summary with this tile
+    tile_f[j] = wf;
+    tile_v[j] = wv;
+    tile_h[j] = wh;
+    seg_combine(wf, wv, tf, tv);
+    wf = tf;
+    wv = tv;
+    wh += th;
+  }
+  if (lane == 0) {
+    wave_f[wave] = wf;
+    wave_v[wave] = wv;
+    wave_h[wave] = wh;
+  }
+  __syncthreads();
+
+  // ---- the block's aggregate, look-back, inclusive prefix ------------------------------------
+  if (wave == 0) {
+    unsigned af = 0, ah = 0;
+    float av = 0.0f;
+    for (int w = 0; w < WPB; w++) {
+      unsigned f = wave_f[w];
+      float v = wave_v[w];
+      seg_combine(af, av, f, v);
+      af = f;
+      av = v;
+      ah += wave_h[w];
+    }
+    const bool muted = part + 1 == wait.mute_partition;
+    float prefix = 0.0f;
+    unsigned count = 0;
+    if (part == 0) {
+      if (lane == 0 && !muted) {
+        atomic_store_u64(desc_v, ((unsigned long long)kKeyStatusPrefix << 32) | __float_as_uint(av));
+        if constexpr (REDUCE) atomic_store_u64(desc_c, ((unsigned long long)kKeyStatusPrefix << 32) | ah);
+      }
+    } else {
+      if (lane == 0 && !muted) {
+        atomic_store_u64(desc_v + part, ((unsigned long long)(kKeyStatusAggregate + (af ? kKeyFlagged : 0u)) << 32) | __float_as_uint(av));
+        if constexpr (REDUCE) atomic_store_u64(desc_c + part, ((unsigned long long)kKeyStatusAggregate << 32) | ah);
+      }
+      prefix = look_back_flagged(desc_v, (long long)part, lane, wait);
+      if constexpr (REDUCE) count = look_back_count(desc_c, (long long)part, lane, wait);
+      if (lane == 0 && !muted) {
+        atomic_store_u64(desc_v + part, ((unsigned long long)kKeyStatusPrefix << 32) | __float_as_uint(af ? av : prefix + av));
+        // a count that could not be had stays "unknown" for every later partition
+        if constexpr (REDUCE) atomic_store_u64(desc_c + part, ((unsigned long long)kKeyStatusPrefix << 32) | (count == 0xffffffffu ? count : count + ah));
+      }
+    }
+    if (lane == 0) {
+      s_prefix = prefix;
+      s_count = count;
+    }
+  }
+  __syncthreads();
+
+  // ---- pass 2: carries in, results out -----------------------------------------------------------
+  unsigned cf = 0;
+  float cv = s_prefix;
+  unsigned chd = s_count;
+  const bool count_known = chd != 0xffffffffu;
+  for (int w = 0; w < wave; w++) {
+    unsigned f = wave_f[w];
+    float v = wave_v[w];
+    seg_combine(cf, cv, f, v);
+    cf = f;
+    cv = v;
+    chd += wave_h[w];
+  }
+#pragma unroll
+  for (int j = 0; j < U; j++) {
+    // what precedes the tile: (block prefix, previous waves) (+) (this wave's tiles before j)
+    unsigned tf = tile_f[j];
+    float tv = tile_v[j];
+    seg_combine(cf, cv, tf, tv);
+    // what precedes this lane's chunk
+    unsigned lf = ch[j].fe;
+    float lv = ch[j].ve;
+    seg_combine(tf, tv, lf, lv);
+    const float carry = lv;
+    const size_t e0 = ((tile0 + j) * kTileChunks + lane) * 8;
+    const unsigned heads = ch[j].heads;
+    const int valid = ch[j].valid;
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) r[i] = (heads & ((2u << i) - 1u)) ? ch[j].p[i] : carry + ch[j].p[i];
+    if constexpr (!REDUCE) {
+      if (valid == 8) {
+        const uint4_t packed = {pack_f16x2(r[0], r[1]), pack_f16x2(r[2], r[3]), pack_f16x2(r[4], r[5]), pack_f16x2(r[6], r[7])};
+        store_chunk<NT>(reinterpret_cast<uint4_t *>(out + e0), packed);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+          if (i < valid) out[e0 + i] = f16_bits(r[i]);
+      }
+    } else {
+      if (count_known) {
+        const unsigned hb = chd + tile_h[j] + ch[j].he;  // runs started before this chunk
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          if ((heads >> i) & 1u) {
+            const unsigned idx = hb + (unsigned)__builtin_popcount(heads & ((1u << i) - 1u));  // runs started before element i
+            if (idx > 0) {  // the run that ends at element i - 1
+              out[idx - 1] = f16_bits(i ? r[i - 1] : carry);
+              if (keys_out) keys_out[idx - 1] = keys[e0 + i - 1];  // idx > 0: element 0 is not meant, the read stays inside the array
+            }
+          }
+        }
+        if (valid > 0 && e0 + (size_t)valid == n) {  // the lane that holds the last element closes the last run
+          const unsigned runs = hb + (unsigned)__builtin_popcount(heads);
+          out[runs - 1] = f16_bits(r[valid - 1]);
+          if (keys_out) keys_out[runs - 1] = keys[n - 1];
+          if (num_runs) *num_runs = runs;
+        }
+      } else if (valid > 0 && e0 + (size_t)valid == n && num_runs) {
+        *num_runs = ~0ull;  // a wait expired: the number of runs is unknown
+      }
+    }
+  }
+}
+
+}  // namespace tcu

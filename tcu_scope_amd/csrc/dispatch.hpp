@@ -16,6 +16,7 @@
 #include "seg_reduce.hpp"
 #include "seg_scan.hpp"
 #include "full_array.hpp"
+#include "by_key.hpp"
 #include "gemv.hpp"
 #include "gemm.hpp"
 #include "util_kernels.hpp"
@@ -793,6 +794,64 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
   if (int rc = seg_scan_dispatch(d_in, d_out, d_ws, nseg, S, TCU_VARIANT_MFMA_256N, 0, waves_per_block, stream)) return rc;
   launch(exclusive_scan_f16_kernel, 1u, 1024u, stream, static_cast<uint16_t *>(d_ws), nseg);
   return add_partial_sums_dispatch(d_out, d_ws, nseg, S, stream);
+}
+
+// ----- segments given by a key array ---------------------------------------------------------------
+
+constexpr int kByKeyTiles = 4, kByKeyWaves = 16;                                   // per wave / per block
+constexpr size_t kByKeyPartition = (size_t)kByKeyTiles * kByKeyWaves * kTileHalves;  // elements per block
+
+template <typename KEY>
+inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const void *d_in, void *d_keys_out, void *d_out, void *d_num_runs, size_t n, void *d_ws, size_t *ws_bytes, void *stream) {
+  if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
+  if (n >= ((size_t)1 << 32)) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": at most 2^32 - 1 elements (runs are counted in 32 bits)");
+  const size_t parts = (n + kByKeyPartition - 1) / kByKeyPartition;
+  const size_t words = 64 + 2 * (parts ? parts : 1) * (reduce ? 2 : 1);
+  const size_t need = round_up(4 * words, kWorkspaceAlign);
+  if (!d_ws) {
+    *ws_bytes = need;
+    return TCU_OK;
+  }
+  if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
+  if (n == 0) {
+    if (reduce && d_num_runs) launch(zero_words_kernel, 1u, 256u, stream, static_cast<unsigned *>(d_num_runs), (size_t)2);
+    return TCU_OK;
+  }
+  if (!d_keys || !d_in || !d_out) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  if (!aligned16(d_keys) || !aligned16(d_in) || (!reduce && !aligned16(d_out))) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": keys, values and the scan's output must be 16-byte aligned");
+  if ((reinterpret_cast<uintptr_t>(d_out) & 1u) || (reinterpret_cast<uintptr_t>(d_keys_out) & (sizeof(KEY) - 1)) || (reinterpret_cast<uintptr_t>(d_num_runs) & 7u))
+    return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": misaligned output pointer");
+  unsigned *ws = static_cast<unsigned *>(d_ws);
+  launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
+  const int so = options().static_order ? 1 : 0;
+  const unsigned grid = (unsigned)parts, block = (unsigned)kByKeyWaves * 64u;
+  const KEY *keys = static_cast<const KEY *>(d_keys);
+  const uint16_t *in = static_cast<const uint16_t *>(d_in);
+  uint16_t *out = static_cast<uint16_t *>(d_out);
+  KEY *keys_out = static_cast<KEY *>(d_keys_out);
+  unsigned long long *num_runs = static_cast<unsigned long long *>(d_num_runs);
+  const bool nt = options().nontemporal;
+  if (reduce) {
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, true, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
+    else launch(by_key_kernel<KEY, kByKeyTiles, true, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
+  } else {
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, false, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
+    else launch(by_key_kernel<KEY, kByKeyTiles, false, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
+  }
+  return TCU_OK;
+}
+
+inline int seg_scan_by_key_dispatch(const void *d_keys, const void *d_in, void *d_out, size_t n, int key_bits, void *d_ws, size_t *ws_bytes, void *stream) {
+  const char *what = "tcu_seg_scan_by_key_f16";
+  if (key_bits == 32) return by_key_typed<int32_t>(what, false, d_keys, d_in, nullptr, d_out, nullptr, n, d_ws, ws_bytes, stream);
+  if (key_bits == 64) return by_key_typed<int64_t>(what, false, d_keys, d_in, nullptr, d_out, nullptr, n, d_ws, ws_bytes, stream);
+  return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": key_bits must be 32 or 64");
+}
+inline int seg_reduce_by_key_dispatch(const void *d_keys, const void *d_in, void *d_keys_out, void *d_out, void *d_num_runs, size_t n, int key_bits, void *d_ws, size_t *ws_bytes, void *stream) {
+  const char *what = "tcu_seg_reduce_by_key_f16";
+  if (key_bits == 32) return by_key_typed<int32_t>(what, true, d_keys, d_in, d_keys_out, d_out, d_num_runs, n, d_ws, ws_bytes, stream);
+  if (key_bits == 64) return by_key_typed<int64_t>(what, true, d_keys, d_in, d_keys_out, d_out, d_num_runs, n, d_ws, ws_bytes, stream);
+  return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": key_bits must be 32 or 64");
 }
 
 // ----- GEMV / GEMM -----------------------------------------------------------------------------

@@ -30,6 +30,12 @@ int emu_gemm_f16_f16(const void *A, const void *B, const void *C, void *D, size_
 int emu_gemm_f16_f32(const void *A, const void *B, const void *C, void *D, size_t M, size_t N, size_t K, float alpha, float beta, int variant) {
   return tcu::gemm_dispatch(A, B, C, D, M, N, K, alpha, beta, variant, nullptr);
 }
+int emu_seg_scan_by_key_f16(const void *keys, const void *in, void *out, size_t n, int bits, void *ws, size_t *ws_bytes) {
+  return tcu::seg_scan_by_key_dispatch(keys, in, out, n, bits, ws, ws_bytes, nullptr);
+}
+int emu_seg_reduce_by_key_f16(const void *keys, const void *in, void *keys_out, void *out, void *num_runs, size_t n, int bits, void *ws, size_t *ws_bytes) {
+  return tcu::seg_reduce_by_key_dispatch(keys, in, keys_out, out, num_runs, n, bits, ws, ws_bytes, nullptr);
+}
 int emu_fill_f16(void *d, float v, size_t n) { return tcu::fill_dispatch(d, v, n, nullptr); }
 int emu_convert_f32_to_f16(void *o, const void *i, size_t n) { return tcu::convert_dispatch(o, i, n, nullptr); }
 int emu_generate_f16(void *d, size_t n, uint64_t seed, int dist, size_t first) { return tcu::generate_dispatch(d, n, seed, dist, first, nullptr); }

@@ -360,3 +360,57 @@ def test_gemv_gemm_and_generator(emu, oracle):
     finally:
         for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1), (b"compute_units", 256), (b"gemm_split_tail", 1)):
             emu.emu_set_option(name, val)
+
+
+def run_keys(rng, n, mean_run):
+    """Keys whose runs have geometric lengths around mean_run; equal keys may come back in later runs."""
+    heads = rng.random(n) < 1.0 / mean_run
+    ids = np.cumsum(heads)
+    return (ids * 7919) % 1013 - 500 + (ids % 2) * (1 << 40)  # neighbours always differ; values need 64 bits
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_segments_given_by_keys(emu, oracle, bits):
+    sz = ctypes.c_size_t
+    emu.emu_seg_scan_by_key_f16.argtypes = [ctypes.c_void_p] * 3 + [sz, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(sz)]
+    emu.emu_seg_reduce_by_key_f16.argtypes = [ctypes.c_void_p] * 5 + [sz, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(sz)]
+    kt = np.int32 if bits == 32 else np.int64
+    rng = np.random.default_rng(bits)
+    part = 4 * 16 * 512
+    for n, mean_run in ((1, 1), (7, 2), (513, 1), (part - 3, 40), (part + 1, 5000), (3 * part + 77, 3), (3 * part + 77, 300), (2 * part, 10 ** 9)):
+        keys = run_keys(rng, n, mean_run)
+        if bits == 32:
+            keys = keys % (1 << 20)
+        keys = keys.astype(kt)
+        x = oracle.generate_f16(n, 5 + n, oracle.DIST_GRID)
+        want_scan = oracle.seg_scan_by_key_f64(keys, x).astype(np.float16).view(np.uint16)
+        want_keys, want_sums = oracle.seg_reduce_by_key_f64(keys, x)
+        want_sums = want_sums.astype(np.float16).view(np.uint16)
+        for static_order in (0, 1):
+            emu.emu_set_option(b"static_order", static_order)
+            d_keys, d_x = copy_in(keys, kt), copy_in(x)
+            need = sz(0)
+            assert emu.emu_seg_scan_by_key_f16(None, None, None, n, bits, None, ctypes.byref(need)) == 0
+            ws = aligned(need.value, np.uint8, 0xAB)
+            out = aligned(n, np.uint16, 0xFFFF)
+            assert emu.emu_seg_scan_by_key_f16(d_keys.ctypes.data, d_x.ctypes.data, out.ctypes.data, n, bits, ws.ctypes.data, ctypes.byref(need)) == 0, emu.emu_last_error()
+            assert np.array_equal(out, want_scan), (n, mean_run, static_order)
+            # in place
+            assert emu.emu_seg_scan_by_key_f16(d_keys.ctypes.data, d_x.ctypes.data, d_x.ctypes.data, n, bits, ws.ctypes.data, ctypes.byref(need)) == 0
+            assert np.array_equal(d_x[:n], want_scan)
+            d_x = copy_in(x)
+            assert emu.emu_seg_reduce_by_key_f16(None, None, None, None, None, n, bits, None, ctypes.byref(need)) == 0
+            ws = aligned(need.value, np.uint8, 0xCD)
+            sums, keys_out, runs = aligned(n, np.uint16, 0xFFFF), aligned(n, kt, -1), aligned(1, np.uint64, 99)
+            assert emu.emu_seg_reduce_by_key_f16(d_keys.ctypes.data, d_x.ctypes.data, keys_out.ctypes.data, sums.ctypes.data, runs.ctypes.data, n, bits, ws.ctypes.data, ctypes.byref(need)) == 0, emu.emu_last_error()
+            r = int(runs[0])
+            assert r == want_keys.size, (n, mean_run)
+            assert np.array_equal(sums[:r], want_sums) and np.array_equal(keys_out[:r], want_keys.astype(kt))
+            assert np.all(sums[r:] == 0xFFFF)  # nothing written past the runs
+    emu.emu_set_option(b"static_order", 0)
+    # empty input: no launch needed, the run count is cleared
+    need, runs = sz(1 << 20), aligned(1, np.uint64, 99)
+    ws = aligned(1 << 12, np.uint8)
+    assert emu.emu_seg_reduce_by_key_f16(None, None, None, None, runs.ctypes.data, 0, bits, ws.ctypes.data, ctypes.byref(need)) == 0
+    assert runs[0] == 0
+    assert emu.emu_seg_scan_by_key_f16(None, None, None, 8, 48, ws.ctypes.data, ctypes.byref(need)) == 1  # key width

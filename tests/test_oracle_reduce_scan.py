@@ -226,3 +226,56 @@ def test_offsets_scan_against_numpy_and_the_fixed_size_oracle(oracle):
     b = np.arange(nseg) * seg
     assert np.array_equal(oracle.seg_scan_offsets_f64(x, b, b + seg)[:nseg * seg], oracle.seg_scan_f64(x, nseg, seg))
     assert np.array_equal(oracle.seg_scan_offsets_ref(x, b, b + seg)[:nseg * seg], oracle.seg_scan_ref(x, nseg, seg))
+
+
+def test_by_key_against_numpy_and_the_offsets_oracle(oracle):
+    """Segments as runs of equal consecutive keys, pinned by: numpy's run boundaries (np.flatnonzero of key changes)
+    with np.add.reduceat / per-run cumsum in float64, a sequential float32 loop for the fp16 path, the offsets
+    functions on the same boundaries, a key that comes back later (two runs, not one), and the two extremes
+    (all keys equal = full-array result, all keys distinct = identity)."""
+    rng = np.random.default_rng(11)
+    n = 25000
+    x = oracle.generate_f16(n, 9, oracle.DIST_UNIFORM)
+    xf = x.view(np.float16)
+    lengths = rng.integers(1, 300, 400)
+    lengths = lengths[np.cumsum(lengths) <= n]
+    lengths[-1] += n - lengths.sum()
+    run_key = rng.integers(-5, 5, lengths.size) * (1 << 33)
+    for i in range(1, run_key.size):  # neighbours differ, repeats further apart stay
+        if run_key[i] == run_key[i - 1]:
+            run_key[i] += 1
+    keys = np.repeat(run_key, lengths)
+    starts = np.flatnonzero(np.r_[True, keys[1:] != keys[:-1]])
+    assert np.array_equal(starts, np.r_[0, np.cumsum(lengths)[:-1]])
+    ends = np.r_[starts[1:], n]
+
+    ko, sums = oracle.seg_reduce_by_key_f64(keys, x)
+    assert np.array_equal(ko, run_key)
+    np.testing.assert_allclose(sums, np.add.reduceat(xf.astype(np.float64), starts), rtol=0, atol=1e-9)
+    assert np.array_equal(sums, oracle.seg_reduce_offsets_f64(x, starts, ends))
+    ko16, sums16 = oracle.seg_reduce_by_key_ref(keys, x)
+    assert np.array_equal(ko16, run_key) and np.array_equal(sums16, oracle.seg_reduce_offsets_ref(x, starts, ends))
+
+    sc = oracle.seg_scan_by_key_f64(keys, x)
+    sc16 = oracle.seg_scan_by_key_ref(keys, x)
+    for b, e in zip(starts[:60], ends[:60]):
+        assert np.allclose(sc[b:e], np.cumsum(xf[b:e].astype(np.float64)), rtol=0, atol=1e-9)
+        acc, want = np.float32(0), []
+        for v in xf[b:e]:
+            acc = np.float32(acc + np.float32(v))
+            want.append(np.float16(acc))
+        assert np.array_equal(sc16[b:e], np.array(want, np.float16).view(np.uint16))
+    assert np.array_equal(sc, oracle.seg_scan_offsets_f64(x, starts, ends))
+    assert np.array_equal(sc16, oracle.seg_scan_offsets_ref(x, starts, ends))
+    assert np.array_equal(sc[ends - 1], sums)
+
+    same = np.zeros(n, np.int64)
+    assert np.array_equal(oracle.seg_scan_by_key_f64(same, x), oracle.seg_scan_f64(x, 1, n))
+    k1, s1 = oracle.seg_reduce_by_key_f64(same, x)
+    assert k1.tolist() == [0] and s1[0] == oracle.seg_reduce_f64(x, 1, n)[0]
+    distinct = np.arange(n)[::-1].copy()
+    assert np.array_equal(oracle.seg_scan_by_key_ref(distinct, x), x)
+    k2, s2 = oracle.seg_reduce_by_key_ref(distinct, x)
+    assert np.array_equal(k2, distinct) and np.array_equal(s2, x)
+    k3, s3 = oracle.seg_reduce_by_key_f64(np.array([], np.int64), np.array([], np.uint16))
+    assert k3.size == 0 and s3.size == 0
