@@ -19,7 +19,7 @@
  *     some in stream order from a memory pool the library keeps per device (it is given back
  *     to the pool when the enqueued work has run, and the pool keeps it for the next call):
  *     tcu_seg_reduce_f16 with segments of 2^20 halves and more and tcu_seg_scan_f16 from 2^21
- *     (4 or 8 bytes per 65536 input halves), the *_offsets_f16 entry points with expected
+ *     (4 or 256 bytes per 65536 input halves), the *_offsets_f16 entry points with expected
  *     segment lengths of 2^17 and more (4 bytes per 65536 halves), and tcu_gemm_* when the
  *     last round of output tiles is sparsely filled (up to 128 MiB).  The full-array entry
  *     points work in the caller's workspace; tcu_seg_scan_f16_noalloc never allocates.
@@ -167,12 +167,14 @@ int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_s
  * capture, serving loops, harnesses that forbid hipMalloc): same arguments, same kernels, same
  * results, but the partition descriptors of the look-back path (TCU_VARIANT_AUTO with segments of
  * 2^21 halves and more, the only path of tcu_seg_scan_f16 that takes temporary memory) live in a
- * 512.25 KiB array that is part of the library's device code, so this entry point never calls
- * an allocating routine.  Limit: num_segments * segment_size <= 2^32 halves on that path (65536
+ * 1 MiB + 256 B array that is part of the library's device code, so this entry point never calls
+ * an allocating routine.  Limit: num_segments * segment_size <= 2^33 halves on that path (131072
  * partitions of 65536 halves; larger calls return TCU_ERR_UNSUPPORTED).  Each GPU holds one such
  * array: calls of this entry point that overlap in time on one GPU (different streams or
  * threads) race on it and must be serialised by the caller; calls on the same stream are fine.
- * The array is cleared by a kernel at the start of every call.  No counterpart in the reference,
+ * The descriptors are spaced 256 bytes apart while the call has at most 4096 partitions (2^28 halves) and
+ * closer beyond that, which costs a few per cent of speed.  The array is cleared by a kernel at the start of
+ * every call.  No counterpart in the reference,
  * whose kernels take no temporary memory. */
 int tcu_seg_scan_f16_noalloc(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
 
@@ -186,8 +188,8 @@ int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments,
 
 /* Segments given by a key array: a segment is a run of equal consecutive keys (d_keys: n signed integers of
  * key_bits = 32 or 64 bits in device memory; n < 2^32).  d_keys, d_in and the scan's d_out must be 16-byte
- * aligned.  Workspace: the two-phase protocol of the full-array entry points below (8 or 16 bytes per 32768
- * elements).  One pass over keys and values (decoupled look-back on (head flag, value) pairs).
+ * aligned.  Workspace: the two-phase protocol of the full-array entry points below (256 bytes per 32768
+ * elements + 256).  One pass over keys and values (decoupled look-back on (head flag, value) pairs).
  *
  * tcu_seg_scan_by_key_f16: d_out[i] = fp16( sum of d_in[j .. i] ), j = the first element of i's run.  In place
  * (d_out == d_in) is allowed.  Hand-written counterpart of thrust::inclusive_scan_by_key(keys, keys + n, in, out)

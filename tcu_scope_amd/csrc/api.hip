@@ -8,10 +8,11 @@
 #include "dispatch.hpp"
 
 // Partition descriptors of tcu_seg_scan_f16_noalloc: a ticket counter (64 words) and one 64-bit
-// descriptor for each of at most 65536 partitions of 65536 halves.  Every device the library's
+// descriptor for each partition of 65536 halves: 256 bytes apart for up to 4096 partitions, closer
+// together for more, 131072 partitions at most.  Every device the library's
 // code is loaded on holds its own copy of the array, at its own address, until the process ends;
 // `scratch` itself is only the host-side handle of the symbol, never a device address.
-constexpr size_t kScratchMaxPartitions = 65536;
+constexpr size_t kScratchMaxPartitions = 131072;
 constexpr size_t kScratchWords = 64 + 2 * kScratchMaxPartitions;
 static __device__ __align__(256) unsigned scratch[kScratchWords];
 

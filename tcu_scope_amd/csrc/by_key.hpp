@@ -65,7 +65,7 @@ TCU_DEVICE float look_back_flagged(const unsigned long long *desc, long long par
   unsigned polls = 0;
   while (true) {
     const long long idx = base - lane;
-    const unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : (unsigned long long)kKeyStatusPrefix << 32;
+    const unsigned long long d = idx >= 0 ? atomic_load_u64(desc + ((size_t)idx << wait.desc_shift)) : (unsigned long long)kKeyStatusPrefix << 32;
     const unsigned hi = (unsigned)(d >> 32);
     const unsigned long long is_stop = ballot(hi >= kKeyStatusPrefix);
     const unsigned long long is_empty = ballot(hi == 0u);
@@ -83,32 +83,69 @@ TCU_DEVICE float look_back_flagged(const unsigned long long *desc, long long par
     base -= 64;
   }
 }
-// The same walk over plain {status, count} descriptors (status 1 = aggregate, 2 = inclusive prefix).
-// 0xffffffff when a wait expired.
-TCU_DEVICE unsigned look_back_count(const unsigned long long *desc, long long part, int lane, WaitPolicy wait) {
-  unsigned prefix = 0;
-  long long base = part - 1;
+// Both walks of the reduction in one loop, so that their polls travel together: the value walk as above, and
+// the same walk over the {status, count} descriptors that follow the value descriptors in every slot (status
+// 1 = aggregate, 2 = inclusive prefix; it ends at a published prefix only).  *count = 0xffffffff when a wait
+// expired or a predecessor could not count either; the value is then NaN.
+TCU_DEVICE void look_back_value_and_count(const unsigned long long *desc, long long part, int lane, WaitPolicy wait, float *value, unsigned *count) {
+  float pv = 0.0f;
+  unsigned pc = 0;
+  long long base_v = part - 1, base_c = part - 1;
+  bool v_done = false, c_done = false;
   unsigned polls = 0;
-  while (true) {
-    const long long idx = base - lane;
-    const unsigned long long d = idx >= 0 ? atomic_load_u64(desc + idx) : (unsigned long long)kKeyStatusPrefix << 32;
-    const unsigned hi = (unsigned)(d >> 32);
-    const unsigned long long is_stop = ballot(hi == kKeyStatusPrefix);
-    const unsigned long long is_empty = ballot(hi == 0u);
-    const int first_stop = is_stop ? __builtin_ctzll(is_stop) : 64;
-    const unsigned long long needed = first_stop >= 63 ? ~0ull : ((2ull << first_stop) - 1ull);
-    if (is_empty & needed) {
-      if (polls++ >= wait.poll_limit) return 0xffffffffu;
-      spin_pause();
-      continue;
+  const unsigned long long at_start = (unsigned long long)kKeyStatusPrefix << 32;
+  while (!v_done || !c_done) {
+    const long long iv = base_v - lane, ic = base_c - lane;
+    unsigned long long dv = at_start, dc = at_start;
+    if (!v_done && iv >= 0) dv = atomic_load_u64(desc + ((size_t)iv << wait.desc_shift));
+    if (!c_done && ic >= 0) dc = atomic_load_u64(desc + ((size_t)ic << wait.desc_shift) + 1);
+    bool waiting = false;
+    if (!v_done) {
+      const unsigned hi = (unsigned)(dv >> 32);
+      const unsigned long long is_stop = ballot(hi >= kKeyStatusPrefix), is_empty = ballot(hi == 0u);
+      const int first_stop = is_stop ? __builtin_ctzll(is_stop) : 64;
+      const unsigned long long needed = first_stop >= 63 ? ~0ull : ((2ull << first_stop) - 1ull);
+      if (is_empty & needed) {
+        waiting = true;
+      } else {
+        float val = lane <= first_stop ? __uint_as_float((unsigned)dv) : 0.0f;
+        val = lane_group_sum<6>(val);
+        pv += readlane(val, 63);
+        if (first_stop < 64) v_done = true;
+        else base_v -= 64;
+      }
     }
-    unsigned val = lane <= first_stop ? (unsigned)d : 0u;
-    if (ballot(val == 0xffffffffu) != 0ull) return 0xffffffffu;  // a predecessor could not count either
-    val += wave_exclusive_count(val);  // inclusive in lane 63
-    prefix += readlane_u32(val, 63);
-    if (first_stop < 64) return prefix;
-    base -= 64;
+    if (!c_done) {
+      const unsigned hi = (unsigned)(dc >> 32);
+      const unsigned long long is_stop = ballot(hi == kKeyStatusPrefix), is_empty = ballot(hi == 0u);
+      const int first_stop = is_stop ? __builtin_ctzll(is_stop) : 64;
+      const unsigned long long needed = first_stop >= 63 ? ~0ull : ((2ull << first_stop) - 1ull);
+      if (is_empty & needed) {
+        waiting = true;
+      } else {
+        unsigned val = lane <= first_stop ? (unsigned)dc : 0u;
+        if (ballot(val == 0xffffffffu) != 0ull) {  // a predecessor could not count
+          pc = 0xffffffffu;
+          c_done = true;
+        } else {
+          val += wave_exclusive_count(val);  // inclusive in lane 63
+          pc += readlane_u32(val, 63);
+          if (first_stop < 64) c_done = true;
+          else base_c -= 64;
+        }
+      }
+    }
+    if (waiting) {
+      if (polls++ >= wait.poll_limit) {
+        *value = __builtin_nanf("");
+        *count = 0xffffffffu;
+        return;
+      }
+      spin_pause();
+    }
   }
+  *value = pv;
+  *count = pc;
 }
 
 // the key in lane l - 1 (lane 0: undefined, the caller replaces it)
@@ -123,17 +160,17 @@ TCU_DEVICE int64_t key_of_lane(int64_t k, int l) {
   return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-// What a lane keeps of one chunk (8 elements) between the two passes.
+// What a lane keeps of one chunk (8 elements) between the two passes: 7 registers, so that a wave can hold
+// many tiles; the prefix sums inside the chunk are taken again from the raw values in the second pass.
 struct KeyChunk {
-  float p[8];     // inclusive prefix inside the chunk, restarted at every head, without any carry
+  half8_t raw;    // the values (zero beyond the end of the array)
   unsigned heads; // bit i: element i starts a run
   unsigned fe;    // exclusive scan over the tile's lanes: a head lies between the tile start and this chunk
   float ve;       //   ... and the value carried from the tile start (or from that head) to this chunk
-  unsigned he;    // heads between the tile start and this chunk
-  int valid;      // elements of the chunk inside the array (0 ... 8)
+  unsigned he;    // heads between the tile start and this chunk (reduction only)
 };
 
-// workspace words: [0] ticket, [64 ...) u64 value descriptors, then (REDUCE) u64 count descriptors
+// workspace words: [0] ticket, [64 ...) per partition a u64 value descriptor followed by a u64 count descriptor
 template <typename KEY, int U, bool REDUCE, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict__ keys, const uint16_t *in, uint16_t *out, KEY *__restrict__ keys_out, unsigned long long *num_runs,
                                                            size_t n, unsigned *ws, unsigned n_parts, int static_order, WaitPolicy wait) {
@@ -143,8 +180,9 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
   __shared__ float s_prefix;
   const int lane = lane_id(), wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
+  // a partition's two descriptors (value, head count) are neighbours; partitions are 8 << wait.desc_shift bytes apart
   unsigned long long *desc_v = reinterpret_cast<unsigned long long *>(ws + 64);
-  unsigned long long *desc_c = desc_v + n_parts;
+  unsigned long long *desc_c = desc_v + 1;
 
   if (!static_order) {
     if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
@@ -165,11 +203,9 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
     const size_t e0 = ((tile0 + j) * kTileChunks + lane) * 8;  // first element of this lane's chunk
     const int valid = e0 >= n ? 0 : (n - e0 >= 8 ? 8 : (int)(n - e0));
     KEY k[8];
-    float x[8];
+    half8_t v;
     if (valid == 8) {
-      const half8_t v = load_chunk<NT>(reinterpret_cast<const half8_t *>(in + e0));
-#pragma unroll
-      for (int i = 0; i < 8; i++) x[i] = (float)v[i];
+      v = load_chunk<NT>(reinterpret_cast<const half8_t *>(in + e0));
       if constexpr (sizeof(KEY) == 4) {
         const uint4_t a = *reinterpret_cast<const uint4_t *>(keys + e0), b = *reinterpret_cast<const uint4_t *>(keys + e0 + 4);
 #pragma unroll
@@ -189,7 +225,7 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         const bool ok = i < valid;
-        x[i] = ok ? (float)__builtin_bit_cast(half_t, in[e0 + i]) : 0.0f;
+        v[i] = ok ? __builtin_bit_cast(half_t, in[e0 + i]) : (half_t)0.0f;
         k[i] = ok ? keys[e0 + i] : (KEY)0;
       }
     }
@@ -210,12 +246,9 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
     }
     float run = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      run = ((heads >> i) & 1u) ? x[i] : run + x[i];
-      ch[j].p[i] = run;
-    }
+    for (int i = 0; i < 8; i++) run = ((heads >> i) & 1u) ? (float)v[i] : run + (float)v[i];
+    ch[j].raw = v;
     ch[j].heads = heads;
-    ch[j].valid = valid;
     // chunk summary, its exclusive scan over the lanes, and the tile's summary (lane 63's inclusive value)
     const unsigned F = heads ? 1u : 0u;
     wave_exclusive_seg_scan(F, run, ch[j].fe, ch[j].ve);
@@ -262,6 +295,7 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
     const bool muted = part + 1 == wait.mute_partition;
     float prefix = 0.0f;
     unsigned count = 0;
+    const size_t mine = (size_t)part << wait.desc_shift;
     if (part == 0) {
       if (lane == 0 && !muted) {
         atomic_store_u64(desc_v, ((unsigned long long)kKeyStatusPrefix << 32) | __float_as_uint(av));
@@ -269,15 +303,17 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
       }
     } else {
       if (lane == 0 && !muted) {
-        atomic_store_u64(desc_v + part, ((unsigned long long)(kKeyStatusAggregate + (af ? kKeyFlagged : 0u)) << 32) | __float_as_uint(av));
-        if constexpr (REDUCE) atomic_store_u64(desc_c + part, ((unsigned long long)kKeyStatusAggregate << 32) | ah);
+        atomic_store_u64(desc_v + mine, ((unsigned long long)(kKeyStatusAggregate + (af ? kKeyFlagged : 0u)) << 32) | __float_as_uint(av));
+        if constexpr (REDUCE) atomic_store_u64(desc_c + mine, ((unsigned long long)kKeyStatusAggregate << 32) | ah);
       }
-      prefix = look_back_flagged(desc_v, (long long)part, lane, wait);
-      if constexpr (REDUCE) count = look_back_count(desc_c, (long long)part, lane, wait);
+      if constexpr (REDUCE)
+        look_back_value_and_count(desc_v, (long long)part, lane, wait, &prefix, &count);
+      else
+        prefix = look_back_flagged(desc_v, (long long)part, lane, wait);
       if (lane == 0 && !muted) {
-        atomic_store_u64(desc_v + part, ((unsigned long long)kKeyStatusPrefix << 32) | __float_as_uint(af ? av : prefix + av));
+        atomic_store_u64(desc_v + mine, ((unsigned long long)kKeyStatusPrefix << 32) | __float_as_uint(af ? av : prefix + av));
         // a count that could not be had stays "unknown" for every later partition
-        if constexpr (REDUCE) atomic_store_u64(desc_c + part, ((unsigned long long)kKeyStatusPrefix << 32) | (count == 0xffffffffu ? count : count + ah));
+        if constexpr (REDUCE) atomic_store_u64(desc_c + mine, ((unsigned long long)kKeyStatusPrefix << 32) | (count == 0xffffffffu ? count : count + ah));
       }
     }
     if (lane == 0) {
@@ -313,10 +349,14 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
     const float carry = lv;
     const size_t e0 = ((tile0 + j) * kTileChunks + lane) * 8;
     const unsigned heads = ch[j].heads;
-    const int valid = ch[j].valid;
+    const int valid = e0 >= n ? 0 : (n - e0 >= 8 ? 8 : (int)(n - e0));
     float r[8];
+    float run = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) r[i] = (heads & ((2u << i) - 1u)) ? ch[j].p[i] : carry + ch[j].p[i];
+    for (int i = 0; i < 8; i++) {
+      run = ((heads >> i) & 1u) ? (float)ch[j].raw[i] : run + (float)ch[j].raw[i];
+      r[i] = (heads & ((2u << i) - 1u)) ? run : carry + run;
+    }
     if constexpr (!REDUCE) {
       if (valid == 8) {
         const uint4_t packed = {pack_f16x2(r[0], r[1]), pack_f16x2(r[2], r[3]), pack_f16x2(r[4], r[5]), pack_f16x2(r[6], r[7])};

@@ -74,7 +74,15 @@ inline int set_option(const char *name, int value) {
   return TCU_OK;
 }
 
-inline WaitPolicy wait_policy() { return WaitPolicy{options().lookback_poll_limit, options().test_mute_partition}; }
+inline WaitPolicy wait_policy(unsigned desc_shift = 0) { return WaitPolicy{options().lookback_poll_limit, options().test_mute_partition, desc_shift}; }
+// 32-bit words of a look-back workspace: the ticket's line, then one slot of 8 << desc_shift bytes per partition
+inline size_t look_back_words(size_t parts, unsigned desc_shift) { return 64 + 2 * ((parts ? parts : 1) << desc_shift); }
+// 256 bytes per descriptor while that stays within 4 MiB, closer together for the (slow anyway) launches with more partitions
+inline unsigned desc_shift_for(size_t parts) {
+  unsigned shift = kDescShift;
+  while (shift > 0 && (parts << shift) > ((size_t)1 << 19)) shift--;
+  return shift;
+}
 
 inline bool is_pow2(size_t x) { return x && !(x & (x - 1)); }
 inline int ilog2(size_t x) {
@@ -271,23 +279,27 @@ struct ScanScratch {
 inline int seg_scan_huge(const char *what, const half8_t *in, uint4_t *out, uint16_t *totals, size_t num_segments, size_t S, bool nt, void *stream, ScanScratch scratch) {
   const size_t pps = S / kHugePartHalves, parts = num_segments * pps;
   if (parts > kMaxGrid || pps > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-  const size_t words = 64 + 2 * parts;  // ticket counter, then one 64-bit descriptor per partition
+  // ticket counter, then one 64-bit descriptor per partition, 256 bytes apart where the buffer has the room
+  unsigned shift = desc_shift_for(parts);
   unsigned *ws = scratch.words;
   if (ws) {
-    if (words > scratch.capacity)
+    while (shift > 0 && look_back_words(parts, shift) > scratch.capacity) shift--;
+    if (look_back_words(parts, shift) > scratch.capacity)
       return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": " + std::to_string(parts) + " partitions of 65536 halves exceed the built-in scratch buffer (at most " +
                                            std::to_string((scratch.capacity - 64) / 2) + " partitions, i.e. " + std::to_string((scratch.capacity - 64) / 2 * kHugePartHalves) + " halves per call)");
-  } else {
+  }
+  const size_t words = look_back_words(parts, shift);
+  if (!ws) {
     ws = static_cast<unsigned *>(stream_alloc(words * sizeof(unsigned), stream));
     if (!ws) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partition descriptors");
   }
   const size_t n_chunks = num_segments * S / 8;
-  launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
+  launch(zero_look_back_kernel, (unsigned)((parts + 255) / 256), 256u, stream, ws, parts, shift);
   const int static_order = options().static_order ? 1 : 0;
   if (nt)
-    launch(full_scan_kernel<8, false, true>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy());
+    launch(full_scan_kernel<8, false, true>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy(shift));
   else
-    launch(full_scan_kernel<8, false, false>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy());
+    launch(full_scan_kernel<8, false, false>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy(shift));
   if (!scratch.words) stream_free(ws, stream);
   return TCU_OK;
 }
@@ -755,7 +767,8 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
     const size_t n_chunks = n / 8;
     const size_t n_tiles = (n_chunks + kTileChunks - 1) / kTileChunks;
     const size_t parts = (n_tiles + (size_t)p.wpb * p.u - 1) / ((size_t)p.wpb * p.u);
-    const size_t need = round_up(256 + 8 * (parts ? parts : 1), kWorkspaceAlign);
+    const unsigned shift = desc_shift_for(parts);
+    const size_t need = round_up(4 * look_back_words(parts, shift), kWorkspaceAlign);
     if (!d_ws) {
       *ws_bytes = need;
       return TCU_OK;
@@ -765,17 +778,16 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
     if (!d_in || !d_out) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
     if (parts > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     unsigned *ws = static_cast<unsigned *>(d_ws);
-    const size_t words = 64 + 2 * parts;
-    launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
+    launch(zero_look_back_kernel, (unsigned)((parts + 255) / 256), 256u, stream, ws, parts, shift);
     if (lds_held) {  // partitions of 16 x 12 tiles: fewer than `parts`, same workspace layout
       const size_t big_parts = (n_tiles + 16 * 12 - 1) / (16 * 12);
       if (nt)
-        launch(full_scan_lds_kernel<8, 4, true>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy());
+        launch(full_scan_lds_kernel<8, 4, true>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy(shift));
       else
-        launch(full_scan_lds_kernel<8, 4, false>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy());
+        launch(full_scan_lds_kernel<8, 4, false>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy(shift));
       return TCU_OK;
     }
-    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, mfma, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr), wait_policy());
+    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, mfma, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr), wait_policy(shift));
     return TCU_OK;
   }
   // the reference's three-kernel sequence: segmented scan + totals, exclusive scan of the totals, add
@@ -806,7 +818,8 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
   if (!ws_bytes) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": workspace_bytes must not be null");
   if (n >= ((size_t)1 << 32)) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": at most 2^32 - 1 elements (runs are counted in 32 bits)");
   const size_t parts = (n + kByKeyPartition - 1) / kByKeyPartition;
-  const size_t words = 64 + 2 * (parts ? parts : 1) * (reduce ? 2 : 1);
+  const unsigned shift = desc_shift_for(parts) ? desc_shift_for(parts) : 1;  // a slot holds the value and the count descriptor: at least 16 bytes
+  const size_t words = look_back_words(parts, shift);
   const size_t need = round_up(4 * words, kWorkspaceAlign);
   if (!d_ws) {
     *ws_bytes = need;
@@ -822,7 +835,7 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
   if ((reinterpret_cast<uintptr_t>(d_out) & 1u) || (reinterpret_cast<uintptr_t>(d_keys_out) & (sizeof(KEY) - 1)) || (reinterpret_cast<uintptr_t>(d_num_runs) & 7u))
     return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": misaligned output pointer");
   unsigned *ws = static_cast<unsigned *>(d_ws);
-  launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
+  launch(zero_look_back_kernel, (unsigned)((parts + 255) / 256), 256u, stream, ws, parts, shift);
   const int so = options().static_order ? 1 : 0;
   const unsigned grid = (unsigned)parts, block = (unsigned)kByKeyWaves * 64u;
   const KEY *keys = static_cast<const KEY *>(d_keys);
@@ -832,11 +845,11 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
   unsigned long long *num_runs = static_cast<unsigned long long *>(d_num_runs);
   const bool nt = options().nontemporal;
   if (reduce) {
-    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, true, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
-    else launch(by_key_kernel<KEY, kByKeyTiles, true, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, true, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
+    else launch(by_key_kernel<KEY, kByKeyTiles, true, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
   } else {
-    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, false, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
-    else launch(by_key_kernel<KEY, kByKeyTiles, false, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy());
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, false, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
+    else launch(by_key_kernel<KEY, kByKeyTiles, false, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
   }
   return TCU_OK;
 }

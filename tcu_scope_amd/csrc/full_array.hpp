@@ -35,6 +35,22 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned *words, size_t
   if (i < n) words[i] = 0u;
 }
 
+// Clears a look-back workspace: the ticket word and the first four words (two 64-bit descriptors) of
+// every partition's slot; the rest of a slot is never read.
+__global__ __launch_bounds__(256) void zero_look_back_kernel(unsigned *ws, size_t parts, unsigned desc_shift) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i == 0) ws[0] = 0u;
+  if (i < parts) {
+    unsigned *slot = ws + 64 + 2 * (i << desc_shift);
+    slot[0] = 0u;
+    slot[1] = 0u;
+    if (desc_shift) {
+      slot[2] = 0u;
+      slot[3] = 0u;
+    }
+  }
+}
+
 // One partition (blockDim/64 * U tiles) per block, no loop: blocks dispatched in order sweep
 // the array as one moving window, which is what HBM serves fastest (a persistent
 // grid-stride version of this kernel measured 2-3x slower).
@@ -57,11 +73,18 @@ constexpr unsigned long long kPublished = 1ull << 32;
 // that depend on the missing value NaN, never a finite wrong number.  mute_partition (tests
 // only, 0 = none): partition mute_partition - 1 computes its own results but publishes
 // nothing, which makes every wait for it expire while all kernels still run to their end.
+// desc_shift: the look-back descriptors of consecutive partitions lie 8 << desc_shift bytes apart.  Packed
+// descriptors (shift 0) put 16 partitions into one 128-byte line that hundreds of waiting waves poll while
+// its owners keep storing into it; one descriptor per 256 bytes (shift 5) took the full-array scan of 2^28
+// halves from 212 to 191 us.
 struct WaitPolicy {
   unsigned poll_limit;
   unsigned mute_partition;
+  unsigned desc_shift;
 };
 constexpr unsigned kDefaultPollLimit = 1u << 20;
+constexpr unsigned kDescShift = 5;
+
 
 // sum over lanes of the published values at p[lane], lane < count (count <= 64); false if a
 // value never showed up
@@ -158,7 +181,7 @@ TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long 
   unsigned polls = 0;
   while (true) {
     const long long idx = base - lane;
-    const unsigned long long d = idx >= floor ? atomic_load_u64(desc + idx) : kFlagPrefix;
+    const unsigned long long d = idx >= floor ? atomic_load_u64(desc + ((size_t)idx << wait.desc_shift)) : kFlagPrefix;
     const unsigned flag = (unsigned)(d >> 32);
     const unsigned long long is_prefix = ballot(flag == 2u);
     const unsigned long long is_empty = ballot(flag == 0u);
@@ -178,7 +201,7 @@ TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long 
 }
 
 // One partition (blockDim/64 * U tiles) per block.  workspace: ticket counter at word 0,
-// descriptors (64-bit: flag << 32 | float bits) from byte 256.
+// descriptors (64-bit: flag << 32 | float bits) from byte 256, 8 << wait.desc_shift bytes apart.
 // parts_per_segment = 0: one scan over the whole array.  Otherwise the array is a sequence of
 // segments of parts_per_segment whole partitions each, scanned independently (segments far
 // larger than what one block can walk), and `totals`, if given, receives every segment's sum.
@@ -220,12 +243,13 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
     const unsigned in_segment = parts_per_segment ? part % parts_per_segment : part;
     const long long floor = (long long)part - in_segment;
     const bool muted = part + 1 == wait.mute_partition;
+    unsigned long long *mine = desc + ((size_t)part << wait.desc_shift);
     if (in_segment == 0) {
-      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagPrefix | __float_as_uint(aggregate));
     } else {
-      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagAggregate | __float_as_uint(aggregate));
       prefix = look_back(desc, (long long)part, floor, lane, wait);
-      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagPrefix | __float_as_uint(prefix + aggregate));
     }
     if (totals && parts_per_segment && in_segment == parts_per_segment - 1 && lane == 0) totals[part / parts_per_segment] = f16_bits(prefix + aggregate);
     if (lane == 0) s_prefix = prefix;
@@ -294,12 +318,13 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t 
     for (int w = 0; w < WPB; w++) aggregate += wave_total[w];
     float prefix = 0.0f;
     const bool muted = part + 1 == wait.mute_partition;
+    unsigned long long *mine = desc + ((size_t)part << wait.desc_shift);
     if (part == 0) {
-      if (lane == 0 && !muted) atomic_store_u64(desc, kFlagPrefix | __float_as_uint(aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagPrefix | __float_as_uint(aggregate));
     } else {
-      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagAggregate | __float_as_uint(aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagAggregate | __float_as_uint(aggregate));
       prefix = look_back(desc, (long long)part, 0, lane, wait);
-      if (lane == 0 && !muted) atomic_store_u64(desc + part, kFlagPrefix | __float_as_uint(prefix + aggregate));
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagPrefix | __float_as_uint(prefix + aggregate));
     }
     if (lane == 0) s_prefix = prefix;
   }

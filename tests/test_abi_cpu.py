@@ -45,7 +45,7 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.tcu_seg_scan_f16(p, p, None, 4, 16, 7, 5, 0, None) == 1
     need = sz(0)
     assert lib.tcu_full_scan_f16(None, None, 1 << 30, None, ctypes.byref(need), 0, 0, 0, None) == 0
-    assert need.value == 256 + 8 * ((1 << 30) // 65536)
+    assert need.value == 256 + 256 * ((1 << 30) // 65536)  # one look-back descriptor per 256 bytes
     assert lib.tcu_full_reduce_f16(None, None, 1 << 30, None, ctypes.byref(need), 0, 0, 0, None) == 0 and need.value > 0
     assert lib.tcu_full_reduce_f16(None, None, 1000, None, ctypes.byref(need), 2, 2048, 0, None) == 2  # n % segment_size
     assert lib.tcu_full_scan_f16(None, None, 1 << 20, None, None, 0, 0, 0, None) == 1

@@ -81,10 +81,10 @@ def test_noalloc_other_paths_and_limit(tcu, oracle):
         assert torch.equal(out, tcu.seg_scan(xs, seg, variant=variant)), (seg, variant.name)
     # empty input
     tcu.seg_scan_noalloc(xd[:0], 1 << 21, xd[:0])
-    # beyond the built-in array: 65537 partitions of 65536 halves.  Rejected on the host before anything is
+    # beyond the built-in array: 131073 partitions of 65536 halves.  Rejected on the host before anything is
     # launched, so the (far too small) buffers are never touched
     small = torch.zeros(1 << 21, dtype=torch.float16, device="cuda")
     with pytest.raises(tcu.TcuError) as e:
-        tcu.seg_scan_noalloc(small, 1 << 21, small, num_segments=(1 << 11) + 1)
+        tcu.seg_scan_noalloc(small, 1 << 21, small, num_segments=(1 << 12) + 1)
     assert e.value.status == 2 and "scratch" in str(e.value)
     # exactly at the limit the host side accepts the size; not launched here (that would need 16 GiB)
