@@ -4,13 +4,16 @@
 // cub::DeviceScan::InclusiveSum), CUB_DEVICE_SEGMENTED_REDUCTION and its TUNE sweep
 // (src/reduction/seg_cub_device.cu:18-63: cub::DeviceSegmentedReduce::Sum over an offsets
 // array), CUBLAS_WMMA_GEMM (src/gemm/cublas.cu:65: cublasGemmEx, fp16 in, fp32 out) and
-// CUBLAS_GEMV.  Here they run hipCUB (rocPRIM) and rocBLAS, the libraries this GPU ships with.
+// CUBLAS_GEMV.  Here they run hipCUB (rocPRIM) and rocBLAS, the libraries this GPU ships with;
+// HIPBLASLT_GEMM / HIPBLASLT_HGEMM time the same products through hipBLASLt (hipblasLtMatmul with
+// the algorithm its heuristic ranks first), the library PyTorch calls for fp16 matrix products.
 // Nothing of the product calls these libraries; the file only feeds the benchmark executable.
 // Arithmetic: the reductions and the scan read fp16, accumulate in fp32 and write fp16 (the
 // reference's patched CUB adds in fp16), so they move the same bytes as the kernels they are
 // compared with.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
 #include <hipcub/hipcub.hpp>
 #include <rocblas/rocblas.h>
 
@@ -239,6 +242,68 @@ BENCHMARK(CUBLAS_HGEMM)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUBLAS_WMMA_HGEMM)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUBLAS_WMMA_HGEMM_GemmEx)->Apply(GemmArgs)->UseManualTime();
 BENCHMARK(CUBLAS_HGEMM_GemmEx)->Apply(GemmArgs)->UseManualTime();
+
+// The same product through hipBLASLt: in its column-major terms D^T (N x M) = B^T (N x K) * A' (K x M).
+static void lt_check(hipblasStatus_t s, const char *what) {
+  if (s != HIPBLAS_STATUS_SUCCESS) throw std::runtime_error(std::string(what) + ": hipBLASLt status " + std::to_string((int)s));
+}
+static void blaslt_gemm(benchmark::State &state, bool half_out) {
+  guarded(state, [&] {
+    const size_t M = state.range(0), N = state.range(1), K = state.range(2);
+    const float alpha = 1.1f, beta = 1.2f;
+    const size_t out_size = half_out ? 2 : 4;
+    const hipDataType out_type = half_out ? HIP_R_16F : HIP_R_32F;
+    DeviceBuffer A(M * K * 2), B(N * K * 2), C(M * N * out_size), D(M * N * out_size);
+    TCU_CHECK(tcu_generate_f16(A.get(), M * K, harness::flags().seed, TCU_DIST_NORMAL, 0, nullptr));
+    TCU_CHECK(tcu_generate_f16(B.get(), N * K, harness::flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
+    PRINT_IF_ERROR(hipMemset(C.get(), 0, M * N * out_size));
+    static hipblasLtHandle_t lt = [] {
+      hipblasLtHandle_t h = nullptr;
+      lt_check(hipblasLtCreate(&h), "hipblasLtCreate");
+      return h;
+    }();
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr, ld = nullptr;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    lt_check(hipblasLtMatmulDescCreate(&desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "hipblasLtMatmulDescCreate");
+    const hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
+    lt_check(hipblasLtMatmulDescSetAttribute(desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof(op_t)), "TRANSA");
+    lt_check(hipblasLtMatmulDescSetAttribute(desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n)), "TRANSB");
+    lt_check(hipblasLtMatrixLayoutCreate(&la, HIP_R_16F, K, N, K), "layout of B");
+    lt_check(hipblasLtMatrixLayoutCreate(&lb, HIP_R_16F, K, M, K), "layout of A");
+    lt_check(hipblasLtMatrixLayoutCreate(&lc, out_type, N, M, N), "layout of C");
+    lt_check(hipblasLtMatrixLayoutCreate(&ld, out_type, N, M, N), "layout of D");
+    lt_check(hipblasLtMatmulPreferenceCreate(&pref), "hipblasLtMatmulPreferenceCreate");
+    size_t ws_bytes = (size_t)128 << 20;
+    lt_check(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws_bytes, sizeof(ws_bytes)), "workspace preference");
+    DeviceBuffer ws(ws_bytes);
+    hipblasLtMatmulHeuristicResult_t found[1];
+    int n_found = 0;
+    lt_check(hipblasLtMatmulAlgoGetHeuristic(lt, desc, la, lb, lc, ld, pref, 1, found, &n_found), "hipblasLtMatmulAlgoGetHeuristic");
+    if (n_found == 0) throw std::runtime_error("hipBLASLt offers no algorithm for this product");
+    auto run = [&] {
+      lt_check(hipblasLtMatmul(lt, desc, &alpha, B.get(), la, A.get(), lb, &beta, C.get(), lc, D.get(), ld, &found[0].algo, ws.get(), ws_bytes, nullptr), "hipblasLtMatmul");
+    };
+    run();
+    PRINT_IF_ERROR(hipDeviceSynchronize());
+    timed_loop(state, [&](size_t) { run(); });
+    state.counters.insert({{"M", (double)M},
+                           {"N", (double)N},
+                           {"K", (double)K},
+                           {"flops", {state.iterations() * 2.0 * M * N * K, benchmark::Counter::kAvgThreadsRate}},
+                           {"mfma_peak_fraction", {state.iterations() * 2.0 * M * N * K / 2.5e15, benchmark::Counter::kAvgThreadsRate}}});
+    hipblasLtMatmulPreferenceDestroy(pref);
+    hipblasLtMatrixLayoutDestroy(la);
+    hipblasLtMatrixLayoutDestroy(lb);
+    hipblasLtMatrixLayoutDestroy(lc);
+    hipblasLtMatrixLayoutDestroy(ld);
+    hipblasLtMatmulDescDestroy(desc);
+  });
+}
+static void HIPBLASLT_GEMM(benchmark::State &state) { blaslt_gemm(state, false); }
+static void HIPBLASLT_HGEMM(benchmark::State &state) { blaslt_gemm(state, true); }
+BENCHMARK(HIPBLASLT_GEMM)->Apply(GemmArgs)->UseManualTime();
+BENCHMARK(HIPBLASLT_HGEMM)->Apply(GemmArgs)->UseManualTime();
 
 // y (M) = alpha * A (M x K row-major) x + beta * y as a one-column GEMM (fp16 in, fp32 accumulate; y in fp32 or fp16):
 // what the reference's CUDA_WMMA_GEMV_CUBLAS / CUDA_WMMA_HGEMV_CUBLAS do with cuBLAS (src/gemv/wmma_cublas.cu:245-246) and,
