@@ -74,14 +74,15 @@ def test_harness_runs_verifies_and_reports(tmp_path):
             "|CUDA_WMMA_FULL_(REDUCTION_(2KERS_BASE_16|ATOMIC_W_BLOCK_SYNC)|PREFIXSUM_(3KERS|CG))<8 \\* 256, 4>/num_elements:4194304/"
             "|CUDA_WMMA_H?GEM[MV](_NAIVE)?/M:512/|TCU_WAVE_H?GEMV/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/"
             "|CUDA_UNSAFE_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16N<4>|256N_BLOCK<4>)/.*num_elements:4194304/"
-            "|CUB_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/|CUB_DEVICE_SEGMENTED_REDUCTION/.*segment_size:256/num_elements:4194304/|CUBLAS_(WMMA_H?GEMM|GEMV)/M:512/")
+            "|CUB_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/|CUB_DEVICE_SEGMENTED_REDUCTION/.*segment_size:256/num_elements:4194304/|CUBLAS_(WMMA_H?GEMM|GEMV)/M:512/|HIPBLASLT_H?GEMM/M:512/"
+            "|(THRUST|TCU_BY_KEY)_SEGMENTED_(REDUCTION|PREFIXSUM)/.*segment_size:(16|2048)/num_elements:4194304/|THRUST_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/")
     p = subprocess.run([BENCH, f"--benchmark_filter={filt}", "--benchmark_min_time=0.02", f"--benchmark_out={out}", "--benchmark_out_format=json", "--tcu_verify=all", "--v=1"],
                        capture_output=True, text=True, timeout=300)
     assert p.returncode == 0, p.stdout + p.stderr
     assert "ERROR OCCURRED" not in p.stdout, p.stdout
     data = json.loads(out.read_text())
     rows = data["benchmarks"]
-    assert len(rows) >= 40
+    assert len(rows) >= 52
     for r in rows:
         assert r["iterations"] >= 1 and r["real_time"] > 0 and r["flops"] > 0, r
         assert r["name"].endswith("/manual_time")
