@@ -890,13 +890,19 @@ inline int gemv_dispatch_typed(const char *what, const void *A, const void *x, v
   const half8_t *a = static_cast<const half8_t *>(A), *xv = static_cast<const half8_t *>(x);
   OUT *yy = static_cast<OUT *>(y);
   if (variant == TCU_VARIANT_MFMA_16N) {
-    const size_t strips = (M + 15) / 16;
-    const size_t grid = (strips + 3) / 4;
+    // a block per 16-row strip; its waves split K, at least two steps of 256 k each (16384 x 16384: 1 wave 109 us,
+    // 2 waves 112, 4 waves 108, 8 waves 124, 16 waves 117; one wave per strip and 16-byte pieces per row and load: 171)
+    const size_t grid = (M + 15) / 16, steps = (K + 255) / 256;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    int wpb = options().gemv_waves;
+    if (!(wpb == 1 || wpb == 2 || wpb == 4 || wpb == 8 || wpb == 16)) {
+      wpb = 4;
+      while (wpb > 1 && (size_t)wpb * 2 > steps) wpb /= 2;
+    }
     if (nt)
-      launch(gemv_mfma_kernel<true, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+      launch(gemv_mfma_kernel<true, OUT>, (unsigned)grid, (unsigned)wpb * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
     else
-      launch(gemv_mfma_kernel<false, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
+      launch(gemv_mfma_kernel<false, OUT>, (unsigned)grid, (unsigned)wpb * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
     return TCU_OK;
   }
   const size_t k_tiles = (K / 8 + 63) / 64;

@@ -10,11 +10,11 @@
 //   gemv_block_kernel: rows of 8 KiB and more: a block of waves shares two rows (the access
 //                      shape of the block-per-segment reduction), partials meet in LDS.
 //   gemv_mfma_kernel : the reference's formulation (GEMV as a 16-wide GEMM,
-//                      src/gemv/wmma_naive.cu:29-94): a wave owns a 16-row strip, the strip
+//                      src/gemv/wmma_naive.cu:29-94): a block owns a 16-row strip, the strip
 //                      is the A operand of v_mfma_f32_16x16x32_f16 and x, replicated over
-//                      the 16 columns, the B operand.  Lane (r, b) reads 64 contiguous
-//                      bytes of row r per 4 MFMAs (k order inside a step is permuted
-//                      identically for A and x, which a contraction does not see).
+//                      the 16 columns, the B operand; the block's waves split K (k order
+//                      inside a step is permuted identically for A and x, which a
+//                      contraction does not see).
 //   Both of the first two also run with the matrix unit in place of the dot products
 //   (GemvAcc<true>: a row tile times the x tile, trace of the product), which keeps their
 //   access shape.
@@ -143,43 +143,57 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_block_kernel(const half8_t *__
   }
 }
 
-// K must be a multiple of 8.  One wave per 16-row strip.
+// K must be a multiple of 8.  A block per 16-row strip; its waves split K and meet in LDS (one wave per
+// strip leaves a 16384-row matrix with 1024 waves, too few loads in flight: 171 us for 16384 x 16384 where
+// the dot-product kernel needs 80).  Lane (r, b) reads chunks 4 s + b, s = 0 .. 3, of each half step, so that
+// one load instruction reads 64 contiguous bytes of each of the 16 rows.
 template <bool NT, typename OUT>
 __global__ __launch_bounds__(kMaxBlock) void gemv_mfma_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t k_chunks, float alpha,
                                                                float beta) {
-  const int lane = lane_id();
+  __shared__ float partial[kMaxWaves][16];
+  const int lane = lane_id(), wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
   const int r = lane & 15, b = lane >> 4;
-  const size_t strip = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
-  const size_t row0 = strip * 16;
-  if (row0 >= M) return;
+  const size_t row0 = (size_t)blockIdx.x * 16;
   const size_t row = row0 + r < M ? row0 + r : M - 1;
   const half8_t *arow = A + row * k_chunks;
+  // this wave's share of K, in steps of 256 k = 32 chunks
+  const size_t steps = (k_chunks + 31) / 32, per_wave = (steps + WPB - 1) / WPB;
+  const size_t c_begin = (size_t)wave * per_wave * 32;
+  const size_t c_end = c_begin + per_wave * 32 < k_chunks ? c_begin + per_wave * 32 : k_chunks;
   float4_t acc = {0, 0, 0, 0};
-  // a step covers 256 k = 32 chunks in two halves; lane (r, b) takes chunks 4b .. 4b+3 of each half
-  for (size_t c0 = 0; c0 < k_chunks; c0 += 32) {
-    half8_t av[2][4], xv[2][4];
+  constexpr int kSteps = 1;  // steps of 256 k whose loads are in flight together (two measured 181 us against 108 at 16384 x 16384)
+  for (size_t c0 = c_begin; c0 < c_end; c0 += 32 * kSteps) {
+    half8_t av[kSteps][2][4], xv[kSteps][2][4];
 #pragma unroll
-    for (int h = 0; h < 2; h++)
+    for (int t = 0; t < kSteps; t++)
 #pragma unroll
-      for (int s = 0; s < 4; s++) {
-        const size_t c = c0 + (size_t)h * 16 + 4 * b + s;
-        const bool ok = c < k_chunks;
-        const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-        av[h][s] = ok ? load_chunk<NT>(arow + c) : zero;
-        xv[h][s] = ok ? x[c] : zero;
-      }
+      for (int h = 0; h < 2; h++)
 #pragma unroll
-    for (int h = 0; h < 2; h++)
+        for (int s = 0; s < 4; s++) {
+          const size_t c = c0 + (size_t)t * 32 + (size_t)h * 16 + 4 * s + b;
+          const bool ok = c < c_end;
+          const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+          av[t][h][s] = ok ? load_chunk<NT>(arow + c) : zero;
+          xv[t][h][s] = ok ? x[c] : zero;
+        }
 #pragma unroll
-      for (int s = 0; s < 4; s++) acc = mfma_16x16x32(av[h][s], xv[h][s], acc);
+    for (int t = 0; t < kSteps; t++)
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int s = 0; s < 4; s++) acc = mfma_16x16x32(av[t][h][s], xv[t][h][s], acc);
   }
-  // every column of D holds the strip's 16 results; column 0 writes them
+  // every column of D holds the strip's 16 partial results; column 0 hands them over
   if (r == 0) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const size_t m = row0 + 4 * b + i;
-      if (m < M) gemv_update(y + m, acc[i], alpha, beta);
-    }
+    for (int i = 0; i < 4; i++) partial[wave][4 * b + i] = acc[i];
+  }
+  __syncthreads();
+  if (threadIdx.x < 16 && row0 + threadIdx.x < M) {
+    float sum = 0.0f;
+    for (int w = 0; w < WPB; w++) sum += partial[w][threadIdx.x];
+    gemv_update(y + row0 + threadIdx.x, sum, alpha, beta);
   }
 }
 
