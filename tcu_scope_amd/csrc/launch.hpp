@@ -43,14 +43,24 @@ inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void
 // The pool keeps what it has handed out once (release threshold at its maximum): the default
 // pool gives unused memory back to the driver at every synchronisation, which turns the next
 // request into a real allocation of a millisecond or more.  The block may be used by work
-// enqueued on `stream` between stream_alloc and stream_free.  The pool is that of the current
-// device, which must be the device of `stream` (as for every launch made through this library).
+// enqueued on `stream` between stream_alloc and stream_free.  The pool is that of the stream's
+// device (of the current device for the default stream).
 inline void *stream_alloc(size_t bytes, void *stream) {
   constexpr int kMaxDevices = 64;
   static hipMemPool_t pools[kMaxDevices] = {};
   static std::mutex pools_mutex;
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  if (stream) {
+    hipDevice_t of_stream = 0;
+    if (hipStreamGetDevice(static_cast<hipStream_t>(stream), &of_stream) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    dev = (int)of_stream;
+  } else if (hipGetDevice(&dev) != hipSuccess) {
+    return nullptr;
+  }
+  if (dev < 0 || dev >= kMaxDevices) return nullptr;
   std::lock_guard<std::mutex> lock(pools_mutex);
   if (!pools[dev]) {
     hipMemPoolProps props = {};
