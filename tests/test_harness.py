@@ -104,3 +104,53 @@ def test_harness_runs_verifies_and_reports(tmp_path):
     p = subprocess.run([BENCH, "--benchmark_filter=CUDA_WMMA_SEGMENTED_REDUCTION_16N_BLOCK<4>/.*segment_size:512/num_elements:4096/", "--tcu_input=constant", "--benchmark_min_time=0.01"],
                        capture_output=True, text=True, timeout=120)
     assert p.returncode == 0 and "ERROR OCCURRED" not in p.stdout, p.stdout
+
+
+def _series_points(rows, regex, xfield, yfield):
+    """What the reference's plotting tool does with one `series:` entry (tools/plot.py:105-163, restated): anchor the
+    regex, keep the benchmarks it finds that did not fail, take the key:value parts of the name as fields where the
+    row has none of that name, drop rows whose x or y is missing or zero, sort by x."""
+    rx = re.compile(regex if regex.startswith("^") else "^" + regex)
+    pts = []
+    for b in rows:
+        if not rx.search(b["name"]) or b.get("error_occurred", False):
+            continue
+        fields = dict(b)
+        for part in b["name"].split("/")[1:]:
+            if part != "manual_time" and ":" in part:
+                k, v = part.split(":", 1)
+                fields.setdefault(k, float(v))
+        if xfield in fields and yfield in fields and float(fields[xfield]) != 0 and float(fields[yfield]) != 0:
+            pts.append((float(fields[xfield]), float(fields[yfield])))
+    return sorted(pts)
+
+
+@pytest.mark.gpu
+def test_json_output_feeds_the_reference_figure_specs(tmp_path):
+    """The JSON the harness writes goes through the selection steps of the reference's plotting tool for three of
+    its figure specifications (one per x axis: num_elements, num_segments, M) and yields a curve for every series
+    this build has benchmarks for."""
+    spec = json.loads(open(os.path.join(os.path.dirname(__file__), "golden", "plot_spec_series.json")).read())
+    out = tmp_path / "figs.json"
+    filt = ("^(CUB_FULL_PREFIXSUM|CUDA_WMMA_FULL_PREFIXSUM_3KERS<(256|8 \\* 256), (1|2|4|8)>)/num_elements:(4096|65536|1048576|16777216)/"
+            "|^(THRUST_SEGMENTED_PREFIXSUM|CUB_WARP_SEGMENTED_PREFIXSUM<256, 16>|CUDA_WMMA_SEGMENTED_PREFIXSUM_16<(1|2), 2>)/num_segments:(1024|16384|262144)/segment_size:16/"
+            "|^(CUDA_WMMA_HGEMM|CUDA_WMMA_GEMM_NAIVE|CUBLAS_HGEMM|CUBLAS_WMMA_HGEMM)/M:(256|512|1024)/N:(256|512|1024)/K:(256|512|1024)/")
+    p = subprocess.run([BENCH, f"--benchmark_filter={filt}", "--benchmark_min_time=0.01", f"--benchmark_out={out}", "--benchmark_out_format=json"], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stdout + p.stderr
+    doc = json.loads(out.read_text())
+    assert {"context", "benchmarks"} <= set(doc) and "date" in doc["context"]
+    rows = doc["benchmarks"]
+    curves = 0
+    for fig, min_points in (("full_prefixsum.yml", 3), ("segmented_prefixsum_16.yml", 3), ("gemm_16_16.yml", 3)):
+        s = spec[fig]
+        xfield, yfield = s["xaxis"]["field"], s["yaxis"]["field"]
+        assert yfield == "flops"
+        for series in s["series"]:
+            pts = _series_points(rows, series["regex"], series.get("xfield", xfield), series.get("yfield", yfield))
+            if not pts:
+                continue  # a series whose benchmarks the filter above leaves out (other template arguments, CUTLASS)
+            xs = [x for x, _ in pts]
+            assert len(pts) >= min_points and len(set(xs)) == len(xs), (fig, series["regex"], pts)
+            assert all(y > 0 and y == y for _, y in pts)
+            curves += 1
+    assert curves >= 12, curves
