@@ -103,7 +103,10 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
  *   "scan_lds_tiles"  0/1, default 1: full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves)
  *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step
- *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more)
+ *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more);
+ *                     "gemv_waves" also sets the waves that split K in the strip kernels (TCU_VARIANT_MFMA_16N)
+ *   "gemv_strip_lds"  0/1, default 1: TCU_VARIANT_MFMA_16N stages the 16-row strip through LDS where K is a
+ *                     multiple of 512 (0: operands straight from global memory at every K)
  *   "gemm_big_tiles"  -1/0/1, default -1: 256 x 256 block tiles wherever M and N allow (1), never (0), or
  *                     where the output has at least 128 of them (-1; smaller outputs take 128 x 128 tiles)
  *   "gemm_direct_lds" -1/0/3/4/64/65/66, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS

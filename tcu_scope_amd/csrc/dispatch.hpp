@@ -40,6 +40,7 @@ struct Options {
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
+  bool gemv_strip_lds = true;  // strip GEMV (TCU_VARIANT_MFMA_16N): stage the strip through LDS where K is a multiple of 512
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
   int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
   int gemm_split_tail = 1;     // spread the K steps of the tiles of a last, partly filled round of the GEMM grid over all compute units: 0 never, 1 where it pays, 2 always
@@ -63,6 +64,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_rows") o.gemv_rows = value;
   else if (n == "gemv_tiles") o.gemv_tiles = value;
   else if (n == "gemv_waves") o.gemv_waves = value;
+  else if (n == "gemv_strip_lds") o.gemv_strip_lds = value != 0;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
@@ -895,6 +897,12 @@ inline int gemv_dispatch_typed(const char *what, const void *A, const void *x, v
     const size_t grid = (M + 15) / 16, steps = (K + 255) / 256;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     int wpb = options().gemv_waves;
+    if (K % 512 == 0 && options().gemv_strip_lds) {  // whole steps of 512 k: the strip goes through LDS
+      if (!(wpb == 1 || wpb == 2 || wpb == 4)) wpb = 4;
+      while (wpb > 1 && (size_t)wpb > K / 512) wpb /= 2;
+      launch(gemv_strip_lds_kernel<OUT>, (unsigned)grid, (unsigned)wpb * 64u, stream, a, xv, yy, M, K / 8, alpha, beta);
+      return TCU_OK;
+    }
     if (!(wpb == 1 || wpb == 2 || wpb == 4 || wpb == 8 || wpb == 16)) {
       wpb = 4;
       while (wpb > 1 && (size_t)wpb * 2 > steps) wpb /= 2;
