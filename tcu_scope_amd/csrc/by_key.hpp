@@ -350,12 +350,15 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
     const size_t e0 = ((tile0 + j) * kTileChunks + lane) * 8;
     const unsigned heads = ch[j].heads;
     const int valid = e0 >= n ? 0 : (n - e0 >= 8 ? 8 : (int)(n - e0));
+    const bool last_lane = valid > 0 && e0 + (size_t)valid == n;  // holds the last element of the array
     float r[8];
-    float run = 0.0f;
+    if (!REDUCE || heads != 0u || last_lane) {  // the reduction needs the sums only where a run ends
+      float run = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      run = ((heads >> i) & 1u) ? (float)ch[j].raw[i] : run + (float)ch[j].raw[i];
-      r[i] = (heads & ((2u << i) - 1u)) ? run : carry + run;
+      for (int i = 0; i < 8; i++) {
+        run = ((heads >> i) & 1u) ? (float)ch[j].raw[i] : run + (float)ch[j].raw[i];
+        r[i] = (heads & ((2u << i) - 1u)) ? run : carry + run;
+      }
     }
     if constexpr (!REDUCE) {
       if (valid == 8) {
@@ -379,13 +382,13 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
             }
           }
         }
-        if (valid > 0 && e0 + (size_t)valid == n) {  // the lane that holds the last element closes the last run
+        if (last_lane) {  // closes the last run
           const unsigned runs = hb + (unsigned)__builtin_popcount(heads);
           out[runs - 1] = f16_bits(r[valid - 1]);
           if (keys_out) keys_out[runs - 1] = keys[n - 1];
           if (num_runs) *num_runs = runs;
         }
-      } else if (valid > 0 && e0 + (size_t)valid == n && num_runs) {
+      } else if (last_lane && num_runs) {
         *num_runs = ~0ull;  // a wait expired: the number of runs is unknown
       }
     }
