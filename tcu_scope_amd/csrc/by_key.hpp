@@ -173,7 +173,7 @@ struct KeyChunk {
 // workspace words: [0] ticket, [64 ...) per partition a u64 value descriptor followed by a u64 count descriptor
 template <typename KEY, int U, bool REDUCE, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict__ keys, const uint16_t *in, uint16_t *out, KEY *__restrict__ keys_out, unsigned long long *num_runs,
-                                                           size_t n, unsigned *ws, unsigned n_parts, int static_order, WaitPolicy wait) {
+                                                           size_t n, unsigned *ws, int static_order, WaitPolicy wait) {
   __shared__ float wave_v[kMaxWaves];
   __shared__ unsigned wave_f[kMaxWaves], wave_h[kMaxWaves];
   __shared__ unsigned s_part, s_count;

@@ -847,11 +847,11 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
   unsigned long long *num_runs = static_cast<unsigned long long *>(d_num_runs);
   const bool nt = options().nontemporal;
   if (reduce) {
-    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, true, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
-    else launch(by_key_kernel<KEY, kByKeyTiles, true, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, true, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
+    else launch(by_key_kernel<KEY, kByKeyTiles, true, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
   } else {
-    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, false, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
-    else launch(by_key_kernel<KEY, kByKeyTiles, false, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, (unsigned)parts, so, wait_policy(shift));
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, false, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
+    else launch(by_key_kernel<KEY, kByKeyTiles, false, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
   }
   return TCU_OK;
 }
