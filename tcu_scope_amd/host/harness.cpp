@@ -43,6 +43,8 @@ void init_flags(int *argc, char **argv) {
       f.verify = v;
     else if (take(argv[i], "tcu_seed", &v))
       f.seed = std::strtoull(v.c_str(), nullptr, 0);
+    else if (take(argv[i], "tcu_option", &v))
+      f.options.push_back(v);
     else if (take(argv[i], "v", &v))
       f.verbose = std::atoi(v.c_str());
     else if (take(argv[i], "help", &v) || std::strcmp(argv[i], "-h") == 0)
@@ -59,6 +61,7 @@ void init_flags(int *argc, char **argv) {
         "  --cuda_device_id=<n>   device to run on (0 when absent)\n"
         "  --tcu_input=uniform|constant|grid   inputs: seeded uniform [-1,1) (default), the constant 0.001, or k/2048\n"
         "  --tcu_verify=auto|all|none          check results against a CPU fp64 sum before timing (auto: up to 2^26 elements)\n"
+        "  --tcu_option=<name>:<value>         a tuning switch of the library (tcu_set_option), may be given several times\n"
         "  --tcu_seed=<n>  --v=<level>\n");
   }
 }
@@ -68,6 +71,13 @@ bool init_device() {
   if (rc != TCU_OK) {
     std::fprintf(stderr, "tcu_init failed: %s\n", tcu_last_error());
     return false;
+  }
+  for (const std::string &o : flags().options) {  // after tcu_init, which sets some of them from the device
+    const size_t colon = o.find(':');
+    if (colon == std::string::npos || tcu_set_option(o.substr(0, colon).c_str(), std::atoi(o.c_str() + colon + 1)) != TCU_OK) {
+      std::fprintf(stderr, "--tcu_option=%s: %s\n", o.c_str(), colon == std::string::npos ? "expected <name>:<value>" : tcu_last_error());
+      return false;
+    }
   }
   int cus = 0, wave = 0, lds = 0, gfx950 = 0;
   tcu_device_info(&cus, &wave, &lds, &gfx950);
