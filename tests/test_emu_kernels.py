@@ -128,7 +128,7 @@ def test_segmented_reduction_over_offsets(emu, oracle):
     x = oracle.generate_f16(n, 9, oracle.DIST_GRID)  # exact partial sums: any order gives the same bits
     xi = copy_in(x)
     for max_len, expected, bits in ((20, 16, 32), (20, 0, 64), (300, 128, 64), (3000, 0, 32), (3000, 2048, 32), (40, 64, 32), (9000, 4096, 32), (40000, 20000, 64), (3000, 100000, 32), (40000, 1 << 17, 64), (3000, 3 << 17, 32)):
-        nseg = 12 if expected >= (1 << 17) else 200 if max_len > 1000 else 600
+        nseg = 12 if expected >= (1 << 17) else 100 if max_len > 1000 else 300
         begin, end = ragged_offsets(rng, n, nseg, max_len)
         want = oracle.seg_reduce_offsets_f64(x, begin, end).astype(np.float16).view(np.uint16)
         assert np.array_equal(want, oracle.seg_reduce_offsets_ref(x, begin, end))
