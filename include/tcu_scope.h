@@ -73,7 +73,7 @@ typedef enum {
 /* Strategies of the full-array entry points. */
 typedef enum {
   TCU_FULL_AUTO = 0,
-  TCU_FULL_SINGLE_PASS = 1, /* one kernel: atomic ticket + carry (reduce), decoupled look-back (scan);
+  TCU_FULL_SINGLE_PASS = 1, /* one kernel: published partials added by the grid's last blocks (reduce), decoupled look-back (scan);
                                replaces reference *_ATOMIC_W_BLOCK_SYNC / _ATOMIC_BALLOT / _CG */
   TCU_FULL_MULTI_KERNEL = 2, /* reference "2 kernels" (reduce) / "3 kernels" (scan) sequences */
   TCU_FULL_MFMA = 0x100     /* flag, OR-ed onto a strategy: the single-pass kernels add (reduce: D += A * ones) and scan

@@ -2,9 +2,9 @@
 //
 // Single-pass kernels:
 //   full_reduce_kernel : one partition per block; every block publishes {1, fp32 partial} as
-//     one 64-bit word and takes a ticket from its group's counter; the last block of a group
-//     adds the group's words, the last group adds the group sums (index order, so the result
-//     does not depend on timing) and writes the fp16 result.  Replaces the reference's
+//     one 64-bit word; the last block of every group of 64 adds the group's words, the last
+//     block of the grid adds the group sums (index order, so the result does not depend on
+//     timing) and writes the fp16 result.  Replaces the reference's
 //     atomic / cooperative-groups full reductions (src/reduction/kernel.cuh:564-786), whose
 //     combine step is an atomicAdd on one half (or a serial loop in global thread 0).
 //   full_scan_kernel, full_scan_lds_kernel : decoupled look-back.  Partitions are handed out
@@ -56,15 +56,20 @@ __global__ __launch_bounds__(256) void zero_look_back_kernel(unsigned *ws, size_
 // grid-stride version of this kernel measured 2-3x slower).
 // Completion is detected without fences (an agent-scope release/acquire pair per block costs
 // about 90 ns of L2 write-back/invalidate and made this kernel 20x slower than the data
-// movement) and without a hot counter (same-address device-scope atomics retire at about
-// one per 11 ns): every block publishes {1, partial} as ONE 64-bit word, then takes a
-// ticket from the counter of its group of 64 blocks; the block that draws the last ticket
-// of a group reads the group's 64 words (polling the few that may still be in flight),
-// publishes the group sum the same way and takes a ticket from the top counter; the last
-// group adds the group sums and writes the result.  All sums run in index order, so the
-// result does not depend on timing.
-// workspace words: [0] top counter, [64 .. 64+groups) group counters, then (8-byte
-// aligned) u64 partial[blocks], u64 group_sum[groups]; all zeroed before the launch.
+// movement), without a hot counter (same-address device-scope atomics retire at about one
+// per 11 ns) and without any atomic that returns a value (a block that waits for its ticket
+// holds its compute unit 1-2 us longer: 352 against 314 us for the plain partition sums at
+// 2^30): every block publishes {1, partial} as ONE 64-bit word and is done, like a block of
+// partition_sums_kernel.  The last block BY INDEX of every group of 64 blocks goes on: its
+// first wave reads the group's 64 words (polling the few that are still in flight: its
+// predecessors were dispatched before it) and publishes the group sum the same way; the last
+// block of the grid then adds the group sums and writes the result.  A block that adds never
+// waits for a block that adds on the same level, and the blocks that only publish never wait
+// at all, so the kernel finishes in whatever order the blocks are dispatched; every wait is
+// bounded all the same, and a value that never shows up makes the result NaN.  All sums run
+// in index order, so the result does not depend on timing.
+// workspace words: [0 .. 64 + groups) unused (64 + groups rounded up to an even number),
+// then u64 partial[blocks], u64 group_sum[groups]; zeroed before the launch.
 constexpr unsigned kFullReduceGroup = 64;
 constexpr unsigned long long kPublished = 1ull << 32;
 
@@ -104,13 +109,11 @@ TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, in
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, unsigned *ws, WaitPolicy wait) {
   __shared__ float partial[kMaxWaves];
-  __shared__ unsigned ticket;
   const int lane = lane_id();
   const int wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
   const unsigned n_blocks = gridDim.x;
   const unsigned n_groups = (n_blocks + kFullReduceGroup - 1) / kFullReduceGroup;
-  unsigned *group_counter = ws + 64;
   unsigned long long *partials = reinterpret_cast<unsigned long long *>(ws + 64 + ((n_groups + 1) & ~1u));
   unsigned long long *group_sum = partials + n_blocks;
   const half8_t ones = splat8(1.0f);
@@ -131,42 +134,28 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   }
   if (lane == 63) partial[wave] = total;
   __syncthreads();
-  const unsigned g = blockIdx.x / kFullReduceGroup;
-  if (threadIdx.x == 0) {
-    float s = 0.0f;
-    for (int w = 0; w < WPB; w++) s += partial[w];
-    if (blockIdx.x + 1 != wait.mute_partition) atomic_store_u64(partials + blockIdx.x, kPublished | __float_as_uint(s));
-    ticket = atomic_add_u32(group_counter + g, 1u);
-  }
-  __syncthreads();
+  if (wave != 0) return;
+  float s = 0.0f;
+  for (int w = 0; w < WPB; w++) s += partial[w];
+  const unsigned b = blockIdx.x;
+  if (lane == 0 && b + 1 != wait.mute_partition) atomic_store_u64(partials + b, kPublished | __float_as_uint(s));
+  const unsigned g = b / kFullReduceGroup;
   const unsigned first = g * kFullReduceGroup;
   const unsigned members = n_blocks - first < kFullReduceGroup ? n_blocks - first : kFullReduceGroup;
-  if (ticket != members - 1) return;  // block-uniform
-  if (wave != 0) return;
-  const uint16_t failed = 0x7e00u;  // NaN: a published value never became visible
-  float s;
-  if (!gather_published(partials + first, members, lane, &s, wait.poll_limit)) {
-    if (lane == 0) out[0] = failed;
-    return;
-  }
-  unsigned top = 0;
-  if (lane == 63) {
-    atomic_store_u64(group_sum + g, kPublished | __float_as_uint(s));
-    top = atomic_add_u32(ws, 1u);
-  }
-  top = readlane_u32(top, 63);
-  if (top != n_groups - 1) return;  // wave-uniform
+  if (b != first + members - 1) return;  // wave-uniform: only a group's last block goes on
+  const float failed = __builtin_nanf("");  // a published value never became visible
+  float gs;
+  if (!gather_published(partials + first, members, lane, &gs, wait.poll_limit)) gs = failed;
+  if (lane == 0) atomic_store_u64(group_sum + g, kPublished | __float_as_uint(gs));
+  if (g != n_groups - 1) return;  // wave-uniform: only the last block of the grid goes on
   float t = 0.0f;
   for (unsigned base = 0; base < n_groups; base += 64) {
     const unsigned count = n_groups - base < 64 ? n_groups - base : 64;
     float part;
-    if (!gather_published(group_sum + base, count, lane, &part, wait.poll_limit)) {
-      if (lane == 0) out[0] = failed;
-      return;
-    }
+    if (!gather_published(group_sum + base, count, lane, &part, wait.poll_limit)) part = failed;
     t += part;
   }
-  if (lane == 0) out[0] = f16_bits(t);
+  if (lane == 0) out[0] = t != t ? (uint16_t)0x7e00u : f16_bits(t);
 }
 
 // Decoupled look-back of partition `part` over the descriptors desc[floor .. part): wave 0 reads
