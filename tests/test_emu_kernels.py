@@ -5,6 +5,7 @@ fibers per wave; it is strict about divergence around cross-lane operations.  Th
 indexing, lane-layout arithmetic, masks and tails without a GPU; the hardware behaviour
 the emulation assumes is checked by tests/test_gpu_probe.py on the GPU."""
 import ctypes
+import mmap
 import os
 import subprocess
 
@@ -46,10 +47,25 @@ def emu():
     return L
 
 
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+PAGE = mmap.PAGESIZE
+# Every array handed to the emulated kernels lies between two inaccessible pages, so an access outside it ends the
+# test run with a segmentation fault instead of reading or writing a neighbour.  "end" (default): the array's last
+# byte (rounded up to 16) is the last byte before the page behind it; "start": its first byte follows the page in front.
+GUARD = os.environ.get("TCU_EMU_GUARD", "end")
+
+
 def aligned(n, dtype, fill=None):
-    raw = np.zeros(n * np.dtype(dtype).itemsize + 256, np.uint8)
-    off = (-raw.ctypes.data) % 256
-    a = raw[off:off + n * np.dtype(dtype).itemsize].view(dtype)
+    nbytes = n * np.dtype(dtype).itemsize
+    body = max((nbytes + PAGE - 1) // PAGE, 1) * PAGE
+    m = mmap.mmap(-1, body + 2 * PAGE)
+    base = ctypes.addressof(ctypes.c_char.from_buffer(m))
+    for guard in (base, base + PAGE + body):
+        if _libc.mprotect(guard, PAGE, 0) != 0:  # PROT_NONE
+            raise OSError(ctypes.get_errno(), "mprotect")
+    off = PAGE if GUARD == "start" else PAGE + body - (nbytes + 15) // 16 * 16
+    a = np.frombuffer(m, dtype=np.uint8, count=nbytes, offset=off).view(dtype)
     if fill is not None:
         a[:] = fill
     return a
