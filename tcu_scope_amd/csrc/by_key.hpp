@@ -178,6 +178,12 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
   __shared__ unsigned wave_f[kMaxWaves], wave_h[kMaxWaves];
   __shared__ unsigned s_part, s_count;
   __shared__ float s_prefix;
+  // The reduction writes a run's key where the run ends, after the look-back.  By then the partition's keys have
+  // left the registers, and the 4 MiB of L2 of an XCD as well (32 partitions of 128 KiB in flight per XCD), so reading
+  // them again from memory costs a second pass over the key array when runs are short (measured: 1.5x the
+  // algorithmic bytes at 16 elements per run).  32-bit keys are therefore parked in LDS (128 KiB per partition).
+  constexpr bool STAGE_KEYS = REDUCE && sizeof(KEY) == 4 && U <= 4;
+  __shared__ __attribute__((aligned(16))) KEY staged_keys[STAGE_KEYS ? kMaxWaves * U * kTileChunks * 8 : 4];
   const int lane = lane_id(), wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
   // a partition's two descriptors (value, head count) are neighbours; partitions are 8 << wait.desc_shift bytes apart
@@ -213,6 +219,11 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
           k[i] = (KEY)a[i];
           k[4 + i] = (KEY)b[i];
         }
+        if constexpr (STAGE_KEYS) {
+          uint4_t *slot = reinterpret_cast<uint4_t *>(staged_keys + (((size_t)wave * U + j) * kTileChunks + lane) * 8);
+          slot[0] = a;
+          slot[1] = b;
+        }
       } else {
 #pragma unroll
         for (int q = 0; q < 4; q++) {
@@ -227,6 +238,7 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
         const bool ok = i < valid;
         v[i] = ok ? __builtin_bit_cast(half_t, in[e0 + i]) : (half_t)0.0f;
         k[i] = ok ? keys[e0 + i] : (KEY)0;
+        if constexpr (STAGE_KEYS) staged_keys[(((size_t)wave * U + j) * kTileChunks + lane) * 8 + i] = k[i];
       }
     }
     // the key before the chunk: the previous lane's last key; lane 0 takes it from the wave's previous tile or from memory
@@ -378,7 +390,10 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
             const unsigned idx = hb + (unsigned)__builtin_popcount(heads & ((1u << i) - 1u));  // runs started before element i
             if (idx > 0) {  // the run that ends at element i - 1
               out[idx - 1] = f16_bits(i ? r[i - 1] : carry);
-              if (keys_out) keys_out[idx - 1] = keys[e0 + i - 1];  // idx > 0: element 0 is not meant, the read stays inside the array
+              if (keys_out) {  // idx > 0: element 0 is not meant, the read stays inside the array
+                const size_t local = (((size_t)wave * U + j) * kTileChunks + lane) * 8 + i;  // position in the partition
+                keys_out[idx - 1] = STAGE_KEYS && local > 0 ? staged_keys[STAGE_KEYS ? local - 1 : 0] : keys[e0 + i - 1];
+              }
             }
           }
         }
