@@ -182,8 +182,12 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
   // left the registers, and the 4 MiB of L2 of an XCD as well (32 partitions of 128 KiB in flight per XCD), so reading
   // them again from memory costs a second pass over the key array when runs are short (measured: 1.5x the
   // algorithmic bytes at 16 elements per run).  32-bit keys are therefore parked in LDS (128 KiB per partition).
+  // 64-bit keys do not fit; for them every chunk parks one key, the one in front of the chunk's first run start (32 KiB),
+  // which serves every run of 8 elements and more; only the further run starts of a chunk read their key again.
   constexpr bool STAGE_KEYS = REDUCE && sizeof(KEY) == 4 && U <= 4;
+  constexpr bool STAGE_FIRST = REDUCE && !STAGE_KEYS;
   __shared__ __attribute__((aligned(16))) KEY staged_keys[STAGE_KEYS ? kMaxWaves * U * kTileChunks * 8 : 4];
+  __shared__ KEY staged_first[STAGE_FIRST ? kMaxWaves * U * kTileChunks : 1];
   const int lane = lane_id(), wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
   // a partition's two descriptors (value, head count) are neighbours; partitions are 8 << wait.desc_shift bytes apart
@@ -255,6 +259,16 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
     for (int i = 0; i < 8; i++) {
       const KEY before = i ? k[i - 1] : pk;
       if (i < valid && (k[i] != before || e0 + i == 0)) heads |= 1u << i;
+    }
+    if constexpr (STAGE_FIRST) {
+      if (heads != 0u) {
+        const int first = __builtin_ctz(heads);
+        KEY kb = pk;
+#pragma unroll
+        for (int i = 1; i < 8; i++)
+          if (first == i) kb = k[i - 1];
+        staged_first[((size_t)wave * U + j) * kTileChunks + lane] = kb;
+      }
     }
     float run = 0.0f;
 #pragma unroll
@@ -391,8 +405,12 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
             if (idx > 0) {  // the run that ends at element i - 1
               out[idx - 1] = f16_bits(i ? r[i - 1] : carry);
               if (keys_out) {  // idx > 0: element 0 is not meant, the read stays inside the array
-                const size_t local = (((size_t)wave * U + j) * kTileChunks + lane) * 8 + i;  // position in the partition
-                keys_out[idx - 1] = STAGE_KEYS && local > 0 ? staged_keys[STAGE_KEYS ? local - 1 : 0] : keys[e0 + i - 1];
+                const size_t slot = ((size_t)wave * U + j) * kTileChunks + lane;  // this chunk's position in the partition
+                const size_t local = slot * 8 + i;
+                if constexpr (STAGE_KEYS)
+                  keys_out[idx - 1] = local > 0 ? staged_keys[local - 1] : keys[e0 + i - 1];
+                else
+                  keys_out[idx - 1] = (heads & ((1u << i) - 1u)) == 0u ? staged_first[slot] : keys[e0 + i - 1];
               }
             }
           }
