@@ -190,6 +190,22 @@ inline int block_family_tiles(int variant, size_t S, int wpb, int otherwise) {
   return u;
 }
 
+// The launch of a block kernel (seg_*_block_kernel) whose block could hold more tiles than a segment has: a wave
+// takes no more tiles than the segment has, the waves form groups of `group` that share a segment each (the
+// smallest power of two whose waves cover the segment in one step, at most the block), and the block owns at
+// least as many segments as it has groups.  All arguments are powers of two.
+struct BlockShape {
+  int u;
+  unsigned group, spb;
+};
+inline BlockShape block_shape(size_t tiles_per_seg, int u, int wpb, unsigned spb) {
+  while (u > 1 && (size_t)u > tiles_per_seg) u /= 2;
+  unsigned group = 1;
+  while (group < (unsigned)wpb && (size_t)group * u < tiles_per_seg) group *= 2;
+  const unsigned in_flight = (unsigned)wpb / group;
+  return {u, group, spb < in_flight ? in_flight : spb};
+}
+
 // ----- segmented reduction ----------------------------------------------------------------
 
 template <int LPS_LOG2, int U, bool MFMA>
@@ -338,10 +354,11 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
 
   if (use_block) {
     const size_t tiles_per_seg = S / kTileHalves;
-    const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;  // the reference's 16n_block owns 16 segments per block
-    const size_t grid = (num_segments + spb - 1) / spb;
+    // the reference's 16n_block owns 16 segments per block
+    const BlockShape shape = block_shape(tiles_per_seg, u, wpb, variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u);
+    const size_t grid = (num_segments + shape.spb - 1) / shape.spb;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_f16: grid exceeds the launch limit");
-    TCU_SWITCH_U_MFMA_NT(seg_reduce_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tiles_per_seg, spb, run);
+    TCU_SWITCH_U_MFMA_NT(seg_reduce_block_kernel, shape.u, a.mfma, nt, (unsigned)grid, block, stream, in, out, n_chunks, num_segments, tiles_per_seg, shape.spb, shape.group, run);
     return TCU_OK;
   }
   if (S <= 512) {
@@ -523,10 +540,10 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
 
   if (use_block) {
     const size_t tiles_per_seg = S / kTileHalves;
-    const unsigned spb = variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u;
-    const size_t grid = (num_segments + spb - 1) / spb;
+    const BlockShape shape = block_shape(tiles_per_seg, u, wpb, variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u);
+    const size_t grid = (num_segments + shape.spb - 1) / shape.spb;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    TCU_SWITCH_U_MFMA_NT(seg_scan_block_kernel, u, a.mfma, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, spb, run);
+    TCU_SWITCH_U_MFMA_NT(seg_scan_block_kernel, shape.u, a.mfma, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, shape.spb, shape.group, run);
     return TCU_OK;
   }
   int lps_log2, tps_log2 = 0;

@@ -214,35 +214,43 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_long_kernel(const half8_
 }
 
 // ---------------------------------------------------------------------------------------
-// S >= 512: a block of WPB waves shares each segment (segs_per_block consecutive ones)
+// S >= 512: the waves of a block share segments.  A block owns segs_per_block consecutive
+// segments; groups of waves_per_seg waves (a power of two that divides the block) take one
+// segment each, blockDim / 64 / waves_per_seg segments at a time, so a block with more
+// waves than a segment has tiles still keeps every wave busy.
 // ---------------------------------------------------------------------------------------
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void seg_reduce_block_kernel(const half8_t *__restrict__ in, uint16_t *__restrict__ out, size_t n_chunks, size_t num_segments, size_t tiles_per_seg,
-                                                                      unsigned segs_per_block, unsigned xcd_run) {
+                                                                      unsigned segs_per_block, unsigned waves_per_seg, unsigned xcd_run) {
   __shared__ float partial[kMaxWaves];
   const int lane = lane_id();
   const int wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
+  const int G = (int)waves_per_seg, Q = WPB / G;  // waves per segment, segments in flight
+  const int q = wave / G, wg = wave % G;           // this wave's group, and its place in the group
   const half8_t ones = splat8(1.0f);
   const size_t piece = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run);
-  for (unsigned sb = 0; sb < segs_per_block; sb++) {
-    const size_t seg = piece * segs_per_block + sb;
-    if (seg >= num_segments) break;  // block-uniform
+  for (unsigned sb = 0; sb < segs_per_block; sb += (unsigned)Q) {
+    if (piece * segs_per_block + sb >= num_segments) break;  // block-uniform
+    const size_t seg = piece * segs_per_block + sb + (unsigned)q;
+    const bool live = sb + (unsigned)q < segs_per_block && seg < num_segments;  // uniform over the group
     const size_t tile_base = seg * tiles_per_seg;
     float accs = 0.0f;
     float4_t accm = {0, 0, 0, 0};
-    for (size_t t0 = (size_t)wave * U; t0 < tiles_per_seg; t0 += (size_t)WPB * U) {
-      half8_t v[U];
-      // tiles past the end of the segment must not be read: clamp the chunk limit
-      size_t lim = (tile_base + tiles_per_seg) * kTileChunks;
-      if (lim > n_chunks) lim = n_chunks;
-      load_tiles<U, NT>(v, in, (tile_base + t0) * kTileChunks, lim, lane);
+    if (live) {
+      for (size_t t0 = (size_t)wg * U; t0 < tiles_per_seg; t0 += (size_t)G * U) {
+        half8_t v[U];
+        // tiles past the end of the segment must not be read: clamp the chunk limit
+        size_t lim = (tile_base + tiles_per_seg) * kTileChunks;
+        if (lim > n_chunks) lim = n_chunks;
+        load_tiles<U, NT>(v, in, (tile_base + t0) * kTileChunks, lim, lane);
 #pragma unroll
-      for (int j = 0; j < U; j++) {
-        if constexpr (MFMA)
-          accm = mfma_16x16x32(v[j], ones, accm);
-        else
-          accs = sum8(v[j], accs);
+        for (int j = 0; j < U; j++) {
+          if constexpr (MFMA)
+            accm = mfma_16x16x32(v[j], ones, accm);
+          else
+            accs = sum8(v[j], accs);
+        }
       }
     }
     float total;
@@ -252,9 +260,9 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_block_kernel(const half8
       total = lane_group_sum<6>(accs);
     if (lane == 63) partial[wave] = total;
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (wg == 0 && lane == 0 && live) {
       float s = 0.0f;
-      for (int w = 0; w < WPB; w++) s += partial[w];
+      for (int w = 0; w < G; w++) s += partial[q * G + w];
       out[seg] = f16_bits(s);
     }
     __syncthreads();

@@ -236,29 +236,36 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t 
 }
 
 // ---------------------------------------------------------------------------------------
-// S >= 512: a block of waves shares each segment.  Per step the block takes WPB*U tiles,
-// wave w the U consecutive tiles starting at w*U; wave totals meet in LDS.
+// S >= 512: the waves of a block share segments.  A block owns segs_per_block consecutive
+// segments; groups of waves_per_seg waves take one segment each, blockDim / 64 /
+// waves_per_seg segments at a time (see seg_reduce_block_kernel).  Per step a group takes
+// waves_per_seg * U tiles, its wave w the U consecutive tiles starting at w * U; wave totals
+// meet in LDS.
 // ---------------------------------------------------------------------------------------
 template <int U, bool MFMA, bool NT>
 __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, size_t tiles_per_seg,
-                                                                    unsigned segs_per_block, unsigned xcd_run) {
+                                                                    unsigned segs_per_block, unsigned waves_per_seg, unsigned xcd_run) {
   __shared__ float wave_total[2][kMaxWaves];
   const int lane = lane_id();
   const int wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
+  const int G = (int)waves_per_seg, Q = WPB / G;  // waves per segment, segments in flight
+  const int q = wave / G, wg = wave % G;           // this wave's group, and its place in the group
   ScanOperands ops;
   if constexpr (MFMA) ops = make_scan_operands(lane);
   unsigned parity = 0;
   const size_t piece = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run);
-  for (unsigned sb = 0; sb < segs_per_block; sb++) {
-    const size_t seg = piece * segs_per_block + sb;
-    if (seg >= num_segments) break;  // block-uniform
+  for (unsigned sb = 0; sb < segs_per_block; sb += (unsigned)Q) {
+    if (piece * segs_per_block + sb >= num_segments) break;  // block-uniform
+    const size_t seg = piece * segs_per_block + sb + (unsigned)q;
+    const bool live = sb + (unsigned)q < segs_per_block && seg < num_segments;  // uniform over the group
     const size_t tile_base = seg * tiles_per_seg;
     size_t lim = (tile_base + tiles_per_seg) * kTileChunks;
     if (lim > n_chunks) lim = n_chunks;
+    if (!live) lim = 0;  // a group without a segment loads and stores nothing
     float block_carry = 0.0f;
-    for (size_t step0 = 0; step0 < tiles_per_seg; step0 += (size_t)WPB * U) {
-      const size_t t0 = step0 + (size_t)wave * U;  // first tile of this wave (may lie past the segment)
+    for (size_t step0 = 0; step0 < tiles_per_seg; step0 += (size_t)G * U) {
+      const size_t t0 = step0 + (size_t)wg * U;  // first tile of this wave (may lie past the segment)
       half8_t v[U];
       load_tiles<U, NT>(v, in, (tile_base + t0) * kTileChunks, t0 < tiles_per_seg ? lim : 0, lane);
       // pass 1: this wave's total
@@ -269,9 +276,9 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
       if (lane == 63) wave_total[parity][wave] = acc;
       __syncthreads();
       float carry = block_carry, all = 0.0f;
-      for (int w = 0; w < WPB; w++) {
-        const float x = wave_total[parity][w];
-        if (w < wave) carry += x;
+      for (int w = 0; w < G; w++) {
+        const float x = wave_total[parity][q * G + w];
+        if (w < wg) carry += x;
         all += x;
       }
       block_carry += all;
@@ -284,7 +291,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
         carry += tile_total;
       }
     }
-    if (totals != nullptr && threadIdx.x == 0) totals[seg] = f16_bits(block_carry);
+    if (totals != nullptr && wg == 0 && lane == 0 && live) totals[seg] = f16_bits(block_carry);
   }
 }
 

@@ -84,6 +84,10 @@ CASES = [  # (segment size, variants, (tiles per wave, waves per block) list, se
     (512, (V_WAVE, V_MFMA_16N, V_BLOCK, V_MFMA_256N_BLOCK), ((2, 1),), (9,)),
     (2048, (V_WAVE, V_MFMA_256N, V_BLOCK, V_MFMA_16N_BLOCK, V_AUTO), ((2, 2), (8, 1)), (5,)),
     (8192, (V_WAVE, V_MFMA_16N, V_MFMA_256N_BLOCK), ((4, 2),), (3,)),
+    # blocks with more waves (and tiles per wave) than a segment has tiles: groups of waves take a segment each
+    (512, (V_BLOCK, V_MFMA_256N_BLOCK, V_MFMA_16N_BLOCK), ((4, 4), (1, 16), (2, 2)), (9, 37)),
+    (1024, (V_BLOCK, V_MFMA_16N_BLOCK), ((1, 8), (4, 4)), (7,)),
+    (2048, (V_MFMA_256N_BLOCK,), ((1, 16), (8, 2)), (5,)),
 ]
 
 
