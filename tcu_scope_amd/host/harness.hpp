@@ -95,7 +95,9 @@ void run_seg_scan(benchmark::State &state, int variant, int tiles_per_wave, int 
 // and step, WARPS_PER_BLOCK): their product, capped at what a block of this build holds in registers (8 tiles of 512
 // halves per wave); the reference's kernels loop over larger values, these do not need to
 inline size_t single_pass_partition(size_t segment_size, int waves_per_block) {
-  const size_t want = segment_size * (size_t)waves_per_block, most = (size_t)waves_per_block * 8 * 512;
+  // a wave takes whole 512-half tiles: the reference's SEGMENT_SIZE = 256 instances run one tile per wave
+  const size_t per_wave = segment_size < 512 ? 512 : segment_size;
+  const size_t want = per_wave * (size_t)waves_per_block, most = (size_t)waves_per_block * 8 * 512;
   return want < most ? want : most;
 }
 void run_full_reduce(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);

@@ -71,6 +71,9 @@ template <class Launch>
 void timed_loop(benchmark::State &state, Launch launch) {
   EventPair ev;
   size_t it = 0;
+  // one untimed call first, as the harness gives the hand-written kernels: the first launch out of a code object loads it
+  launch(it++);
+  PRINT_IF_ERROR(hipDeviceSynchronize());
   for (auto _ : state) {
     ev.start();
     launch(it++);
