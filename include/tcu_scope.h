@@ -75,7 +75,8 @@ typedef enum {
   TCU_FULL_AUTO = 0,
   TCU_FULL_SINGLE_PASS = 1, /* one kernel: published partials added by the grid's last blocks (reduce), decoupled look-back (scan);
                                replaces reference *_ATOMIC_W_BLOCK_SYNC / _ATOMIC_BALLOT / _CG */
-  TCU_FULL_MULTI_KERNEL = 2, /* reference "2 kernels" (reduce) / "3 kernels" (scan) sequences */
+  TCU_FULL_MULTI_KERNEL = 2, /* reference "2 kernels" (reduce) / "3 kernels" (scan) sequences; ask for the workspace size, it
+                                is not a fixed number of bytes per segment */
   TCU_FULL_MFMA = 0x100     /* flag, OR-ed onto a strategy: the single-pass kernels add (reduce: D += A * ones) and scan
                                (U * X + carry) on the matrix unit, as the reference's *_CG / *_ATOMIC_* kernels do on
                                WMMA fragments; without it the DPP flavour runs.  AUTO | MFMA runs SINGLE_PASS | MFMA */
@@ -120,6 +121,9 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *   "compute_units"   blocks of the big-tile GEMM kernel the device runs at a time (set by tcu_init; for tests)
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
+ *   "many_totals"     default 65536: TCU_FULL_MULTI_KERNEL adds (reduce) or scans (scan) the per-segment totals with one
+ *                     block below this many segments, and with the two-launch partition sums / the single-pass scan
+ *                     (whose own workspace then follows the totals) from there on
  *   "xcd_run"         -1/0/C, default -1: consecutive blocks of a launch run on different XCDs (block b on XCD
  *                     b % 8); with C > 0 the segmented kernels renumber their blocks inside groups of 8 * C so that
  *                     every XCD works on C consecutive pieces of the array (a piece = what one block takes) while

@@ -44,6 +44,7 @@ struct Options {
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
   int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
   int gemm_split_tail = 1;     // spread the K steps of the tiles of a last, partly filled round of the GEMM grid over all compute units: 0 never, 1 where it pays, 2 always
+  int many_totals = 65536;     // multi-kernel sequences: from this many per-segment totals on, the step over the totals is itself a multi-block launch
   int xcd_run = -1;            // consecutive pieces of work per XCD (xcd_run_piece): -1 = the measured value for the size, 0 = none, C > 0 = C
   unsigned lookback_poll_limit = kDefaultPollLimit;  // polls of an unpublished value before a single-pass kernel gives up (results become NaN)
   unsigned test_mute_partition = 0;                  // tests only: partition test_mute_partition - 1 of a single-pass kernel publishes nothing
@@ -70,6 +71,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
   else if (n == "compute_units") o.compute_units = value < 1 ? 1 : value;
   else if (n == "xcd_run") o.xcd_run = value < 0 ? -1 : value;
+  else if (n == "many_totals") o.many_totals = value < 1 ? 65536 : value;
   else if (n == "lookback_poll_limit") o.lookback_poll_limit = value < 0 ? kDefaultPollLimit : (unsigned)value;
   else if (n == "test_mute_partition") o.test_mute_partition = value < 0 ? 0u : (unsigned)value;
   else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
@@ -649,7 +651,7 @@ inline int seg_scan_offsets_dispatch(const void *d_in, void *d_out, size_t num_s
   return seg_scan_offsets_typed(in, out, num_segments, static_cast<const int64_t *>(d_begin), static_cast<const int64_t *>(d_end), expected, stream);
 }
 
-inline int add_partial_sums_dispatch(void *d_out, const void *d_ps, size_t num_segments, size_t segment_size, void *stream) {
+inline int add_partial_sums_dispatch(void *d_out, const void *d_ps, size_t num_segments, size_t segment_size, void *stream, bool shifted = false) {
   if (segment_size == 0) return fail(TCU_ERR_INVALID_ARG, "tcu_add_partial_sums_f16: segment_size must be positive");
   if (num_segments == 0) return TCU_OK;
   if (!d_out || !d_ps) return fail(TCU_ERR_INVALID_ARG, "tcu_add_partial_sums_f16: null device pointer");
@@ -658,11 +660,11 @@ inline int add_partial_sums_dispatch(void *d_out, const void *d_ps, size_t num_s
     const size_t n_chunks = n / 8;
     const size_t grid = (n_chunks + 255) / 256;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_add_partial_sums_f16: grid exceeds the launch limit");
-    launch(add_partial_sums_kernel, (unsigned)grid, 256u, stream, static_cast<uint4_t *>(d_out), static_cast<const uint16_t *>(d_ps), n_chunks, ilog2(segment_size) - 3);
+    launch(add_partial_sums_kernel, (unsigned)grid, 256u, stream, static_cast<uint4_t *>(d_out), static_cast<const uint16_t *>(d_ps), n_chunks, ilog2(segment_size) - 3, shifted ? 1 : 0);
   } else {
     const size_t grid = (n + 255) / 256;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_add_partial_sums_f16: grid exceeds the launch limit");
-    launch(add_partial_sums_generic_kernel, (unsigned)grid, 256u, stream, static_cast<uint16_t *>(d_out), static_cast<const uint16_t *>(d_ps), n, segment_size);
+    launch(add_partial_sums_generic_kernel, (unsigned)grid, 256u, stream, static_cast<uint16_t *>(d_out), static_cast<const uint16_t *>(d_ps), n, segment_size, shifted ? 1 : 0);
   }
   return TCU_OK;
 }
@@ -748,7 +750,14 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
   if (!is_pow2(S) || S < 16) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment_size must be a power of two >= 16");
   if (n % S != 0) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": num_elements must be a multiple of segment_size");
   const size_t nseg = n / S;
-  const size_t need = round_up(2 * (nseg ? nseg : 1), kWorkspaceAlign);
+  // The second step (the reference calls cub::DeviceReduce::Sum on the totals, src/reduction/wmma_2kers.cu:63-88): one block adds
+  // fewer than `many_totals` totals (option, 65536); beyond that the totals go through the two-launch partition sums, whose partials lie behind them.
+  const size_t totals_bytes = round_up(2 * (nseg ? nseg : 1), kWorkspaceAlign);
+  const bool nested = nseg >= (size_t)options().many_totals;
+  size_t nested_bytes = 0;
+  if (nested)
+    if (int rc = full_reduce_dispatch(nullptr, nullptr, nseg, nullptr, &nested_bytes, TCU_FULL_AUTO, 0, 0, nullptr)) return rc;
+  const size_t need = totals_bytes + nested_bytes;
   if (!d_ws) {
     *ws_bytes = need;
     return TCU_OK;
@@ -756,6 +765,7 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
   if (*ws_bytes < need) return fail(TCU_ERR_WORKSPACE, std::string(what) + ": workspace too small");
   if (!d_out || (n && !d_in)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
   if (int rc = seg_reduce_dispatch(d_in, d_ws, nseg, S, S == 16 ? TCU_VARIANT_MFMA_16 : TCU_VARIANT_MFMA_16N, 0, waves_per_block, stream)) return rc;  // the reference's sequence is built on its WMMA kernels
+  if (nested) return full_reduce_dispatch(d_ws, d_out, nseg, static_cast<char *>(d_ws) + totals_bytes, &nested_bytes, TCU_FULL_AUTO, 0, 0, stream);
   launch(sum_f16_kernel, 1u, 1024u, stream, static_cast<const uint16_t *>(d_ws), static_cast<uint16_t *>(d_out), nseg);
   return TCU_OK;
 }
@@ -814,7 +824,15 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
   if (!is_pow2(S) || S < 256) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": segment_size must be a power-of-two multiple of 256");
   if (n % S != 0) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": num_elements must be a multiple of segment_size");
   const size_t nseg = n / S;
-  const size_t need = round_up(2 * (nseg ? nseg : 1), kWorkspaceAlign);
+  // The step in the middle (the reference calls cub::DeviceScan::ExclusiveSum on the totals, src/prefixsum/wmma_3kers.cu:60-82):
+  // one block walks fewer than `many_totals` totals (option, 65536); beyond that the totals are scanned in place by the single-pass kernel
+  // (inclusive sums; the third kernel then reads them one segment back), which needs its descriptors behind the totals.
+  const size_t totals_bytes = round_up(2 * (nseg ? nseg : 1), kWorkspaceAlign);
+  const bool nested = nseg >= (size_t)options().many_totals && nseg % 8 == 0;
+  size_t nested_bytes = 0;
+  if (nested)
+    if (int rc = full_scan_dispatch(nullptr, nullptr, nseg, nullptr, &nested_bytes, TCU_FULL_AUTO, 0, 0, nullptr)) return rc;
+  const size_t need = totals_bytes + nested_bytes;
   if (!d_ws) {
     *ws_bytes = need;
     return TCU_OK;
@@ -823,6 +841,10 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
   if (!n) return TCU_OK;
   if (!d_in || !d_out) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
   if (int rc = seg_scan_dispatch(d_in, d_out, d_ws, nseg, S, TCU_VARIANT_MFMA_256N, 0, waves_per_block, stream)) return rc;
+  if (nested) {
+    if (int rc = full_scan_dispatch(d_ws, d_ws, nseg, static_cast<char *>(d_ws) + totals_bytes, &nested_bytes, TCU_FULL_AUTO, 0, 0, stream)) return rc;
+    return add_partial_sums_dispatch(d_out, d_ws, nseg, S, stream, true);
+  }
   launch(exclusive_scan_f16_kernel, 1u, 1024u, stream, static_cast<uint16_t *>(d_ws), nseg);
   return add_partial_sums_dispatch(d_out, d_ws, nseg, S, stream);
 }

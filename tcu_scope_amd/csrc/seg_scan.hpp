@@ -315,21 +315,27 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_generic_kernel(const uint1
   if (totals != nullptr && lane == 0) totals[seg] = f16_bits(carry);
 }
 
-// out[s*S + i] += partial_sums[s], one fp16 addition per element (8 per lane per step)
-__global__ __launch_bounds__(256) void add_partial_sums_kernel(uint4_t *out, const uint16_t *partial_sums, size_t n_chunks, int seg_log2_chunks) {
+// out[s*S + i] += partial_sums[s], one fp16 addition per element (8 per lane per step).  With `shifted` the array
+// holds inclusive sums and segment s takes partial_sums[s - 1] (segment 0 nothing): the exclusive sums without a
+// pass that shifts them.
+__global__ __launch_bounds__(256) void add_partial_sums_kernel(uint4_t *out, const uint16_t *partial_sums, size_t n_chunks, int seg_log2_chunks, int shifted) {
   const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= n_chunks) return;
-  const float ps = (float)__builtin_bit_cast(half_t, partial_sums[c >> seg_log2_chunks]);
+  const size_t seg = c >> seg_log2_chunks;
+  if (shifted && seg == 0) return;
+  const float ps = (float)__builtin_bit_cast(half_t, partial_sums[shifted ? seg - 1 : seg]);
   uint4_t raw = out[c];
   half8_t v = __builtin_bit_cast(half8_t, raw);
   uint4_t r = {pack_f16x2((float)v[0] + ps, (float)v[1] + ps), pack_f16x2((float)v[2] + ps, (float)v[3] + ps), pack_f16x2((float)v[4] + ps, (float)v[5] + ps),
                pack_f16x2((float)v[6] + ps, (float)v[7] + ps)};
   out[c] = r;
 }
-__global__ __launch_bounds__(256) void add_partial_sums_generic_kernel(uint16_t *out, const uint16_t *partial_sums, size_t n, size_t segment_size) {
+__global__ __launch_bounds__(256) void add_partial_sums_generic_kernel(uint16_t *out, const uint16_t *partial_sums, size_t n, size_t segment_size, int shifted) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const float ps = (float)__builtin_bit_cast(half_t, partial_sums[i / segment_size]);
+  const size_t seg = i / segment_size;
+  if (shifted && seg == 0) return;
+  const float ps = (float)__builtin_bit_cast(half_t, partial_sums[shifted ? seg - 1 : seg]);
   out[i] = f16_bits((float)__builtin_bit_cast(half_t, out[i]) + ps);
 }
 

@@ -257,6 +257,31 @@ def test_full_array_kernels(emu, oracle):
                     assert oracle.check_f16(out, ref, n)[0] == 0, (op, n, strategy, seg, wpb)
 
 
+def test_multi_kernel_sequences_with_many_totals(emu, oracle):
+    """From `many_totals` per-segment totals on (65536; lowered here), the middle step of the reference's 2- and
+    3-kernel sequences runs the partition sums / the single-pass scan on the totals instead of one block."""
+    sz = ctypes.c_size_t
+    try:
+        assert emu.emu_set_option(b"many_totals", 64) == 0
+        for op, fn, seg, nseg in (("reduce", emu.emu_full_reduce_f16, 16, 4096 + 8), ("reduce", emu.emu_full_reduce_f16, 16, 64 + 3), ("scan", emu.emu_full_scan_f16, 256, 64 + 8),
+                                  ("scan", emu.emu_full_scan_f16, 256, 64 + 9), ("scan", emu.emu_full_scan_f16, 256, 63)):
+            n = seg * nseg
+            x = oracle.generate_f16(n, 9, oracle.DIST_GRID)
+            w64 = oracle.seg_scan_f64(x, 1, n)
+            xi = copy_in(x)
+            need = sz(0)
+            assert fn(xi.ctypes.data, None, n, None, ctypes.byref(need), 2, seg, 0) == 0
+            nested = nseg >= 64 and (op == "reduce" or nseg % 8 == 0)
+            assert (need.value > 2 * nseg + 256) == nested  # the totals, and the nested call's own workspace behind them
+            ws = aligned(need.value, np.uint8, 0xAB)
+            out = aligned(n if op == "scan" else 1, np.uint16, 0xFFFF)
+            assert fn(xi.ctypes.data, out.ctypes.data, n, ws.ctypes.data, ctypes.byref(need), 2, seg, 0) == 0, emu.emu_last_error()
+            ref = w64 if op == "scan" else w64[-1:]
+            assert oracle.check_f16(out, ref, n)[0] == 0, (op, seg, nseg)
+    finally:
+        assert emu.emu_set_option(b"many_totals", 0) == 0
+
+
 def test_a_wait_that_expires_gives_nan(emu, oracle):
     """A partition that publishes nothing (test option) with a small poll limit: the scan is right up to and
     including that partition and NaN after it, the reduction's result is NaN, every kernel returns."""
