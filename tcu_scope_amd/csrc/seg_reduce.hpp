@@ -258,6 +258,10 @@ __global__ __launch_bounds__(kMaxBlock) void seg_reduce_block_kernel(const half8
       total = add_xor32(add_xor16((accm[0] + accm[1]) + (accm[2] + accm[3])));
     else
       total = lane_group_sum<6>(accs);
+    if (G == 1) {  // block-uniform: every wave has a segment of its own, nothing to exchange
+      if (lane == 63 && live) out[seg] = f16_bits(total);
+      continue;
+    }
     if (lane == 63) partial[wave] = total;
     __syncthreads();
     if (wg == 0 && lane == 0 && live) {

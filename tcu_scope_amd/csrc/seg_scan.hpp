@@ -273,16 +273,20 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
 #pragma unroll
       for (int j = 0; j < U; j++) acc = sum8(v[j], acc);
       acc = lane_group_sum<6>(acc);
-      if (lane == 63) wave_total[parity][wave] = acc;
-      __syncthreads();
       float carry = block_carry, all = 0.0f;
-      for (int w = 0; w < G; w++) {
-        const float x = wave_total[parity][q * G + w];
-        if (w < wg) carry += x;
-        all += x;
+      if (G == 1) {  // block-uniform: every wave has a segment of its own, nothing to exchange
+        all = readlane(acc, 63);
+      } else {
+        if (lane == 63) wave_total[parity][wave] = acc;
+        __syncthreads();
+        for (int w = 0; w < G; w++) {
+          const float x = wave_total[parity][q * G + w];
+          if (w < wg) carry += x;
+          all += x;
+        }
+        parity ^= 1u;
       }
       block_carry += all;
-      parity ^= 1u;
       // pass 2: scan the tiles held in registers
 #pragma unroll
       for (int j = 0; j < U; j++) {
