@@ -170,14 +170,14 @@ inline Plan auto_plan_reduce(size_t S) {
   return {true, 1, 8, 0};
 }
 inline Plan auto_plan_scan(size_t S) {
-  if (S <= 512) return {false, 2, 1, 256};
-  if (S == 1024) return {false, 1, 1, 64};
+  if (S <= 512) return {false, 2, 1, 512};
+  if (S == 1024) return {false, 2, 2, 256};
   if (S == 2048) return {true, 2, 2, 256};
   if (S == 4096) return {true, 2, 4, 128};
-  if (S == 8192) return {true, 2, 8, 0};
-  if (S == 16384) return {true, 4, 8, 8};
-  if (S == 32768) return {true, 8, 8, 4};
-  return {true, 8, 16, 0};
+  if (S == 8192) return {true, 2, 8, 128};
+  if (S == 16384) return {true, 4, 8, 32};
+  if (S == 32768) return {true, 8, 8, 16};
+  return {true, 8, 16, 8};
 }
 
 inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || v == TCU_VARIANT_MFMA_256N_BLOCK || v == TCU_VARIANT_BLOCK_LDS; }

@@ -26,6 +26,12 @@
 
 namespace tcu {
 
+// The look-back scans keep every store non-temporal: alternating the policy by tile as the segmented scans do
+// (kTileStoreNT) made them slower (TCU_FULL_AUTO 2^28 / 2^30: 201 / 762 us against 213-225 / 792-864 us with one
+// store in two, three or four through the cache; events around the call).
+template <bool NT, int J>
+constexpr bool kFullScanStoreNT = NT;
+
 constexpr unsigned long long kFlagAggregate = 1ull << 32;
 constexpr unsigned long long kFlagPrefix = 2ull << 32;
 
@@ -246,12 +252,12 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   __syncthreads();
   float carry = s_prefix;
   for (int w = 0; w < wave; w++) carry += wave_total[w];
-#pragma unroll
-  for (int j = 0; j < U; j++) {
+  static_for<U>([&](auto J) {
+    constexpr int j = decltype(J)::value;
     float tile_total;
-    scan_tile<6, MFMA, NT>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    scan_tile<6, MFMA, kFullScanStoreNT<NT, j>>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
     carry += tile_total;
-  }
+  });
 }
 
 // The look-back scan with more bytes in flight per wave slot.  A block of full_scan_kernel
@@ -320,19 +326,19 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t 
   __syncthreads();
   float carry = s_prefix;
   for (int w = 0; w < wave; w++) carry += wave_total[w];
-#pragma unroll
-  for (int j = 0; j < U; j++) {
+  static_for<U>([&](auto J) {
+    constexpr int j = decltype(J)::value;
     float tile_total;
-    scan_tile<6, false, NT>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    scan_tile<6, false, kFullScanStoreNT<NT, j>>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
     carry += tile_total;
-  }
-#pragma unroll
-  for (int j = 0; j < ULDS; j++) {
+  });
+  static_for<ULDS>([&](auto J) {
+    constexpr int j = decltype(J)::value;
     float tile_total;
     const half8_t h = *reinterpret_cast<const half8_t *>(mine + j * kTileHalves + lane * 8);
-    scan_tile<6, false, NT>(h, carry, ops, lane, out, (t0 + U + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    scan_tile<6, false, kFullScanStoreNT<NT, U + j>>(h, carry, ops, lane, out, (t0 + U + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
     carry += tile_total;
-  }
+  });
 }
 
 // Segments far larger than one block's reach, first level: block b adds its partition

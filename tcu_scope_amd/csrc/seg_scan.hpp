@@ -218,12 +218,12 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t 
     const size_t t_it = tile0 + (size_t)it * U;
     half8_t v[U];
     load_tiles<U, NT>(v, in, t_it * kTileChunks, n_chunks, lane);
-#pragma unroll
-    for (int j = 0; j < U; j++) {
+    static_for<U>([&](auto J) {
+      constexpr int j = decltype(J)::value;
       const size_t t = t_it + j;
       if (LPS_LOG2 < 6 || (t & tmask) == 0) carry = 0.0f;
       float tile_total;
-      scan_tile<LPS_LOG2, MFMA, NT>(v[j], carry, ops, lane, out, t * kTileChunks, n_chunks, totals, t * SEGS_PER_TILE, num_segments, &tile_total);
+      scan_tile<LPS_LOG2, MFMA, kTileStoreNT<NT, j>>(v[j], carry, ops, lane, out, t * kTileChunks, n_chunks, totals, t * SEGS_PER_TILE, num_segments, &tile_total);
       if constexpr (LPS_LOG2 == 6) {
         carry += tile_total;
         if (totals != nullptr && ((t + 1) & tmask) == 0) {
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t 
           if (lane == 0 && s < num_segments) totals[s] = f16_bits(carry);
         }
       }
-    }
+    });
   }
 }
 
@@ -288,12 +288,12 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
       }
       block_carry += all;
       // pass 2: scan the tiles held in registers
-#pragma unroll
-      for (int j = 0; j < U; j++) {
+      static_for<U>([&](auto J) {
+        constexpr int j = decltype(J)::value;
         float tile_total;
-        scan_tile<6, MFMA, NT>(v[j], carry, ops, lane, out, (tile_base + t0 + j) * kTileChunks, t0 + j < tiles_per_seg ? lim : 0, nullptr, 0, 0, &tile_total);
+        scan_tile<6, MFMA, kTileStoreNT<NT, j>>(v[j], carry, ops, lane, out, (tile_base + t0 + j) * kTileChunks, t0 + j < tiles_per_seg ? lim : 0, nullptr, 0, 0, &tile_total);
         carry += tile_total;
-      }
+      });
     }
     if (totals != nullptr && wg == 0 && lane == 0 && live) totals[seg] = f16_bits(block_carry);
   }

@@ -67,11 +67,11 @@ __global__ __launch_bounds__(kMaxBlock) void stream_probe_kernel(uint4_t *dst, c
     // keeps the loads alive; one word per wave only when the data says so (never for finite sums)
     if (acc == 123456.0f) reinterpret_cast<float *>(dst)[gw] = acc;
   } else {
-#pragma unroll
-    for (int j = 0; j < U; j++) {
+    static_for<U>([&](auto J) {
+      constexpr int j = decltype(J)::value;
       const size_t c = chunk0 + (size_t)j * kTileChunks + lane;
-      if (c < n_chunks) store_chunk<NT>(dst + c, __builtin_bit_cast(uint4_t, v[j]));
-    }
+      if (c < n_chunks) store_chunk<kTileStoreNT<NT, j>>(dst + c, __builtin_bit_cast(uint4_t, v[j]));
+    });
   }
 }
 

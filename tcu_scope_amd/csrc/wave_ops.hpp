@@ -138,6 +138,30 @@ TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
     *p = v;
 }
 
+// Streaming kernels that write as much as they read (the scans) alternate their stores: tile 0, 2, ... of a wave go
+// out non-temporal, tile 1, 3, ... through the cache, while all loads stay non-temporal.  Measured on the segmented
+// scan of 2^28 halves (HIP events around the call, every assignment of the two policies to the 2 or 4 tiles of a wave):
+// all stores non-temporal 171 us (2 tiles per wave) / 176 us (4), all through the cache 173 / 188, every other one
+// 153-156 / 162, three of four through the cache 188; alternating the LOADS instead (stores non-temporal) 155 / 170,
+// alternating both 172 / 180.  The two kinds of store drain through different paths, and using both is worth 9 %.
+// Kernels that only read gain nothing from mixing their loads (segmented reduction: 72-82 us with all loads
+// non-temporal, 73-104 us with every other one through the cache), and the look-back scans lose (full_array.hpp).
+template <bool NT, int J>
+constexpr bool kTileStoreNT = NT && (J % 2 == 0);
+
+// f(Int<0>{}), f(Int<1>{}), ..., f(Int<N-1>{}): a loop whose index is a compile-time constant in the body
+template <int V>
+struct Int {
+  static constexpr int value = V;
+};
+template <int N, int J = 0, class F>
+TCU_DEVICE void static_for(F &&f) {
+  if constexpr (J < N) {
+    f(Int<J>{});
+    static_for<N, J + 1>(f);
+  }
+}
+
 // Global -> LDS without a register round trip: lane l of the wave moves the 16 bytes at its
 // own global address `src` to lds_base + 16 * l (lds_base is the same for the whole wave).
 // Written as inline assembly on purpose: for the compiler's own form of this instruction the

@@ -365,6 +365,19 @@ template <bool NT>
 inline void store_chunk(uint4_t *p, uint4_t v) {
   *p = v;
 }
+template <bool NT, int J>
+constexpr bool kTileStoreNT = NT && (J % 2 == 0);
+template <int V>
+struct Int {
+  static constexpr int value = V;
+};
+template <int N, int J = 0, class F>
+inline void static_for(F &&f) {
+  if constexpr (J < N) {
+    f(Int<J>{});
+    static_for<N, J + 1>(f);
+  }
+}
 inline void sched_fence() {}
 // lanes run one after another here, so the transfer is a plain copy and nothing is in flight
 using lds_addr_t = uintptr_t;
