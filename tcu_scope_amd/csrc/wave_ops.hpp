@@ -149,6 +149,20 @@ TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
 template <bool NT, int J>
 constexpr bool kTileStoreNT = NT && (J % 2 == 0);
 
+// The same alternation where a tile's place in its wave is not known at compile time: the odd 1 KiB blocks of the
+// output go through the cache.  Written as assembly because the compiler merges two stores that differ only in
+// their cache policy into one store without the hint.
+template <bool NT>
+TCU_DEVICE void store_chunk_alternating(uint4_t *p, uint4_t v) {
+  if constexpr (!(NT && TCU_STORE_NT)) {
+    *p = v;
+  } else if ((reinterpret_cast<uintptr_t>(p) >> 10) & 1u) {
+    asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(p), "v"(v) : "memory");
+  } else {
+    asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(p), "v"(v) : "memory");
+  }
+}
+
 // f(Int<0>{}), f(Int<1>{}), ..., f(Int<N-1>{}): a loop whose index is a compile-time constant in the body
 template <int V>
 struct Int {

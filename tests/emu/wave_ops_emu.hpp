@@ -365,6 +365,10 @@ template <bool NT>
 inline void store_chunk(uint4_t *p, uint4_t v) {
   *p = v;
 }
+template <bool NT>
+inline void store_chunk_alternating(uint4_t *p, uint4_t v) {
+  *p = v;
+}
 template <bool NT, int J>
 constexpr bool kTileStoreNT = NT && (J % 2 == 0);
 template <int V>
