@@ -328,11 +328,10 @@ __global__ __launch_bounds__(256) void add_partial_sums_kernel(uint4_t *out, con
   const size_t seg = c >> seg_log2_chunks;
   if (shifted && seg == 0) return;
   const float ps = (float)__builtin_bit_cast(half_t, partial_sums[shifted ? seg - 1 : seg]);
-  uint4_t raw = out[c];
-  half8_t v = __builtin_bit_cast(half8_t, raw);
+  half8_t v = load_chunk<true>(reinterpret_cast<const half8_t *>(out + c));
   uint4_t r = {pack_f16x2((float)v[0] + ps, (float)v[1] + ps), pack_f16x2((float)v[2] + ps, (float)v[3] + ps), pack_f16x2((float)v[4] + ps, (float)v[5] + ps),
                pack_f16x2((float)v[6] + ps, (float)v[7] + ps)};
-  out[c] = r;
+  store_chunk_alternating<true>(out + c, r);
 }
 __global__ __launch_bounds__(256) void add_partial_sums_generic_kernel(uint16_t *out, const uint16_t *partial_sums, size_t n, size_t segment_size, int shifted) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
