@@ -166,7 +166,9 @@ inline Plan auto_plan_reduce(size_t S) {
   if (S == 4096) return {true, 2, 4, 64};
   if (S == 8192) return {true, 2, 8, 64};
   if (S == 16384) return {true, 2, 8, 64};
-  if (S >= 262144) return {true, 2, 8, 0};
+  if (S == 65536 || S == 131072) return {true, 2, 16, 32};
+  if (S == 262144) return {true, 4, 8, 0};
+  if (S > 262144) return {true, 2, 8, 0};
   return {true, 1, 8, 0};
 }
 inline Plan auto_plan_scan(size_t S) {
@@ -177,7 +179,9 @@ inline Plan auto_plan_scan(size_t S) {
   if (S == 8192) return {true, 2, 8, 128};
   if (S == 16384) return {true, 4, 8, 32};
   if (S == 32768) return {true, 8, 8, 16};
-  return {true, 8, 16, 8};
+  if (S == 65536 || S == 131072) return {true, 4, 16, 32};
+  if (S == 262144) return {true, 4, 16, 0};
+  return {true, 8, 16, 0};
 }
 
 inline bool is_block_variant(int v) { return v == TCU_VARIANT_MFMA_16N_BLOCK || v == TCU_VARIANT_MFMA_256N_BLOCK || v == TCU_VARIANT_BLOCK_LDS; }
