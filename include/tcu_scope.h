@@ -119,6 +119,9 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
  *                     in a fixed order by a second kernel): never, where it pays (round at most a third full,
  *                     K >= 4096), or whenever there is such a round
  *   "compute_units"   blocks of the big-tile GEMM kernel the device runs at a time (set by tcu_init; for tests)
+ *   "gemm_staged_epilogue" 0/1, default 1: the big-tile GEMM kernel on 16x16x32 MFMAs turns its outputs through LDS and
+ *                     writes (and reads C in) whole rows of a wave's 128 columns, 16 bytes per lane, where C and D are
+ *                     16-byte aligned; 0 = straight from the accumulator layout (64 / 32 bytes of 16 rows per store)
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
  *   "many_totals"     default 65536: TCU_FULL_MULTI_KERNEL adds (reduce) or scans (scan) the per-segment totals with one

@@ -37,6 +37,7 @@ struct Options {
   bool static_order = false;
   int gemm_big_tiles = -1;     // 256 x 256 block tiles: 1 wherever M and N allow, 0 never, -1 where there are at least 128 of them
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
+  bool gemm_staged_epilogue = true;   // 16x16x32 big-tile kernel: turn the outputs through LDS so that rows are written whole (C and D 16-byte aligned)
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
@@ -68,6 +69,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_strip_lds") o.gemv_strip_lds = value != 0;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
+  else if (n == "gemm_staged_epilogue") o.gemm_staged_epilogue = value != 0;
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
   else if (n == "compute_units") o.compute_units = value < 1 ? 1 : value;
   else if (n == "xcd_run") o.xcd_run = value < 0 ? -1 : value;
@@ -1045,6 +1047,10 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
       // the 16x16x32 kernel moves four adjacent outputs per access (16 bytes of fp32, 8 of fp16)
       const bool al4 = ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & (4 * sizeof(OUT) - 1)) == 0;
       if (direct_lds == 66 && K % 64 == 0 && al4) {
+        // the epilogue that turns the outputs through LDS moves 16 bytes per lane: whole rows of a wave's 128 columns per store
+        // instead of 64 (fp32) / 32 (fp16) bytes of 16 rows (8192^3, alpha 1.1, beta 1.2 / 0, events around the call, same run:
+        // fp32 outputs 830-858 -> 794-809 / 774-789 -> 762 us, fp16 outputs 807 -> 757 / 776 -> 746 us; 4096^3 fp16 134-151 -> 121 / 126 -> 110)
+        const bool staged = options().gemm_staged_epilogue && ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & 15u) == 0;
         // the tiles of a last, sparsely filled round of the grid: their K steps are spread evenly over all compute
         // units, in runs of at least 8 steps.  The shares cost up to 2 x 256 KiB of fp32 per block written and read
         // back, which pays while the round is at most a third full and a tile takes long enough (8192^3 sizes, same
@@ -1059,13 +1065,19 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
           blocks = (total + run - 1) / run;
           float *ws = static_cast<float *>(stream_alloc(2 * blocks * (size_t)(kGemmBigBM * kGemmBigBN) * sizeof(float), stream));
           if (ws) {
-            launch(gemm_dlds_a3b2_m16_kernel<OUT>, (unsigned)(full + blocks), 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)full, (unsigned)run, ws);
+            if (staged)
+              launch(gemm_dlds_a3b2_m16_kernel<OUT, true>, (unsigned)(full + blocks), 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)full, (unsigned)run, ws);
+            else
+              launch(gemm_dlds_a3b2_m16_kernel<OUT, false>, (unsigned)(full + blocks), 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)full, (unsigned)run, ws);
             launch(gemm_split_fixup_kernel<OUT>, (unsigned)(tail * 64), 256u, stream, static_cast<const float *>(ws), c, d, M, N, K, alpha, beta, (unsigned)full, (unsigned)run);
             stream_free(ws, stream);
             return TCU_OK;
           }
         }
-        launch(gemm_dlds_a3b2_m16_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)grid, 1u, static_cast<float *>(nullptr));
+        if (staged)
+          launch(gemm_dlds_a3b2_m16_kernel<OUT, true>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)grid, 1u, static_cast<float *>(nullptr));
+        else
+          launch(gemm_dlds_a3b2_m16_kernel<OUT, false>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta, (unsigned)grid, 1u, static_cast<float *>(nullptr));
       }
       else if (direct_lds >= 65 && K % 64 == 0)
         launch(gemm_dlds_a3b2_kernel<OUT>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);

@@ -712,6 +712,74 @@ TCU_DEVICE void gemm_store_strip16(OUT *D, const OUT *C, size_t ldc, size_t row0
   }
 }
 
+// The same strip with every row of tiles turned through LDS first, so that global memory sees whole rows: a
+// row of eight tiles is 16 rows of 128 outputs; the lanes park alpha * acc in `stage` (two buffers of
+// kStageRowFloats * 16 floats per wave, rows padded by four floats), and read it back with consecutive lanes
+// along a row: 32 lanes x 4 fp32 outputs (512 bytes of one row, two rows per instruction) or 16 lanes x 8 fp16
+// outputs (256 bytes, four rows per instruction), where the direct form writes 64 / 32 bytes of 16 rows
+// per instruction.  C is read in the same shape, by the lane that writes the same elements of D.
+constexpr int kStageRowFloats = 128 + 4;
+constexpr int kStageWaveFloats = 2 * 16 * kStageRowFloats;
+template <typename OUT>
+TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8][8], int lane, float alpha, float beta, float *stage) {
+  constexpr int PER_LANE = sizeof(OUT) == 4 ? 4 : 8;   // outputs per lane and access (16 bytes)
+  constexpr int LANES_PER_ROW = 128 / PER_LANE;        // 32 or 16
+  constexpr int ROWS_PER_ACCESS = 64 / LANES_PER_ROW;  // 2 or 4
+  constexpr int ACCESSES = 16 / ROWS_PER_ACCESS;       // per row of tiles: 8 or 4
+  using word_t = typename std::conditional<sizeof(OUT) == 4, float4_t, uint4_t>::type;
+  const int wr = lane & 15, wq = lane >> 4;  // accumulator layout: row, group of four columns
+  const int rr = lane / LANES_PER_ROW, rc = (lane % LANES_PER_ROW) * PER_LANE;
+  const size_t at0 = (row0 + rr) * ldc + col0 + rc;  // access t of row of tiles i: at0 + (16 i + ROWS_PER_ACCESS t) * ldc
+  // the C values of a row of tiles are requested one row of tiles ahead, all at once (one wait per load would
+  // leave the epilogue bound by latency); C may be D: a lane reads only what it will itself write, rows later
+  word_t c[2][ACCESSES];
+  if (beta != 0.0f) {
+#pragma unroll
+    for (int t = 0; t < ACCESSES; t++) c[0][t] = __builtin_nontemporal_load(reinterpret_cast<const word_t *>(C + at0 + (size_t)(ROWS_PER_ACCESS * t) * ldc));
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    float *buf = stage + (i & 1) * (16 * kStageRowFloats);
+    if (beta != 0.0f && i + 1 < 8) {
+#pragma unroll
+      for (int t = 0; t < ACCESSES; t++) c[(i + 1) & 1][t] = __builtin_nontemporal_load(reinterpret_cast<const word_t *>(C + at0 + (size_t)(16 * (i + 1) + ROWS_PER_ACCESS * t) * ldc));
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) *reinterpret_cast<float4_t *>(buf + wr * kStageRowFloats + 16 * j + 4 * wq) = alpha * acc[i][j];
+    wave_lds_fence();
+#pragma unroll
+    for (int t = 0; t < ACCESSES; t++) {
+      const int r = t * ROWS_PER_ACCESS + rr;
+      word_t *d = reinterpret_cast<word_t *>(D + at0 + (size_t)(16 * i + ROWS_PER_ACCESS * t) * ldc);
+      float4_t v0 = *reinterpret_cast<const float4_t *>(buf + r * kStageRowFloats + rc);
+      if constexpr (sizeof(OUT) == 4) {
+        if (beta != 0.0f) v0 += beta * c[i & 1][t];
+        __builtin_nontemporal_store(v0, d);
+      } else {
+        float4_t v1 = *reinterpret_cast<const float4_t *>(buf + r * kStageRowFloats + rc + 4);
+        if (beta != 0.0f) {
+          const uint32_t w0 = c[i & 1][t][0], w1 = c[i & 1][t][1], w2 = c[i & 1][t][2], w3 = c[i & 1][t][3];  // scalars first: a bit cast straight from a vector element reads element 0
+          const half2_t c0 = __builtin_bit_cast(half2_t, w0), c1 = __builtin_bit_cast(half2_t, w1), c2 = __builtin_bit_cast(half2_t, w2), c3 = __builtin_bit_cast(half2_t, w3);
+          v0[0] += beta * (float)c0[0];
+          v0[1] += beta * (float)c0[1];
+          v0[2] += beta * (float)c1[0];
+          v0[3] += beta * (float)c1[1];
+          v1[0] += beta * (float)c2[0];
+          v1[1] += beta * (float)c2[1];
+          v1[2] += beta * (float)c3[0];
+          v1[3] += beta * (float)c3[1];
+        }
+        uint4_t o;
+        o[0] = pack_f16x2(v0[0], v0[1]);
+        o[1] = pack_f16x2(v0[2], v0[3]);
+        o[2] = pack_f16x2(v1[0], v1[1]);
+        o[3] = pack_f16x2(v1[2], v1[3]);
+        __builtin_nontemporal_store(o, d);
+      }
+    }
+  }
+}
+
 // gemm_dlds_a3b2_kernel on v_mfma_f32_16x16x32_f16: the same block tile, buffers and transfer
 // schedule, but a wave's 128 x 128 tile is 8 x 8 accumulators of 16 x 16 and a K step of 64 is
 // two substeps of 32, each 16 fragment reads for 64 MFMAs.  Per multiply-add this shape reads
@@ -724,7 +792,7 @@ TCU_DEVICE void gemm_store_strip16(OUT *D, const OUT *C, size_t ldc, size_t row0
 // One tile (or, with share != nullptr, the K steps step0 .. step0 + steps - 1 of one tile, whose raw fp32
 // accumulators go to `share` as a 256 x 256 row-major tile).  May be called several times by a block:
 // every wave waits for its own transfers before it leaves, and nothing reads LDS after the last barrier.
-template <typename OUT>
+template <typename OUT, bool STAGED>
 TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t N, size_t K, size_t tile_m, size_t tile_n, size_t step0, size_t steps,
                                    float *share, float alpha, float beta) {
   constexpr int BK = 64, ROWH = BK, CPR = 8, RPT = 8, RS = 1, SUB = 2, NA = 3, NB = 2;
@@ -823,10 +891,16 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
     cb = nb;
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
-  if (share != nullptr)
+  if (share != nullptr) {
     gemm_store_strip16<float>(share, nullptr, kGemmBigBN, wm * 128, wn * 128, acc, lane, 1.0f, 0.0f);
-  else
+  } else if constexpr (STAGED) {
+    block_barrier_lds_only();  // the other waves have read their last fragments: the A buffers can hold outputs now
+    static_assert(4 * kStageWaveFloats * sizeof(float) <= sizeof(lds_a), "staging area of four waves");
+    gemm_store_strip16_staged(D, C, N, tile_m * kGemmBigBM + wm * 128, tile_n * kGemmBigBN + wn * 128, acc, lane, alpha, beta, reinterpret_cast<float *>(&lds_a[0][0]) + wave * kStageWaveFloats);
+    block_barrier_lds_only();  // a block that goes on to another piece of work starts its transfers only after every wave has read its outputs back
+  } else {
     gemm_store_strip16(D, C, N, tile_m * kGemmBigBM + wm * 128, tile_n * kGemmBigBN + wn * 128, acc, lane, alpha, beta);
+  }
 }
 
 // Blocks 0 .. full_tiles-1 take one tile each.  With T tiles on a chip that runs `units` blocks at a
@@ -837,14 +911,14 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
 // the tail stores its raw accumulators for the two at ws + (2 j + 0 or 1) * 65536 floats, and
 // gemm_split_fixup_kernel adds the shares of a tile in a fixed order and applies alpha, beta and C.
 // full_tiles = grid size turns this off.
-template <typename OUT>
+template <typename OUT, bool STAGED = false>
 __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta,
                                                                  unsigned full_tiles, unsigned run, float *ws) {
   const size_t tiles_m = M / kGemmBigBM, tiles_n = N / kGemmBigBN, steps = K / 64;
   size_t tile_m, tile_n;
   if (blockIdx.x < full_tiles) {  // block-uniform
     gemm_tile_of_block(tiles_m, tiles_n, blockIdx.x, &tile_m, &tile_n);
-    gemm_a3b2_m16_tile(A, B, C, D, N, K, tile_m, tile_n, 0, steps, static_cast<float *>(nullptr), alpha, beta);
+    gemm_a3b2_m16_tile<OUT, STAGED>(A, B, C, D, N, K, tile_m, tile_n, 0, steps, static_cast<float *>(nullptr), alpha, beta);
     return;
   }
   const size_t j = blockIdx.x - full_tiles, total = (tiles_m * tiles_n - full_tiles) * steps;
@@ -854,7 +928,7 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_kernel(const half8_t *
     const size_t t = at / steps, k0 = at % steps;
     const size_t len = end - at < steps - k0 ? end - at : steps - k0;
     gemm_tile_of_block(tiles_m, tiles_n, full_tiles + t, &tile_m, &tile_n);
-    gemm_a3b2_m16_tile(A, B, C, D, N, K, tile_m, tile_n, k0, len, ws + (2 * j + part) * (size_t)(kGemmBigBM * kGemmBigBN), alpha, beta);
+    gemm_a3b2_m16_tile<OUT, STAGED>(A, B, C, D, N, K, tile_m, tile_n, k0, len, ws + (2 * j + part) * (size_t)(kGemmBigBM * kGemmBigBN), alpha, beta);
     at += len;
   }
 }

@@ -365,6 +365,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
     ref = oracle.gemm_f64(A, B, M, N, K, 1.5, 2.0, C0)
     try:
         assert emu.emu_set_option(b"gemm_big_tiles", 1) == 0  # one tile: the default would take the 128 x 128 kernel
+        assert emu.emu_set_option(b"gemm_staged_epilogue", 0) == 0  # outputs straight from the accumulator layout (default: through LDS, below)
         for direct_lds, bk64, depth in ((3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4), (66, 0, 4), (0, 0, 1), (0, 0, 2), (0, 0, 3), (0, 0, 4), (0, 1, 1), (0, 1, 2)):
             for name, val in ((b"gemm_direct_lds", direct_lds), (b"gemm_bk64", bk64), (b"gemm_depth", depth)):
                 assert emu.emu_set_option(name, val) == 0
@@ -374,6 +375,32 @@ def test_gemv_gemm_and_generator(emu, oracle):
             Dh = copy_in(C0.astype(np.float16).view(np.uint16))  # in place: C == D
             rc = emu.emu_gemm_f16_f16(Ai.ctypes.data, Bi.ctypes.data, Dh.ctypes.data, Dh.ctypes.data, M, N, K, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(Dh.reshape(M, N), ref.astype(np.float16).view(np.uint16)), (direct_lds, bk64, depth)
+        # the same kernel with the outputs turned through LDS (whole rows per store): two tiles, fp32 and fp16 outputs,
+        # in place and not, with and without C
+        assert emu.emu_set_option(b"gemm_direct_lds", -1) == 0 and emu.emu_set_option(b"gemm_staged_epilogue", 1) == 0
+        Mt, Nt, Kt = 512, 256, 128
+        At, Bt = oracle.generate_f16(Mt * Kt, 21, oracle.DIST_SMALLINT), oracle.generate_f16(Nt * Kt, 22, oracle.DIST_SMALLINT)
+        Ct = (np.arange(Mt * Nt) % 7).astype(np.float32)
+        Ati, Bti = copy_in(At), copy_in(Bt)
+        for beta in (2.0, 0.0):
+            reft = oracle.gemm_f64(At, Bt, Mt, Nt, Kt, 1.5, beta, Ct)
+            Cti = copy_in(Ct, np.float32)
+            Dt = aligned(Mt * Nt, np.float32, -777)
+            rc = emu.emu_gemm_f16_f32(Ati.ctypes.data, Bti.ctypes.data, Cti.ctypes.data, Dt.ctypes.data, Mt, Nt, Kt, 1.5, beta, V_BLOCK)
+            assert rc == 0 and np.array_equal(Dt.reshape(Mt, Nt).astype(np.float64), reft), ("staged fp32", beta)
+            rc = emu.emu_gemm_f16_f32(Ati.ctypes.data, Bti.ctypes.data, Cti.ctypes.data, Cti.ctypes.data, Mt, Nt, Kt, 1.5, beta, V_BLOCK)
+            assert rc == 0 and np.array_equal(Cti.reshape(Mt, Nt).astype(np.float64), reft), ("staged fp32 in place", beta)
+            Cht = copy_in(Ct.astype(np.float16).view(np.uint16))
+            Dht = aligned(Mt * Nt, np.uint16, 0x7e00)
+            rc = emu.emu_gemm_f16_f16(Ati.ctypes.data, Bti.ctypes.data, Cht.ctypes.data, Dht.ctypes.data, Mt, Nt, Kt, 1.5, beta, V_BLOCK)
+            assert rc == 0 and np.array_equal(Dht.reshape(Mt, Nt), reft.astype(np.float16).view(np.uint16)), ("staged fp16", beta)
+            rc = emu.emu_gemm_f16_f16(Ati.ctypes.data, Bti.ctypes.data, Cht.ctypes.data, Cht.ctypes.data, Mt, Nt, Kt, 1.5, beta, V_BLOCK)
+            assert rc == 0 and np.array_equal(Cht.reshape(Mt, Nt), reft.astype(np.float16).view(np.uint16)), ("staged fp16 in place", beta)
+            # fp16 outputs aligned to 8 bytes only: the direct epilogue takes over
+            Dho = aligned(Mt * Nt + 4, np.uint16, 0x7e00)
+            Cho = copy_in(Ct.astype(np.float16).view(np.uint16))
+            rc = emu.emu_gemm_f16_f16(Ati.ctypes.data, Bti.ctypes.data, Cho.ctypes.data, Dho.ctypes.data + 8, Mt, Nt, Kt, 1.5, beta, V_BLOCK)
+            assert rc == 0 and np.array_equal(Dho[4:].reshape(Mt, Nt), reft.astype(np.float16).view(np.uint16)) and np.all(Dho[:4] == 0x7e00), ("fp16 at 8 bytes", beta)
         # the K-split tail on a device of 4 units: 7 tiles -> the 48 K steps of the last 3 in 4 runs of 12, three of
         # which cross from one tile into the next; 9 tiles -> the last one in 2 runs (tile ids regrouped for 8 XCDs);
         # fp32 outputs in place, fp16 outputs with C
@@ -403,7 +430,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
             rc = emu.emu_gemm_f16_f32(A2i.ctypes.data, B2i.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, Ks, 1.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A2, B2, M, N, Ks, 1.5, 2.0, C0)), (direct_lds, Ks)
     finally:
-        for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1), (b"compute_units", 256), (b"gemm_split_tail", 1)):
+        for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1), (b"compute_units", 256), (b"gemm_split_tail", 1), (b"gemm_staged_epilogue", 1)):
             emu.emu_set_option(name, val)
 
 

@@ -261,28 +261,31 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
             ref0 = oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0)
             ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
-            shapes = [(0, bk64, depth) for bk64 in (0, 1) for depth in (1, 2, 3, 4)] + [(3, 0, 4), (4, 0, 4), (64, 0, 4), (65, 0, 4), (66, 0, 4)]
-            for direct_lds, bk64, depth in shapes:
+            # 66 (the default kernel) with its outputs turned through LDS (default) and straight from the accumulator layout
+            shapes = [(0, bk64, depth, 1) for bk64 in (0, 1) for depth in (1, 2, 3, 4)] + [(3, 0, 4, 1), (4, 0, 4, 1), (64, 0, 4, 1), (65, 0, 4, 1), (66, 0, 4, 1), (66, 0, 4, 0)]
+            for direct_lds, bk64, depth, staged in shapes:
+                tcu.set_option("gemm_staged_epilogue", staged)
                 tcu.set_option("gemm_direct_lds", direct_lds)
                 tcu.set_option("gemm_bk64", bk64)
                 tcu.set_option("gemm_depth", depth)
                 D = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS)
                 torch.cuda.synchronize()
-                assert np.array_equal(D.cpu().numpy().astype(np.float64), ref0), (K, direct_lds, bk64, depth)
+                assert np.array_equal(D.cpu().numpy().astype(np.float64), ref0), (K, direct_lds, bk64, depth, staged)
                 Cd = torch.from_numpy(C0.copy()).cuda().view(M, N)
                 D = tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd, variant=tcu.Variant.BLOCK_LDS)  # in place
                 torch.cuda.synchronize()
-                assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("in place", K, direct_lds, bk64, depth)
+                assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("in place", K, direct_lds, bk64, depth, staged)
                 # the same kernels with fp16 C and D, out of place and in place
                 Dh = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS, out_dtype=torch.float16)
                 Ch = torch.from_numpy(C0.astype(np.float16)).cuda().view(M, N)
                 tcu.gemm(Ad, Bd, 2.0, -1.0, C=Ch, out=Ch, variant=tcu.Variant.BLOCK_LDS)
                 torch.cuda.synchronize()
-                assert np.array_equal(Dh.cpu().numpy().view(np.uint16), ref0.astype(np.float16).view(np.uint16)), ("fp16", K, direct_lds, bk64, depth)
-                assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("fp16 in place", K, direct_lds, bk64, depth)
+                assert np.array_equal(Dh.cpu().numpy().view(np.uint16), ref0.astype(np.float16).view(np.uint16)), ("fp16", K, direct_lds, bk64, depth, staged)
+                assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("fp16 in place", K, direct_lds, bk64, depth, staged)
         # default kernel choice with outputs that are 4-byte but not 8- or 16-byte aligned: the kernel that
-        # moves four adjacent outputs per access must not be picked
+        # moves four adjacent outputs per access must not be picked; aligned to 8 bytes only: not its 16-byte epilogue
         tcu.set_option("gemm_direct_lds", -1)
+        tcu.set_option("gemm_staged_epilogue", 1)
         K = 384
         A = oracle.generate_f16(M * K, 13, oracle.DIST_SMALLINT)
         B = oracle.generate_f16(N * K, 14, oracle.DIST_SMALLINT)
@@ -290,7 +293,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
         ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
         buf32 = torch.zeros(M * N + 4, dtype=torch.float32, device="cuda")
         buf16 = torch.zeros(M * N + 4, dtype=torch.float16, device="cuda")
-        for off32, off16 in ((0, 0), (1, 2)):
+        for off32, off16 in ((0, 0), (1, 2), (2, 4)):
             Cd = buf32[off32:off32 + M * N].view(M, N)
             Cd.copy_(torch.from_numpy(C0).view(M, N))
             Ch = buf16[off16:off16 + M * N].view(M, N)
@@ -339,6 +342,7 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             assert np.array_equal(Dh.cpu().numpy().view(np.uint16), oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0).astype(np.float16).view(np.uint16)), ("128 tiles fp16", direct_lds, K)
     finally:
         tcu.set_option("gemm_split_tail", 1)
+        tcu.set_option("gemm_staged_epilogue", 1)
         tcu.set_option("gemm_direct_lds", -1)
         tcu.set_option("gemm_bk64", 0)
         tcu.set_option("gemm_depth", 4)
