@@ -42,6 +42,20 @@ TCU_DEVICE void gemm_tile_of_block(size_t tiles_m, size_t tiles_n, size_t b, siz
 // MFMA unit has): neighbouring lanes trade one value of each pair of rows, so that an even lane
 // owns two adjacent columns of the even row and the odd lane the same columns of the odd row,
 // and every access moves a 32-bit pair.
+// alpha * a + beta * c in one fixed rounding sequence (alpha * a rounded, then one fused multiply-add with beta * c).  Left
+// to the compiler, which of the two products is folded into the addition depends on the code around it, and two epilogues of
+// the same accumulators then differ in the last bit; with this every GEMM kernel and epilogue gives the same bits.
+// gemm_add_scaled takes the rounded product alpha * a (the epilogue that goes through LDS parks it there).
+TCU_DEVICE float gemm_add_scaled(float alpha_a, float beta, float c) { return __builtin_fmaf(beta, c, alpha_a); }
+TCU_DEVICE float gemm_axpby(float alpha, float a, float beta, float c) { return gemm_add_scaled(alpha * a, beta, c); }
+TCU_DEVICE float4_t gemm_add_scaled(float4_t alpha_a, float beta, float4_t c) {
+  float4_t r;
+#pragma unroll
+  for (int e = 0; e < 4; e++) r[e] = gemm_add_scaled(alpha_a[e], beta, c[e]);
+  return r;
+}
+TCU_DEVICE float4_t gemm_axpby(float alpha, float4_t a, float beta, float4_t c) { return gemm_add_scaled(alpha * a, beta, c); }
+
 template <typename OUT>
 TCU_DEVICE void gemm_store_tile(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float16_t &acc, int lane, float alpha, float beta) {
   if constexpr (sizeof(OUT) == 4) {
@@ -54,7 +68,7 @@ TCU_DEVICE void gemm_store_tile(OUT *D, const OUT *C, size_t ldc, size_t row0, s
 #pragma unroll
       for (int i = 0; i < 16; i++) c[i] = __builtin_nontemporal_load(C + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
 #pragma unroll
-      for (int i = 0; i < 16; i++) __builtin_nontemporal_store(alpha * acc[i] + beta * c[i], D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
+      for (int i = 0; i < 16; i++) __builtin_nontemporal_store(gemm_axpby(alpha, acc[i], beta, c[i]), D + base + (size_t)(8 * (i / 4) + (i % 4)) * ldc);
     }
   } else {
     const bool odd = (lane & 1) != 0;
@@ -81,7 +95,7 @@ TCU_DEVICE void gemm_store_tile(OUT *D, const OUT *C, size_t ldc, size_t row0, s
 #pragma unroll
       for (int p = 0; p < 8; p++) {
         const half2_t cv = __builtin_bit_cast(half2_t, c[p]);
-        __builtin_nontemporal_store(pack_f16x2(alpha * lo[p] + beta * (float)cv[0], alpha * hi[p] + beta * (float)cv[1]), d32 + base + (size_t)(8 * (p / 2) + 2 * (p % 2)) * ldw);
+        __builtin_nontemporal_store(pack_f16x2(gemm_axpby(alpha, lo[p], beta, (float)cv[0]), gemm_axpby(alpha, hi[p], beta, (float)cv[1])), d32 + base + (size_t)(8 * (p / 2) + 2 * (p % 2)) * ldw);
       }
     }
   }
@@ -681,16 +695,13 @@ TCU_DEVICE void gemm_store_row16(OUT *D, size_t ldc, size_t row0, size_t col0, c
   for (int j = 0; j < 8; j++) {
     float4_t r = alpha * acc[j];
     if constexpr (sizeof(OUT) == 4) {
-      if (beta != 0.0f) r += beta * c.v[j];
+      if (beta != 0.0f) r = gemm_axpby(alpha, acc[j], beta, c.v[j]);
       __builtin_nontemporal_store(r, p + j * 4);
     } else {
       if (beta != 0.0f) {
         const uint32_t w01 = c.v[j][0], w23 = c.v[j][1];  // scalars first: a bit cast straight from a vector element reads element 0
         const half2_t c01 = __builtin_bit_cast(half2_t, w01), c23 = __builtin_bit_cast(half2_t, w23);
-        r[0] += beta * (float)c01[0];
-        r[1] += beta * (float)c01[1];
-        r[2] += beta * (float)c23[0];
-        r[3] += beta * (float)c23[1];
+        r = gemm_axpby(alpha, acc[j], beta, float4_t{(float)c01[0], (float)c01[1], (float)c23[0], (float)c23[1]});
       }
       uint2_t v;
       v[0] = pack_f16x2(r[0], r[1]);
@@ -753,21 +764,15 @@ TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size
       word_t *d = reinterpret_cast<word_t *>(D + at0 + (size_t)(16 * i + ROWS_PER_ACCESS * t) * ldc);
       float4_t v0 = *reinterpret_cast<const float4_t *>(buf + r * kStageRowFloats + rc);
       if constexpr (sizeof(OUT) == 4) {
-        if (beta != 0.0f) v0 += beta * c[i & 1][t];
+        if (beta != 0.0f) v0 = gemm_add_scaled(v0, beta, c[i & 1][t]);
         __builtin_nontemporal_store(v0, d);
       } else {
         float4_t v1 = *reinterpret_cast<const float4_t *>(buf + r * kStageRowFloats + rc + 4);
         if (beta != 0.0f) {
           const uint32_t w0 = c[i & 1][t][0], w1 = c[i & 1][t][1], w2 = c[i & 1][t][2], w3 = c[i & 1][t][3];  // scalars first: a bit cast straight from a vector element reads element 0
           const half2_t c0 = __builtin_bit_cast(half2_t, w0), c1 = __builtin_bit_cast(half2_t, w1), c2 = __builtin_bit_cast(half2_t, w2), c3 = __builtin_bit_cast(half2_t, w3);
-          v0[0] += beta * (float)c0[0];
-          v0[1] += beta * (float)c0[1];
-          v0[2] += beta * (float)c1[0];
-          v0[3] += beta * (float)c1[1];
-          v1[0] += beta * (float)c2[0];
-          v1[1] += beta * (float)c2[1];
-          v1[2] += beta * (float)c3[0];
-          v1[3] += beta * (float)c3[1];
+          v0 = gemm_add_scaled(v0, beta, float4_t{(float)c0[0], (float)c0[1], (float)c1[0], (float)c1[1]});
+          v1 = gemm_add_scaled(v1, beta, float4_t{(float)c2[0], (float)c2[1], (float)c3[0], (float)c3[1]});
         }
         uint4_t o;
         o[0] = pack_f16x2(v0[0], v0[1]);
@@ -960,17 +965,14 @@ __global__ __launch_bounds__(256) void gemm_split_fixup_kernel(const float *__re
   const size_t o = (tile_m * kGemmBigBM + row) * N + tile_n * kGemmBigBN + col;
   float4_t r = alpha * sum;
   if constexpr (sizeof(OUT) == 4) {
-    if (beta != 0.0f) r += beta * *reinterpret_cast<const float4_t *>(C + o);
+    if (beta != 0.0f) r = gemm_axpby(alpha, sum, beta, *reinterpret_cast<const float4_t *>(C + o));
     *reinterpret_cast<float4_t *>(D + o) = r;
   } else {
     if (beta != 0.0f) {
       const uint2_t c = *reinterpret_cast<const uint2_t *>(C + o);
       const uint32_t w01 = c[0], w23 = c[1];
       const half2_t c01 = __builtin_bit_cast(half2_t, w01), c23 = __builtin_bit_cast(half2_t, w23);
-      r[0] += beta * (float)c01[0];
-      r[1] += beta * (float)c01[1];
-      r[2] += beta * (float)c23[0];
-      r[3] += beta * (float)c23[1];
+      r = gemm_axpby(alpha, sum, beta, float4_t{(float)c01[0], (float)c01[1], (float)c23[0], (float)c23[1]});
     }
     uint2_t v;
     v[0] = pack_f16x2(r[0], r[1]);
@@ -1006,7 +1008,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const uint16_t *__res
   const size_t m = idx / N, n = idx % N;
   float acc = 0.0f;
   for (size_t k = 0; k < K; k++) acc += (float)__builtin_bit_cast(half_t, A[m * K + k]) * (float)__builtin_bit_cast(half_t, B[n * K + k]);
-  D[idx] = (OUT)(beta == 0.0f ? alpha * acc : alpha * acc + beta * (float)C[idx]);
+  D[idx] = (OUT)(beta == 0.0f ? alpha * acc : gemm_axpby(alpha, acc, beta, (float)C[idx]));
 }
 
 }  // namespace tcu
