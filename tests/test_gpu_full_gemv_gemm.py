@@ -349,6 +349,37 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
         tcu.set_option("gemm_big_tiles", -1)
 
 
+def test_gemm_kernels_round_alike(tcu):
+    """alpha * acc + beta * c is one spelled-out rounding sequence in every GEMM epilogue: the direct kernel, the tiled
+    kernel with its outputs turned through LDS and the same kernel writing straight from the accumulators agree bit
+    for bit on inputs that are not integers (fp32 outputs; with fp16 outputs the two tiled forms agree bit for bit and
+    the direct kernel to one unit in the last place)."""
+    import torch
+
+    M = N = 512
+    K = 1024
+    A = tcu.generate(M * K, 5, tcu.Dist.NORMAL).view(M, K)
+    B = tcu.generate(N * K, 6, tcu.Dist.NORMAL).view(N, K)
+    try:
+        tcu.set_option("gemm_big_tiles", 1)
+        for dt in (torch.float32, torch.float16):
+            C = tcu.generate(M * N, 7, tcu.Dist.UNIFORM).view(M, N).to(dt)
+            bits = torch.int32 if dt == torch.float32 else torch.int16
+            got = {}
+            for name, variant, staged in (("direct kernel", tcu.Variant.MFMA_16N, 1), ("tiled, through LDS", tcu.Variant.AUTO, 1), ("tiled, from the accumulators", tcu.Variant.AUTO, 0)):
+                tcu.set_option("gemm_staged_epilogue", staged)
+                got[name] = tcu.gemm(A, B, 1.1, 1.2, C=C, variant=variant).view(bits)
+            torch.cuda.synchronize()
+            assert torch.equal(got["tiled, through LDS"], got["tiled, from the accumulators"]), dt
+            if dt == torch.float32:
+                assert torch.equal(got["direct kernel"], got["tiled, through LDS"])
+            else:  # the compiler may narrow the fused multiply-add of one kernel in a single rounding: exact ties can fall the other way
+                assert int((got["direct kernel"].int() - got["tiled, through LDS"].int()).abs().max()) <= 1
+    finally:
+        tcu.set_option("gemm_staged_epilogue", 1)
+        tcu.set_option("gemm_big_tiles", -1)
+
+
 def test_gemm_8192(tcu, oracle):
     """M = N = K = 8192, N(0,1) inputs, 1e-2 relative: 64 sampled rows against the fp64 oracle."""
     import torch
