@@ -897,7 +897,13 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
   if (share != nullptr) {
-    gemm_store_strip16<float>(share, nullptr, kGemmBigBN, wm * 128, wn * 128, acc, lane, 1.0f, 0.0f);
+    if constexpr (STAGED) {  // raw accumulators, whole rows of the 256 x 256 share (it is 16-byte aligned)
+      block_barrier_lds_only();
+      gemm_store_strip16_staged<float>(share, nullptr, kGemmBigBN, wm * 128, wn * 128, acc, lane, 1.0f, 0.0f, reinterpret_cast<float *>(&lds_a[0][0]) + wave * kStageWaveFloats);
+      block_barrier_lds_only();  // the block's next piece of work starts its transfers only after every wave has read its outputs back
+    } else {
+      gemm_store_strip16<float>(share, nullptr, kGemmBigBN, wm * 128, wn * 128, acc, lane, 1.0f, 0.0f);
+    }
   } else if constexpr (STAGED) {
     block_barrier_lds_only();  // the other waves have read their last fragments: the A buffers can hold outputs now
     static_assert(4 * kStageWaveFloats * sizeof(float) <= sizeof(lds_a), "staging area of four waves");
