@@ -19,7 +19,9 @@ elements already resident in HBM.  Order of the run:
 5. the CPU baseline: the reference's CPU path (restated in oracle/) on the same sweep.
 
 Two input buffers alternate between launches so that no launch finds its input in the 256 MB
-Infinity Cache.
+Infinity Cache, and the launches write their outputs to `--output-buffers` buffers in turn (default 3:
+1.5 GiB of scan output between two launches that write the same lines), so that no launch
+overwrites lines an earlier one left dirty in that cache: what a kernel writes has to reach HBM.
 """
 import argparse
 import hashlib
@@ -105,6 +107,9 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="skip the comparison with the CPU oracle before timing (for profiler runs)")
     ap.add_argument("--no-all-sizes", action="store_true", help="skip the second list (every power of two 16 ... 16384)")
     ap.add_argument("--with-copy-probe", action="store_true", help="also launch the plain copy kernel over 2^n_log2 halves before timing (calibrates hardware counters)")
+    ap.add_argument("--output-buffers", type=int, default=3, help="output buffers the launches take in turn (1 = every launch rewrites the same buffer)")
+    ap.add_argument("--scan-store-policy", type=int, default=0, choices=(0, 1, 2), help="stores of the scan kernels: 0 = the library's default, 1 = every other tile of a wave through the cache, 2 = all non-temporal")
+    ap.add_argument("--large-n-log2", type=int, default=30, help="element count of the second, larger run of the sweep's segment sizes (0 = leave it out)")
     ap.add_argument("--cpu-n-log2", type=int, default=28, help="element count of the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -124,17 +129,31 @@ def main():
 
     seeds = (1, 2)
     inputs = [tcu.generate(n, s, tcu.Dist.UNIFORM) for s in seeds]
-    red_out = torch.empty(n // 16, dtype=torch.float16, device="cuda")
-    scan_out = torch.empty(n, dtype=torch.float16, device="cuda")
+    if args.scan_store_policy:
+        tcu.set_option("scan_store_policy", args.scan_store_policy)
+    n_out = max(1, args.output_buffers)
+    red_outs = [torch.empty(n // 16, dtype=torch.float16, device="cuda") for _ in range(n_out)]
+    scan_outs = [torch.empty(n, dtype=torch.float16, device="cuda") for _ in range(n_out)]
+    red_out, scan_out = red_outs[0], scan_outs[0]  # what launch 0 writes (the checks read these)
     configs = [("reduce", s) for s in REDUCE_SEGS] + [("scan", s) for s in SCAN_SEGS]
     all_sizes = [] if args.no_all_sizes else [("reduce", s) for s in ALL_SIZES] + [("scan", s) for s in ALL_SIZES]
 
+    class Buffers:
+        """the arrays one element count works on: alternating inputs, outputs taken in turn"""
+
+        def __init__(self, n, inputs, red_outs, scan_outs):
+            self.n, self.inputs, self.red_outs, self.scan_outs = n, inputs, red_outs, scan_outs
+
+    main_buffers = Buffers(n, inputs, red_outs, scan_outs)
+    current = [main_buffers]
+
     def launch(i, kind, seg):
-        x = inputs[i & 1]
+        b = current[0]
+        x = b.inputs[i % len(b.inputs)]
         if kind == "reduce":
-            tcu.seg_reduce(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=red_out, stream=stream)
+            tcu.seg_reduce(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=b.red_outs[i % len(b.red_outs)], stream=stream)
         else:
-            tcu.seg_scan(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=scan_out, stream=stream)
+            tcu.seg_scan(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=b.scan_outs[i % len(b.scan_outs)], stream=stream)
 
     # families do not cover every size (MFMA_16 is 16 only, ...): such launches are left out and said so
     skipped = []
@@ -225,6 +244,7 @@ def main():
         for c, (kind, seg) in enumerate(launches):
             ms = sorted(events[k][c][0].elapsed_time(events[k][c][1]) for k in range(repeats))
             avg = sum(ms) / len(ms)
+            n = current[0].n
             by = algorithmic_bytes(kind, n, seg)
             rows.append({
                 "op": kind, "segment_size": seg, "avg_ms": round(avg, 5), "min_ms": round(ms[0], 5), "median_ms": round(ms[len(ms) // 2], 5),
@@ -246,6 +266,41 @@ def main():
             launch(counter, kind, seg)
             counter += 1
         all_rows, _ = timed_with_events(all_sizes, max(5, args.steps // 2))
+
+    # 4b. the sweep's segment sizes once more at a larger element count (not part of `value`): an output of
+    # 2^(large_n_log2 + 1) bytes is several times the 256 MiB memory-side cache by itself
+    large_rows = None
+    if args.large_n_log2 and variant == tcu.Variant.AUTO:
+        ln = 1 << args.large_n_log2
+        large = Buffers(ln, [tcu.generate(ln, s, tcu.Dist.UNIFORM) for s in seeds],
+                        [torch.empty(ln // 16, dtype=torch.float16, device="cuda") for _ in range(n_out)],
+                        [torch.empty(ln, dtype=torch.float16, device="cuda") for _ in range(min(n_out, 2))])
+        current[0] = large
+        if not args.no_check:
+            from oracle import binding as oracle
+
+            w = 1 << CHECK_WINDOW_LOG2
+            first = ln - w  # the last window of the array
+            x_host = oracle.generate_f16(w, seeds[0], oracle.DIST_UNIFORM, first=first)
+            for kind, seg in configs:
+                launch(0, kind, seg)
+                torch.cuda.synchronize()
+                if kind == "reduce":
+                    got = large.red_outs[0][first // seg:first // seg + w // seg].cpu().numpy().view(np.uint16)
+                    ref = oracle.seg_reduce_f64(x_host, w // seg, seg)
+                else:
+                    got = large.scan_outs[0][first:first + w].cpu().numpy().view(np.uint16)
+                    ref = oracle.seg_scan_f64(x_host, w // seg, seg)
+                bad, worst, first_bad = oracle.check_f16(got, ref, seg, 2.0, 1e-3)
+                if bad:
+                    print(f"bench.py: seg_{kind} segment_size={seg} at N=2^{args.large_n_log2} disagrees with the CPU oracle: {bad} of {got.size}, first at {first_bad}", file=sys.stderr)
+                    sys.exit(1)
+        for kind, seg in configs:  # warm
+            launch(counter, kind, seg)
+            counter += 1
+        large_rows, _ = timed_with_events(configs, max(5, args.steps // 2))
+        current[0] = main_buffers
+        del large
 
     total_s = t1 - t0
     elems_per_step = len(configs) * n
@@ -269,6 +324,7 @@ def main():
         "config": {"workload": "segmented sum reduction (seg %s) + segmented inclusive scan (seg %s), N=2^%d fp16 each" % (
                        ",".join(str(s) for k, s in configs if k == "reduce"), ",".join(str(s) for k, s in configs if k == "scan"), args.n_log2),
                    "variant": variant.name, "tiles_per_wave": args.tiles_per_wave, "waves_per_block": args.waves_per_block, "compute_units": info["compute_units"],
+                   "input_buffers": len(inputs), "output_buffers": n_out, "scan_store_policy": args.scan_store_policy,
                    "kernel_sources_digest": kernel_sources_digest()},
         "roofline": roofline,
         "checked_against_cpu_oracle": checked,
@@ -279,6 +335,9 @@ def main():
         result["skipped"] = skipped
     if all_rows:
         result["all_sizes"] = all_rows
+    if large_rows:
+        result["larger_n"] = {"n_log2": args.large_n_log2, "scan_output_buffers": min(n_out, 2), "rows": large_rows}
+        roofline["min_frac_larger_n"] = min(r["frac_hbm_peak"] for r in large_rows)
     if not args.no_cpu_baseline:
         cpu1, dt1 = cpu_baseline(args.cpu_n_log2, 1)
         threads = min(16, os.cpu_count() or 1)

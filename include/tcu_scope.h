@@ -101,6 +101,9 @@ int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int
 /* Tuning switches used by the benchmarks and tests (process-wide, not thread-safe against
  * concurrent launches):
  *   "nontemporal"     0/1, default 1: non-temporal loads and stores in the streaming kernels
+ *   "scan_store_policy"  1/2, default 1: while "nontemporal" is on, the segmented scans (and mode 0 of
+ *                     tcu_stream_probe) store every other 1 KiB tile of a wave through the cache and the others
+ *                     non-temporally (1), or all of them non-temporally (2)
  *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
  *   "scan_lds_tiles"  0/1, default 1: full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves)
  *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step

@@ -34,6 +34,7 @@ inline int fail(int code, const std::string &msg) {
 
 struct Options {
   bool nontemporal = true;
+  int scan_store_policy = kStoreStream;     // stores of the segmented scans and of the copy probe while `nontemporal` is on: kStoreAlternate or kStoreStream
   bool static_order = false;
   int gemm_big_tiles = -1;     // 256 x 256 block tiles: 1 wherever M and N allow, 0 never, -1 where there are at least 128 of them
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
@@ -59,6 +60,7 @@ inline int set_option(const char *name, int value) {
   const std::string n(name);
   Options &o = options();
   if (n == "nontemporal") o.nontemporal = value != 0;
+  else if (n == "scan_store_policy") o.scan_store_policy = value == kStoreStream ? kStoreStream : kStoreAlternate;
   else if (n == "static_order") o.static_order = value != 0;
   else if (n == "gemm_big_tiles") o.gemm_big_tiles = value < 0 ? -1 : (value != 0);
   else if (n == "gemm_direct_lds") o.gemm_direct_lds = value;
@@ -79,6 +81,9 @@ inline int set_option(const char *name, int value) {
   else return fail(TCU_ERR_INVALID_ARG, "tcu_set_option: unknown option " + n);
   return TCU_OK;
 }
+
+// the NT template argument of the scan kernels and of the copy probe (wave_ops.hpp: kTileStoreNT)
+inline int scan_store_policy() { return options().nontemporal ? options().scan_store_policy : kStoreCached; }
 
 inline WaitPolicy wait_policy(unsigned desc_shift = 0) { return WaitPolicy{options().lookback_poll_limit, options().test_mute_partition, desc_shift}; }
 // 32-bit words of a look-back workspace: the ticket's line, then one slot of 8 << desc_shift bytes per partition
@@ -178,8 +183,8 @@ inline Plan auto_plan_scan(size_t S) {
   if (S == 1024) return {false, 2, 2, 256};
   if (S == 2048) return {true, 2, 2, 256};
   if (S == 4096) return {true, 2, 4, 128};
-  if (S == 8192) return {true, 2, 8, 128};
-  if (S == 16384) return {true, 4, 8, 32};
+  if (S == 8192) return {true, 2, 8, 32};
+  if (S == 16384) return {true, 4, 8, 8};
   if (S == 32768) return {true, 8, 8, 16};
   if (S == 65536 || S == 131072) return {true, 4, 16, 32};
   if (S == 262144) return {true, 4, 16, 0};
@@ -264,6 +269,22 @@ inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned b
       case 13: launch(KERNEL<8, false, true>, __VA_ARGS__); break;         \
       case 14: launch(KERNEL<8, true, false>, __VA_ARGS__); break;         \
       default: launch(KERNEL<8, true, true>, __VA_ARGS__); break;          \
+    }                                                                      \
+  } while (0)
+
+// the same choice for kernels whose last template argument is fixed by the caller (a store policy)
+#define TCU_SWITCH_U_MFMA(KERNEL, u, mfma, LAST, ...)                      \
+  do {                                                                     \
+    const int _k = ((u) == 1 ? 0 : (u) == 2 ? 1 : (u) == 4 ? 2 : 3) * 2 + ((mfma) ? 1 : 0); \
+    switch (_k) {                                                          \
+      case 0: launch(KERNEL<1, false, LAST>, __VA_ARGS__); break;          \
+      case 1: launch(KERNEL<1, true, LAST>, __VA_ARGS__); break;           \
+      case 2: launch(KERNEL<2, false, LAST>, __VA_ARGS__); break;          \
+      case 3: launch(KERNEL<2, true, LAST>, __VA_ARGS__); break;           \
+      case 4: launch(KERNEL<4, false, LAST>, __VA_ARGS__); break;          \
+      case 5: launch(KERNEL<4, true, LAST>, __VA_ARGS__); break;           \
+      case 6: launch(KERNEL<8, false, LAST>, __VA_ARGS__); break;          \
+      default: launch(KERNEL<8, true, LAST>, __VA_ARGS__); break;          \
     }                                                                      \
   } while (0)
 
@@ -488,13 +509,15 @@ inline int seg_reduce_offsets_dispatch(const void *d_in, void *d_out, size_t num
 // ----- segmented inclusive prefix sum -------------------------------------------------------
 
 template <int LPS_LOG2, bool MFMA>
-inline void launch_scan_wave_u(int u, bool nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg, int tps_log2,
+inline void launch_scan_wave_u(int u, int nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg, int tps_log2,
                                unsigned iters, unsigned run) {
-#define TCU_SCAN_CASE(UU)                                                                                                               \
-  if (nt)                                                                                                                               \
-    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, true>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run); \
-  else                                                                                                                                  \
-    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, false>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run); \
+#define TCU_SCAN_CASE(UU)                                                                                                                         \
+  if (nt == kStoreAlternate)                                                                                                                      \
+    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, kStoreAlternate>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run); \
+  else if (nt == kStoreStream)                                                                                                                    \
+    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, kStoreStream>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);    \
+  else                                                                                                                                            \
+    launch(seg_scan_wave_kernel<LPS_LOG2, UU, MFMA, kStoreCached>, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);    \
   return
   switch (u) {
     case 1: TCU_SCAN_CASE(1);
@@ -505,7 +528,7 @@ inline void launch_scan_wave_u(int u, bool nt, unsigned grid, unsigned block, vo
 #undef TCU_SCAN_CASE
 }
 template <bool MFMA>
-inline void launch_scan_wave_s(int lps_log2, int u, bool nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg,
+inline void launch_scan_wave_s(int lps_log2, int u, int nt, unsigned grid, unsigned block, void *stream, const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t nseg,
                                int tps_log2, unsigned iters, unsigned run) {
   switch (lps_log2) {
     case 1: return launch_scan_wave_u<1, MFMA>(u, nt, grid, block, stream, in, out, totals, n_chunks, nseg, tps_log2, iters, run);
@@ -528,6 +551,7 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   uint4_t *out = static_cast<uint4_t *>(d_out);
   uint16_t *totals = static_cast<uint16_t *>(d_totals);
   const bool nt = options().nontemporal;
+  const int policy = scan_store_policy();
 
   if (generic) {
     const int gw = waves_per_block ? waves_per_block : 4;
@@ -551,7 +575,12 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
     const BlockShape shape = block_shape(tiles_per_seg, u, wpb, variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u);
     const size_t grid = (num_segments + shape.spb - 1) / shape.spb;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    TCU_SWITCH_U_MFMA_NT(seg_scan_block_kernel, shape.u, a.mfma, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, shape.spb, shape.group, run);
+    if (policy == kStoreStream)
+      TCU_SWITCH_U_MFMA(seg_scan_block_kernel, shape.u, a.mfma, kStoreStream, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, shape.spb, shape.group, run);
+    else if (policy == kStoreAlternate)
+      TCU_SWITCH_U_MFMA(seg_scan_block_kernel, shape.u, a.mfma, kStoreAlternate, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, shape.spb, shape.group, run);
+    else
+      TCU_SWITCH_U_MFMA(seg_scan_block_kernel, shape.u, a.mfma, kStoreCached, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, shape.spb, shape.group, run);
     return TCU_OK;
   }
   int lps_log2, tps_log2 = 0;
@@ -571,9 +600,9 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   const size_t grid = (waves + wpb - 1) / wpb;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
   if (a.mfma)
-    launch_scan_wave_s<true>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters, run);
+    launch_scan_wave_s<true>(lps_log2, u, policy, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters, run);
   else
-    launch_scan_wave_s<false>(lps_log2, u, nt, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters, run);
+    launch_scan_wave_s<false>(lps_log2, u, policy, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tps_log2, (unsigned)iters, run);
   return TCU_OK;
 }
 
@@ -666,7 +695,10 @@ inline int add_partial_sums_dispatch(void *d_out, const void *d_ps, size_t num_s
     const size_t n_chunks = n / 8;
     const size_t grid = (n_chunks + 255) / 256;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_add_partial_sums_f16: grid exceeds the launch limit");
-    launch(add_partial_sums_kernel, (unsigned)grid, 256u, stream, static_cast<uint4_t *>(d_out), static_cast<const uint16_t *>(d_ps), n_chunks, ilog2(segment_size) - 3, shifted ? 1 : 0);
+    if (options().nontemporal)
+      launch(add_partial_sums_kernel<true>, (unsigned)grid, 256u, stream, static_cast<uint4_t *>(d_out), static_cast<const uint16_t *>(d_ps), n_chunks, ilog2(segment_size) - 3, shifted ? 1 : 0);
+    else
+      launch(add_partial_sums_kernel<false>, (unsigned)grid, 256u, stream, static_cast<uint4_t *>(d_out), static_cast<const uint16_t *>(d_ps), n_chunks, ilog2(segment_size) - 3, shifted ? 1 : 0);
   } else {
     const size_t grid = (n + 255) / 256;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_add_partial_sums_f16: grid exceeds the launch limit");
@@ -1165,12 +1197,14 @@ inline int generate_dispatch(void *d, size_t n, uint64_t seed, int dist, size_t 
 }
 
 template <int U>
-inline void launch_probe(int mode, bool nt, unsigned grid, unsigned block, void *stream, uint4_t *dst, const half8_t *src, size_t n_chunks) {
-#define TCU_PROBE_CASE(MODE)                                                                   \
-  if (nt)                                                                                      \
-    launch(stream_probe_kernel<U, MODE, true>, grid, block, stream, dst, src, n_chunks);       \
-  else                                                                                         \
-    launch(stream_probe_kernel<U, MODE, false>, grid, block, stream, dst, src, n_chunks);      \
+inline void launch_probe(int mode, int nt, unsigned grid, unsigned block, void *stream, uint4_t *dst, const half8_t *src, size_t n_chunks) {
+#define TCU_PROBE_CASE(MODE)                                                                             \
+  if (nt == kStoreAlternate)                                                                             \
+    launch(stream_probe_kernel<U, MODE, kStoreAlternate>, grid, block, stream, dst, src, n_chunks);      \
+  else if (nt == kStoreStream)                                                                           \
+    launch(stream_probe_kernel<U, MODE, kStoreStream>, grid, block, stream, dst, src, n_chunks);         \
+  else                                                                                                   \
+    launch(stream_probe_kernel<U, MODE, kStoreCached>, grid, block, stream, dst, src, n_chunks);         \
   return
   switch (mode) {
     case 0: TCU_PROBE_CASE(0);
@@ -1192,7 +1226,7 @@ inline int stream_probe_dispatch(void *d_dst, const void *d_src, size_t bytes, i
   const size_t waves = (tiles + u - 1) / u;
   const size_t grid = (waves + wpb - 1) / wpb;
   if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-  const bool nt = options().nontemporal;
+  const int nt = scan_store_policy();
   uint4_t *dst = static_cast<uint4_t *>(d_dst);
   const half8_t *src = static_cast<const half8_t *>(d_src);
   switch (u) {

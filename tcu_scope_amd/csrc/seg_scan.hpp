@@ -201,7 +201,7 @@ TCU_DEVICE void scan_tile(half8_t v, float carry, const ScanOperands &ops, int l
 // S = 512 << tiles_per_seg_log2, a wave walks its segment(s) carrying the running sum.
 // Each wave owns iters*U consecutive tiles.
 // ---------------------------------------------------------------------------------------
-template <int LPS_LOG2, int U, bool MFMA, bool NT>
+template <int LPS_LOG2, int U, bool MFMA, int NT>
 __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, int tiles_per_seg_log2, unsigned iters,
                                                                    unsigned xcd_run) {
   const int lane = lane_id();
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t 
   for (unsigned it = 0; it < iters; it++) {
     const size_t t_it = tile0 + (size_t)it * U;
     half8_t v[U];
-    load_tiles<U, NT>(v, in, t_it * kTileChunks, n_chunks, lane);
+    load_tiles<U, NT != 0>(v, in, t_it * kTileChunks, n_chunks, lane);
     static_for<U>([&](auto J) {
       constexpr int j = decltype(J)::value;
       const size_t t = t_it + j;
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t 
 // waves_per_seg * U tiles, its wave w the U consecutive tiles starting at w * U; wave totals
 // meet in LDS.
 // ---------------------------------------------------------------------------------------
-template <int U, bool MFMA, bool NT>
+template <int U, bool MFMA, int NT>
 __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t *in, uint4_t *out, uint16_t *totals, size_t n_chunks, size_t num_segments, size_t tiles_per_seg,
                                                                     unsigned segs_per_block, unsigned waves_per_seg, unsigned xcd_run) {
   __shared__ float wave_total[2][kMaxWaves];
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
     for (size_t step0 = 0; step0 < tiles_per_seg; step0 += (size_t)G * U) {
       const size_t t0 = step0 + (size_t)wg * U;  // first tile of this wave (may lie past the segment)
       half8_t v[U];
-      load_tiles<U, NT>(v, in, (tile_base + t0) * kTileChunks, t0 < tiles_per_seg ? lim : 0, lane);
+      load_tiles<U, NT != 0>(v, in, (tile_base + t0) * kTileChunks, t0 < tiles_per_seg ? lim : 0, lane);
       // pass 1: this wave's total
       float acc = 0.0f;
 #pragma unroll
@@ -322,16 +322,17 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_generic_kernel(const uint1
 // out[s*S + i] += partial_sums[s], one fp16 addition per element (8 per lane per step).  With `shifted` the array
 // holds inclusive sums and segment s takes partial_sums[s - 1] (segment 0 nothing): the exclusive sums without a
 // pass that shifts them.
+template <bool NT>
 __global__ __launch_bounds__(256) void add_partial_sums_kernel(uint4_t *out, const uint16_t *partial_sums, size_t n_chunks, int seg_log2_chunks, int shifted) {
   const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= n_chunks) return;
   const size_t seg = c >> seg_log2_chunks;
   if (shifted && seg == 0) return;
   const float ps = (float)__builtin_bit_cast(half_t, partial_sums[shifted ? seg - 1 : seg]);
-  half8_t v = load_chunk<true>(reinterpret_cast<const half8_t *>(out + c));
+  half8_t v = load_chunk<NT>(reinterpret_cast<const half8_t *>(out + c));
   uint4_t r = {pack_f16x2((float)v[0] + ps, (float)v[1] + ps), pack_f16x2((float)v[2] + ps, (float)v[3] + ps), pack_f16x2((float)v[4] + ps, (float)v[5] + ps),
                pack_f16x2((float)v[6] + ps, (float)v[7] + ps)};
-  store_chunk_alternating<true>(out + c, r);
+  store_chunk_alternating<NT>(out + c, r);
 }
 __global__ __launch_bounds__(256) void add_partial_sums_generic_kernel(uint16_t *out, const uint16_t *partial_sums, size_t n, size_t segment_size, int shifted) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

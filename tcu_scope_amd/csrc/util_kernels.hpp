@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void generate_f16_kernel(uint16_t *out, size_t
 
 // Streaming probes with the access shape of the reduction / scan kernels: each wave takes
 // U consecutive tiles.  MODE 0 copy, 1 read only, 2 write only.
-template <int U, int MODE, bool NT>
+template <int U, int MODE, int NT>
 __global__ __launch_bounds__(kMaxBlock) void stream_probe_kernel(uint4_t *dst, const half8_t *src, size_t n_chunks) {
   const int lane = lane_id();
   const size_t gw = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(kMaxBlock) void stream_probe_kernel(uint4_t *dst, c
   if (chunk0 >= n_chunks) return;
   half8_t v[U];
   if constexpr (MODE != 2) {
-    load_tiles<U, NT>(v, src, chunk0, n_chunks, lane);
+    load_tiles<U, NT != 0>(v, src, chunk0, n_chunks, lane);
   } else {
 #pragma unroll
     for (int j = 0; j < U; j++) v[j] = splat8((float)lane);

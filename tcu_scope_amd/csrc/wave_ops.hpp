@@ -146,8 +146,12 @@ TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
 // alternating both 172 / 180.  The two kinds of store drain through different paths, and using both is worth 9 %.
 // Kernels that only read gain nothing from mixing their loads (segmented reduction: 72-82 us with all loads
 // non-temporal, 73-104 us with every other one through the cache), and the look-back scans lose (full_array.hpp).
-template <bool NT, int J>
-constexpr bool kTileStoreNT = NT && (J % 2 == 0);
+// The NT template argument of the scan kernels and of the copy probe names one of three policies (all loads are
+// non-temporal unless it is 0): 0 = every access through the cache, 1 = the alternation above (a bool `true`
+// converts to it), 2 = every store non-temporal.
+constexpr int kStoreCached = 0, kStoreAlternate = 1, kStoreStream = 2;
+template <int NT, int J>
+constexpr bool kTileStoreNT = NT == kStoreStream || (NT == kStoreAlternate && J % 2 == 0);
 
 // The same alternation where a tile's place in its wave is not known at compile time: the odd 1 KiB blocks of the
 // output go through the cache.  Written as assembly because the compiler merges two stores that differ only in

@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <thread>
 
 namespace harness {
@@ -43,6 +44,8 @@ void init_flags(int *argc, char **argv) {
       f.verify = v;
     else if (take(argv[i], "tcu_seed", &v))
       f.seed = std::strtoull(v.c_str(), nullptr, 0);
+    else if (take(argv[i], "tcu_out_buffers", &v))
+      f.out_buffers = std::atoi(v.c_str());
     else if (take(argv[i], "tcu_option", &v))
       f.options.push_back(v);
     else if (take(argv[i], "v", &v))
@@ -62,6 +65,7 @@ void init_flags(int *argc, char **argv) {
         "  --tcu_input=uniform|constant|grid   inputs: seeded uniform [-1,1) (default), the constant 0.001, or k/2048\n"
         "  --tcu_verify=auto|all|none          check results against a CPU fp64 sum before timing (auto: up to 2^26 elements)\n"
         "  --tcu_option=<name>:<value>         a tuning switch of the library (tcu_set_option), may be given several times\n"
+        "  --tcu_out_buffers=<n>               output buffers the scan benchmarks' timed launches take in turn (default 3)\n"
         "  --tcu_seed=<n>  --v=<level>\n");
   }
 }
@@ -261,6 +265,26 @@ static void guarded(benchmark::State &state, Body body) {
   }
 }
 
+// Output buffers of the scan benchmarks that the timed launches take in turn (--tcu_out_buffers, default 3): a
+// launch then never rewrites lines that the launch before it left dirty in the 256 MiB memory-side cache, so every
+// byte a kernel writes has to reach HBM at the rate it is written.  The reference writes one d_out
+// (src/prefixsum/seg_wmma_256n.cu:12-222); its V100 has no such cache.
+class RotatingOutputs {
+ public:
+  explicit RotatingOutputs(size_t bytes) {
+    int n = flags().out_buffers < 1 ? 1 : flags().out_buffers;
+    while (n > 1 && (double)bytes * n > 24.0 * 1024 * 1024 * 1024) n--;
+    for (int i = 0; i < n; i++) bufs_.emplace_back(new DeviceBuffer(bytes));
+  }
+  void *first() const { return bufs_[0]->get(); }
+  void *next() { return bufs_[turn_++ % bufs_.size()]->get(); }
+  size_t count() const { return bufs_.size(); }
+
+ private:
+  std::vector<std::unique_ptr<DeviceBuffer>> bufs_;
+  size_t turn_ = 0;
+};
+
 static void set_common_counters(benchmark::State &state, size_t num_segments, size_t segment_size, size_t num_elements, int waves_per_block, double bytes_per_iteration) {
   state.counters.insert({{"num_segments", (double)num_segments},
                          {"segment_size", (double)segment_size},
@@ -344,7 +368,8 @@ void run_seg_scan_offsets(benchmark::State &state, const char *name) {
     }
     const int nin = num_elements <= ((size_t)1 << 29) ? 2 : 1;
     DeviceBuffer in[2] = {DeviceBuffer(num_elements * 2), DeviceBuffer(nin == 2 ? num_elements * 2 : 16)};
-    DeviceBuffer out(num_elements * 2), offsets((num_segments + 1) * sizeof(int));
+    DeviceBuffer offsets((num_segments + 1) * sizeof(int));
+    RotatingOutputs out(num_elements * 2);
     for (int i = 0; i < nin; i++) fill_input(in[i].get(), num_elements, flags().seed + i);
     {
       std::vector<int> h(num_segments + 1);
@@ -352,20 +377,21 @@ void run_seg_scan_offsets(benchmark::State &state, const char *name) {
       PRINT_IF_ERROR(hipMemcpy(offsets.get(), h.data(), h.size() * sizeof(int), hipMemcpyHostToDevice));
     }
     const int *off = static_cast<const int *>(offsets.get());
-    TCU_CHECK(tcu_seg_scan_offsets_f16(in[0].get(), out.get(), num_segments, off, off + 1, 32, segment_size, nullptr));
+    TCU_CHECK(tcu_seg_scan_offsets_f16(in[0].get(), out.first(), num_segments, off, off + 1, 32, segment_size, nullptr));
     PRINT_IF_ERROR(hipDeviceSynchronize());
-    if (should_verify(num_elements)) verify_seg_scan(in[0].get(), out.get(), num_segments, segment_size, name);
+    if (should_verify(num_elements)) verify_seg_scan(in[0].get(), out.first(), num_segments, segment_size, name);
     EventPair ev;
     size_t it = 0;
     for (auto _ : state) {
       ev.start();
-      TCU_CHECK(tcu_seg_scan_offsets_f16(in[it++ % nin].get(), out.get(), num_segments, off, off + 1, 32, segment_size, nullptr));
+      TCU_CHECK(tcu_seg_scan_offsets_f16(in[it++ % nin].get(), out.next(), num_segments, off, off + 1, 32, segment_size, nullptr));
       const float ms = ev.stop_ms();
       state.PauseTiming();
       state.SetIterationTime(ms / 1000);
       state.ResumeTiming();
     }
     set_common_counters(state, num_segments, segment_size, num_elements, 0, 4.0 * num_elements + 4.0 * num_segments);
+    state.counters.insert({"output_buffers", (double)out.count()});
   });
 }
 
@@ -375,26 +401,28 @@ void run_seg_scan(benchmark::State &state, int variant, int tiles_per_wave, int 
     const size_t num_elements = num_segments * segment_size;
     const int nin = num_elements <= ((size_t)1 << 29) ? 2 : 1;
     DeviceBuffer in[2] = {DeviceBuffer(num_elements * 2), DeviceBuffer(nin == 2 ? num_elements * 2 : 16)};
-    DeviceBuffer out(num_elements * 2), totals(with_totals ? num_segments * 2 : 16);
+    DeviceBuffer totals(with_totals ? num_segments * 2 : 16);
+    RotatingOutputs out(num_elements * 2);
     for (int i = 0; i < nin; i++) fill_input(in[i].get(), num_elements, flags().seed + i);
     void *tp = with_totals ? totals.get() : nullptr;
-    TCU_CHECK(tcu_seg_scan_f16(in[0].get(), out.get(), tp, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, nullptr));
+    TCU_CHECK(tcu_seg_scan_f16(in[0].get(), out.first(), tp, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, nullptr));
     PRINT_IF_ERROR(hipDeviceSynchronize());
     if (should_verify(num_elements)) {
-      verify_seg_scan(in[0].get(), out.get(), num_segments, segment_size, name);
+      verify_seg_scan(in[0].get(), out.first(), num_segments, segment_size, name);
       if (with_totals) verify_seg_reduce(in[0].get(), totals.get(), num_segments, segment_size, name);
     }
     EventPair ev;
     size_t it = 0;
     for (auto _ : state) {
       ev.start();
-      TCU_CHECK(tcu_seg_scan_f16(in[it++ % nin].get(), out.get(), tp, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, nullptr));
+      TCU_CHECK(tcu_seg_scan_f16(in[it++ % nin].get(), out.next(), tp, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, nullptr));
       const float ms = ev.stop_ms();
       state.PauseTiming();
       state.SetIterationTime(ms / 1000);
       state.ResumeTiming();
     }
     set_common_counters(state, num_segments, segment_size, num_elements, waves_per_block, 4.0 * num_elements);
+    state.counters.insert({"output_buffers", (double)out.count()});
   });
 }
 
@@ -434,21 +462,23 @@ void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, i
     }
     size_t ws_bytes = 0;
     TCU_CHECK(tcu_full_scan_f16(nullptr, nullptr, num_elements, nullptr, &ws_bytes, strategy, segment_size, waves_per_block, nullptr));
-    DeviceBuffer in(num_elements * 2), out(num_elements * 2), ws(ws_bytes);
+    DeviceBuffer in(num_elements * 2), ws(ws_bytes);
+    RotatingOutputs out(num_elements * 2);
     fill_input(in.get(), num_elements, flags().seed);
-    TCU_CHECK(tcu_full_scan_f16(in.get(), out.get(), num_elements, ws.get(), &ws_bytes, strategy, segment_size, waves_per_block, nullptr));
+    TCU_CHECK(tcu_full_scan_f16(in.get(), out.first(), num_elements, ws.get(), &ws_bytes, strategy, segment_size, waves_per_block, nullptr));
     PRINT_IF_ERROR(hipDeviceSynchronize());
-    if (should_verify(num_elements)) verify_seg_scan(in.get(), out.get(), 1, num_elements, name);
+    if (should_verify(num_elements)) verify_seg_scan(in.get(), out.first(), 1, num_elements, name);
     EventPair ev;
     for (auto _ : state) {
       ev.start();
-      TCU_CHECK(tcu_full_scan_f16(in.get(), out.get(), num_elements, ws.get(), &ws_bytes, strategy, segment_size, waves_per_block, nullptr));
+      TCU_CHECK(tcu_full_scan_f16(in.get(), out.next(), num_elements, ws.get(), &ws_bytes, strategy, segment_size, waves_per_block, nullptr));
       const float ms = ev.stop_ms();
       state.PauseTiming();
       state.SetIterationTime(ms / 1000);
       state.ResumeTiming();
     }
     set_common_counters(state, segment_size ? num_elements / segment_size : 1, segment_size, num_elements, waves_per_block, 4.0 * num_elements);
+    state.counters.insert({"output_buffers", (double)out.count()});
   });
 }
 

@@ -22,6 +22,7 @@ struct Flags {
   std::string input = "uniform";     // --tcu_input=uniform|constant|grid   (constant = the reference's 0.001 fill)
   std::string verify = "auto";       // --tcu_verify=auto|all|none          (auto: up to 2^26 elements)
   uint64_t seed = 1;                 // --tcu_seed
+  int out_buffers = 3;               // --tcu_out_buffers: output buffers the timed launches of the scan benchmarks take in turn
   std::vector<std::string> options;  // --tcu_option=<name>:<value>, handed to tcu_set_option after tcu_init
   int verbose = 0;                   // --v
   bool help = false;                 // --help / -h

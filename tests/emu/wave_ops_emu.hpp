@@ -369,8 +369,9 @@ template <bool NT>
 inline void store_chunk_alternating(uint4_t *p, uint4_t v) {
   *p = v;
 }
-template <bool NT, int J>
-constexpr bool kTileStoreNT = NT && (J % 2 == 0);
+constexpr int kStoreCached = 0, kStoreAlternate = 1, kStoreStream = 2;
+template <int NT, int J>
+constexpr bool kTileStoreNT = NT == kStoreStream || (NT == kStoreAlternate && J % 2 == 0);
 template <int V>
 struct Int {
   static constexpr int value = V;
