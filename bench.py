@@ -94,6 +94,22 @@ def cpu_baseline(n_log2, threads):
     return elems / dt / 1e9, dt
 
 
+def cpu_baseline_config1(threads, seconds=2.0):
+    """The same CPU path on the configuration it is quoted on upstream: N = 2^20 halves from seed 0 in 65536
+    segments of 16, repeated until about `seconds` of CPU work are done."""
+    from oracle import binding as oracle
+
+    n, seg = 1 << 20, 16
+    x = oracle.generate_f16(n, 0, oracle.DIST_UNIFORM)
+    oracle.seg_reduce_ref(x, n // seg, seg, nthreads=threads)
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        oracle.seg_reduce_ref(x, n // seg, seg, nthreads=threads)
+        reps += 1
+    dt = time.perf_counter() - t0
+    return reps * n / dt / 1e9, reps, dt
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -345,6 +361,9 @@ def main():
         sample = "same 9-launch sweep at N=2^%d per launch (%.1f s of CPU work)" % (args.cpu_n_log2, dt1)
         result["cpu_baseline"] = {"value": round(cpu1, 4), "unit": "Gelem/s", "cores": 1, "kind": "port", "sample": sample}
         result["cpu_baseline_threaded"] = {"value": round(cpun, 4), "unit": "Gelem/s", "cores": threads, "kind": "port", "sample": sample.replace("%.1f s" % dt1, "%.1f s" % dtn)}
+        c1, reps1, dtc = cpu_baseline_config1(1)
+        result["cpu_baseline_config1"] = {"value": round(c1, 4), "unit": "Gelem/s", "cores": 1, "kind": "port",
+                                          "sample": "segmented sum reduction, N=2^20 fp16 from seed 0, 65536 segments of 16: %d passes in %.1f s" % (reps1, dtc)}
     print(json.dumps(result))
 
 

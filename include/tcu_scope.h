@@ -30,6 +30,9 @@
  *     state.SkipWithError (e.g. "segment size must be 16").
  *   - thread-compatible: concurrent calls must use different streams and, where a
  *     workspace is taken, different workspaces.
+ *   - this header holds what replaces a reference kernel or harness helper.  Tuning switches,
+ *     the test hooks and the measurement aids of this build's own benchmarks and tests are
+ *     declared in tcu_scope_dev.h; a caller of the entry points below needs none of them.
  *   - results: fp32 accumulation, one round-to-nearest-even conversion to fp16.
  */
 #ifndef TCU_SCOPE_H
@@ -42,7 +45,11 @@
 extern "C" {
 #endif
 
-#define TCU_SCOPE_ABI_VERSION 1
+/* 2: entry points over offsets and key arrays, tcu_seg_scan_f16_noalloc, the TCU_FULL_MFMA flag, block variants from 16
+ * halves per segment, 256 bytes of workspace per partition of the full-array scan (a cached size from version 1 is too
+ * small), tcu_init fails when the scratch symbol cannot be resolved; the tuning switches and measurement aids moved to
+ * tcu_scope_dev.h. */
+#define TCU_SCOPE_ABI_VERSION 2
 
 typedef enum {
   TCU_OK = 0,
@@ -98,52 +105,6 @@ const char *tcu_last_error(void);
 int tcu_abi_version(void);
 /* Compute units, wavefront size, LDS bytes per CU, 1 if the device is gfx950. */
 int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int *is_gfx950);
-/* Tuning switches used by the benchmarks and tests (process-wide, not thread-safe against
- * concurrent launches):
- *   "nontemporal"     0/1, default 1: non-temporal loads and stores in the streaming kernels
- *   "scan_store_policy"  1/2, default 1: while "nontemporal" is on, the segmented scans (and mode 0 of
- *                     tcu_stream_probe) store every other 1 KiB tile of a wave through the cache and the others
- *                     non-temporally (1), or all of them non-temporally (2)
- *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
- *   "scan_lds_tiles"  0/1, default 1: full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves)
- *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step
- *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more);
- *                     "gemv_waves" also sets the waves that split K in the strip kernels (TCU_VARIANT_MFMA_16N)
- *   "gemv_strip_lds"  0/1, default 1: TCU_VARIANT_MFMA_16N stages the 16-row strip through LDS where K is a
- *                     multiple of 512 (0: operands straight from global memory at every K)
- *   "gemm_big_tiles"  -1/0/1, default -1: 256 x 256 block tiles wherever M and N allow (1), never (0), or
- *                     where the output has at least 128 of them (-1; smaller outputs take 128 x 128 tiles)
- *   "gemm_direct_lds" -1/0/3/4/64/65/66, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
- *                     buffers; 64 = K step 64, two buffers; 65 = K step 64, three buffers for A and two for B;
- *                     66 = as 65 on 16x16x32 instead of 32x32x16 MFMAs (C and D aligned to four outputs, else 65);
- *                     0 = register-staged kernel; -1 = 66 where K is a multiple of 64, else 4
- *   "gemm_split_tail" 0/1/2, default 1: the K steps of the tiles of a last, partly filled round of the big-tile GEMM
- *                     grid are spread over all compute units (fp32 shares in stream-ordered temporary memory, added
- *                     in a fixed order by a second kernel): never, where it pays (round at most a third full,
- *                     K >= 4096), or whenever there is such a round
- *   "compute_units"   blocks of the big-tile GEMM kernel the device runs at a time (set by tcu_init; for tests)
- *   "gemm_staged_epilogue" 0/1, default 1: the big-tile GEMM kernel on 16x16x32 MFMAs turns its outputs through LDS and
- *                     writes (and reads C in) whole rows of a wave's 128 columns, 16 bytes per lane, where C and D are
- *                     16-byte aligned; 0 = straight from the accumulator layout (64 / 32 bytes of 16 rows per store)
- *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
- *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
- *   "many_totals"     default 65536: TCU_FULL_MULTI_KERNEL adds (reduce) or scans (scan) the per-segment totals with one
- *                     block below this many segments, and with the two-launch partition sums / the single-pass scan
- *                     (whose own workspace then follows the totals) from there on
- *   "xcd_run"         -1/0/C, default -1: consecutive blocks of a launch run on different XCDs (block b on XCD
- *                     b % 8); with C > 0 the segmented kernels renumber their blocks inside groups of 8 * C so that
- *                     every XCD works on C consecutive pieces of the array (a piece = what one block takes) while
- *                     the launch still sweeps the array front to back; 0 = no renumbering; -1 = the value measured
- *                     best for the segment size and launch shape
- *   "lookback_poll_limit"  default 2^20 (negative restores it): how often a block of a single-pass full-array
- *                     kernel (and of the look-back path of tcu_seg_scan_f16 for segments of 2^21 halves and more)
- *                     looks again for a value another block has not published yet before it gives up.  Giving up
- *                     never yields a finite wrong number: the reduction's result, or the scan's outputs from the
- *                     waiting partition to the end of the array (or segment), become NaN
- *   "test_mute_partition"  default 0; p > 0: partition p - 1 of those kernels publishes nothing, so every wait
- *                     for it expires (for tests of the rule above; all kernels still run to their end)
- * Unknown names return TCU_ERR_INVALID_ARG. */
-int tcu_set_option(const char *name, int value);
 
 /* ---- segmented reduction -------------------------------------------------------------- */
 
@@ -238,7 +199,15 @@ int tcu_full_reduce_f16(const void *d_in, void *d_out, size_t n, void *d_workspa
 
 /* d_out[i] = fp16(d_in[0] + ... + d_in[i]).  Replaces compute_wmma_prefixsum_cg /
  * _atomic_w_atomicballot (reference src/prefixsum/kernel.cuh:779-972) and the 3-kernel
- * sequence (src/prefixsum/wmma_3kers.cu:60-82). */
+ * sequence (src/prefixsum/wmma_3kers.cu:60-82).
+ * The single-pass strategies are not bit-reproducible on general inputs: a partition's fp32 carry is the sum of the
+ * aggregates of the predecessors it had to walk plus the first published prefix it met, and where that prefix is met
+ * depends on timing, so the last bit of a carry (and of outputs that round differently because of it) can differ
+ * between two runs.  Every run is within 2 ulp_fp16 + 1e-3 * sqrt(n) of the exact sum; inputs whose partial sums are
+ * exact in fp32 give identical bits every time.  TCU_FULL_MULTI_KERNEL and the reductions add in a fixed order.
+ * A wait for another partition that expires ("lookback_poll_limit" in tcu_scope_dev.h) is reported: the call still
+ * returns TCU_OK (nothing is known when it returns), d_out then holds NaN from the waiting partition on, and word 1
+ * of the workspace (a 32-bit unsigned, zeroed by every call) holds the number of partitions that gave up. */
 int tcu_full_scan_f16(const void *d_in, void *d_out, size_t n, void *d_workspace, size_t *workspace_bytes, int strategy, size_t segment_size, int waves_per_block, void *stream);
 
 /* ---- dense contractions -------------------------------------------------------------------- */
@@ -286,27 +255,6 @@ int tcu_convert_f32_to_f16(void *d_out, const void *d_in, size_t n, void *stream
  * src/gemm/wmma.cu:110-127), which are not reproducible without cuRAND.  UNIFORM, GRID
  * and SMALLINT are bit-identical to the host generator used by the tests. */
 int tcu_generate_f16(void *d, size_t n, uint64_t seed, int dist, size_t first, void *stream);
-
-/* ---- measurement aids ---------------------------------------------------------------------------- */
-
-/* Plain streaming kernels with the same access shape as the reductions/scans: mode 0
- * copies `bytes` from d_src to d_dst, mode 1 only reads d_src (one word per block is
- * written to d_dst), mode 2 only writes d_dst.  Used to calibrate hardware counters and
- * to report what fraction of peak a pure copy reaches.  bytes must be a multiple of 16. */
-int tcu_stream_probe(void *d_dst, const void *d_src, size_t bytes, int mode, int tiles_per_wave, int waves_per_block, void *stream);
-/* The next kernel that this host thread launches through the library carries the two events
- * (hipEvent_t created with timing enabled; either may be NULL): its dispatch stamps
- * start_event with the time the kernel begins and stop_event with the time it ends, so that
- * hipEventElapsedTime(start, stop) is the kernel's own duration, without the event packets a
- * hipEventRecord pair puts on the stream around it.  Meant for entry points that launch one
- * kernel; with several, only the first carries the events.  The reference brackets its
- * launches with cudaEventRecord (e.g. src/reduction/seg_wmma_16n.cu:57-73). */
-int tcu_time_next_launch(void *start_event, void *stop_event);
-/* Runs every cross-lane primitive the kernels rely on (MFMA 16x16x32 / 32x32x16 operand
- * layouts, DPP controls, lane swaps) on lane-indexed inputs and writes the raw results
- * to d_out (fp32 / u32 words; lane_probe_kernel in tcu_scope_amd/csrc/util_kernels.hpp has the record layout).
- * *out_words receives the number of 32-bit words (call with d_out == NULL to query). */
-int tcu_lane_probe(void *d_out, size_t *out_words, void *stream);
 
 #ifdef __cplusplus
 }

@@ -36,5 +36,6 @@ from .binding import (  # noqa: F401
     seg_reduce_by_key,
     set_option,
     stream_probe,
+    temporary_allocations,
     time_next_launch,
 )

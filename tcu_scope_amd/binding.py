@@ -13,7 +13,7 @@ EXPORTS = [
     "tcu_abi_version", "tcu_last_error", "tcu_init", "tcu_device_info", "tcu_set_option",
     "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_f16_noalloc", "tcu_seg_scan_offsets_f16", "tcu_seg_scan_by_key_f16", "tcu_seg_reduce_by_key_f16", "tcu_add_partial_sums_f16",
     "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32", "tcu_gemv_f16_f16", "tcu_gemm_f16_f16",
-    "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_time_next_launch", "tcu_lane_probe",
+    "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_time_next_launch", "tcu_lane_probe", "tcu_temporary_allocations",
 ]
 
 
@@ -105,8 +105,10 @@ def lib():
         L.tcu_stream_probe.argtypes = [vp, vp, sz, ci, ci, ci, vp]
         L.tcu_lane_probe.argtypes = [vp, c.POINTER(sz), vp]
         L.tcu_time_next_launch.argtypes = [vp, vp]
+        L.tcu_temporary_allocations.argtypes = []
+        L.tcu_temporary_allocations.restype = c.c_ulong
         for name in EXPORTS:
-            if name not in ("tcu_last_error",):
+            if name not in ("tcu_last_error", "tcu_temporary_allocations"):
                 getattr(L, name).restype = ci
         _lib = L
     return _lib
@@ -378,6 +380,11 @@ def generate(n, seed, dist=Dist.UNIFORM, first=0, out=None, device="cuda", strea
 
 def stream_probe(dst, src, nbytes, mode, tiles_per_wave=0, waves_per_block=0, stream=None):
     _check(lib().tcu_stream_probe(_ptr(dst), _ptr(src), nbytes, mode, tiles_per_wave, waves_per_block, _stream(stream)))
+
+
+def temporary_allocations():
+    """How many times the library has taken temporary device memory since the process began."""
+    return int(lib().tcu_temporary_allocations())
 
 
 def time_next_launch(start, stop):

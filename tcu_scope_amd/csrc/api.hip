@@ -18,20 +18,34 @@ static __device__ __align__(256) unsigned scratch[kScratchWords];
 
 namespace {
 
-// The address of `scratch` on the current device, resolved once per device (tcu_init does it
-// for the device it selects; otherwise the first call that needs it).
-int scratch_on_current_device(const char *what, unsigned **out) {
+// The address of `scratch` on the device the work will run on: the stream's device, or the current device for the
+// default stream (the rule tcu::stream_alloc follows).  Resolved once per device (tcu_init does it for the device it
+// selects; otherwise the first call that needs it); hipGetSymbolAddress answers for the current device, so a stream
+// of another device makes that device current for the query and restores the caller's afterwards.
+int scratch_on_device_of(const char *what, void *stream, unsigned **out) {
   constexpr int kMaxDevices = 64;
   static unsigned *address[kMaxDevices] = {};
   static std::mutex address_mutex;
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
+  int current = 0;
+  hipError_t e = hipGetDevice(&current);
   if (e != hipSuccess) return tcu::fail(TCU_ERR_RUNTIME, std::string(what) + ": hipGetDevice: " + hipGetErrorString(e));
+  int dev = current;
+  if (stream) {
+    hipDevice_t of_stream = 0;
+    e = hipStreamGetDevice(static_cast<hipStream_t>(stream), &of_stream);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return tcu::fail(TCU_ERR_RUNTIME, std::string(what) + ": hipStreamGetDevice: " + hipGetErrorString(e));
+    }
+    dev = (int)of_stream;
+  }
   if (dev < 0 || dev >= kMaxDevices) return tcu::fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": device ordinal beyond what the library keeps scratch addresses for");
   std::lock_guard<std::mutex> lock(address_mutex);
   if (!address[dev]) {
+    if (dev != current && (e = hipSetDevice(dev)) != hipSuccess) return tcu::fail(TCU_ERR_RUNTIME, std::string(what) + ": hipSetDevice: " + hipGetErrorString(e));
     unsigned *p = nullptr;
     e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+    if (dev != current) (void)hipSetDevice(current);
     if (e != hipSuccess || !p) {
       (void)hipGetLastError();
       return tcu::fail(TCU_ERR_RUNTIME, std::string(what) + ": hipGetSymbolAddress(scratch): " + hipGetErrorString(e));
@@ -98,7 +112,7 @@ int tcu_init(int device_id) {
   if (s.compute_units > 0) tcu::options().compute_units = s.compute_units;
   if (!s.gfx950) return tcu::fail(TCU_ERR_UNSUPPORTED, std::string("tcu_init: this library is built for gfx950 only, device is ") + prop.gcnArchName);
   unsigned *scratch_address = nullptr;
-  return scratch_on_current_device("tcu_init", &scratch_address);
+  return scratch_on_device_of("tcu_init", nullptr, &scratch_address);
 }
 
 int tcu_device_info(int *compute_units, int *wavefront_size, int *lds_bytes, int *is_gfx950) {
@@ -134,7 +148,7 @@ int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_s
 int tcu_seg_scan_f16_noalloc(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream) {
   const char *what = "tcu_seg_scan_f16_noalloc";
   tcu::ScanScratch s;
-  if (int rc = scratch_on_current_device(what, &s.words)) return rc;
+  if (int rc = scratch_on_device_of(what, stream, &s.words)) return rc;
   s.capacity = kScratchWords;
   const unsigned long before = tcu::launch_count();
   return after_launch(what, before, tcu::seg_scan_dispatch(d_in, d_out, d_totals, num_segments, segment_size, variant, tiles_per_wave, waves_per_block, stream, what, s));
@@ -211,6 +225,8 @@ int tcu_time_next_launch(void *start_event, void *stop_event) {
   ev.stop = static_cast<hipEvent_t>(stop_event);
   return TCU_OK;
 }
+
+unsigned long tcu_temporary_allocations(void) { return tcu::stream_alloc_count().load(); }
 
 int tcu_lane_probe(void *d_out, size_t *out_words, void *stream) { const unsigned long before = tcu::launch_count();
   return after_launch("tcu_lane_probe", before, tcu::lane_probe_dispatch(d_out, out_words, stream)); }

@@ -72,7 +72,10 @@ TCU_DEVICE float look_back_flagged(const unsigned long long *desc, long long par
     const int first_stop = is_stop ? __builtin_ctzll(is_stop) : 64;
     const unsigned long long needed = first_stop >= 63 ? ~0ull : ((2ull << first_stop) - 1ull);
     if (is_empty & needed) {
-      if (polls++ >= wait.poll_limit) return __builtin_nanf("");
+      if (polls++ >= wait.poll_limit) {
+        note_expired_wait(wait, lane);
+        return __builtin_nanf("");
+      }
       spin_pause();
       continue;
     }
@@ -137,6 +140,7 @@ TCU_DEVICE void look_back_value_and_count(const unsigned long long *desc, long l
     }
     if (waiting) {
       if (polls++ >= wait.poll_limit) {
+        note_expired_wait(wait, lane);
         *value = __builtin_nanf("");
         *count = 0xffffffffu;
         return;

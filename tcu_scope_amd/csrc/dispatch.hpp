@@ -12,6 +12,7 @@
 #include <string>
 
 #include "../../include/tcu_scope.h"
+#include "../../include/tcu_scope_dev.h"
 #include "launch.hpp"
 #include "seg_reduce.hpp"
 #include "seg_scan.hpp"
@@ -85,7 +86,8 @@ inline int set_option(const char *name, int value) {
 // the NT template argument of the scan kernels and of the copy probe (wave_ops.hpp: kTileStoreNT)
 inline int scan_store_policy() { return options().nontemporal ? options().scan_store_policy : kStoreCached; }
 
-inline WaitPolicy wait_policy(unsigned desc_shift = 0) { return WaitPolicy{options().lookback_poll_limit, options().test_mute_partition, desc_shift}; }
+// workspace: where the waits that give up are counted (word 1 of a look-back or single-pass reduction workspace)
+inline WaitPolicy wait_policy(unsigned desc_shift, unsigned *workspace) { return WaitPolicy{options().lookback_poll_limit, options().test_mute_partition, desc_shift, workspace ? workspace + 1 : nullptr}; }
 // 32-bit words of a look-back workspace: the ticket's line, then one slot of 8 << desc_shift bytes per partition
 inline size_t look_back_words(size_t parts, unsigned desc_shift) { return 64 + 2 * ((parts ? parts : 1) << desc_shift); }
 // 256 bytes per descriptor while that stays within 4 MiB, closer together for the (slow anyway) launches with more partitions
@@ -344,9 +346,9 @@ inline int seg_scan_huge(const char *what, const half8_t *in, uint4_t *out, uint
   launch(zero_look_back_kernel, (unsigned)((parts + 255) / 256), 256u, stream, ws, parts, shift);
   const int static_order = options().static_order ? 1 : 0;
   if (nt)
-    launch(full_scan_kernel<8, false, true>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy(shift));
+    launch(full_scan_kernel<8, false, true>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy(shift, ws));
   else
-    launch(full_scan_kernel<8, false, false>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy(shift));
+    launch(full_scan_kernel<8, false, false>, (unsigned)parts, 1024u, stream, in, out, n_chunks, ws, static_order, (unsigned)pps, totals, wait_policy(shift, ws));
   if (!scratch.words) stream_free(ws, stream);
   return TCU_OK;
 }
@@ -780,7 +782,7 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
     }
     unsigned *ws = static_cast<unsigned *>(d_ws);
     launch(zero_words_kernel, (unsigned)((words + 255) / 256), 256u, stream, ws, words);
-    TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, mfma, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws, wait_policy());
+    TCU_SWITCH_U_MFMA_NT(full_reduce_kernel, p.u, mfma, nt, (unsigned)grid, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint16_t *>(d_out), n_chunks, ws, wait_policy(0, ws));
     return TCU_OK;
   }
   // the reference's two-kernel sequence: segmented reduction into fp16 totals, then a sum of the totals
@@ -849,12 +851,12 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
     if (lds_held) {  // partitions of 16 x 12 tiles: fewer than `parts`, same workspace layout
       const size_t big_parts = (n_tiles + 16 * 12 - 1) / (16 * 12);
       if (nt)
-        launch(full_scan_lds_kernel<8, 4, true>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy(shift));
+        launch(full_scan_lds_kernel<8, 4, true>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy(shift, ws));
       else
-        launch(full_scan_lds_kernel<8, 4, false>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy(shift));
+        launch(full_scan_lds_kernel<8, 4, false>, (unsigned)big_parts, 1024u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, wait_policy(shift, ws));
       return TCU_OK;
     }
-    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, mfma, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr), wait_policy(shift));
+    TCU_SWITCH_U_MFMA_NT(full_scan_kernel, p.u, mfma, nt, (unsigned)parts, (unsigned)p.wpb * 64u, stream, static_cast<const half8_t *>(d_in), static_cast<uint4_t *>(d_out), n_chunks, ws, options().static_order ? 1 : 0, 0u, static_cast<uint16_t *>(nullptr), wait_policy(shift, ws));
     return TCU_OK;
   }
   // the reference's three-kernel sequence: segmented scan + totals, exclusive scan of the totals, add
@@ -924,11 +926,11 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
   unsigned long long *num_runs = static_cast<unsigned long long *>(d_num_runs);
   const bool nt = options().nontemporal;
   if (reduce) {
-    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, true, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
-    else launch(by_key_kernel<KEY, kByKeyTiles, true, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, true, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift, ws));
+    else launch(by_key_kernel<KEY, kByKeyTiles, true, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift, ws));
   } else {
-    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, false, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
-    else launch(by_key_kernel<KEY, kByKeyTiles, false, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift));
+    if (nt) launch(by_key_kernel<KEY, kByKeyTiles, false, true>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift, ws));
+    else launch(by_key_kernel<KEY, kByKeyTiles, false, false>, grid, block, stream, keys, in, out, keys_out, num_runs, n, ws, so, wait_policy(shift, ws));
   }
   return TCU_OK;
 }

@@ -26,12 +26,6 @@
 
 namespace tcu {
 
-// The look-back scans keep every store non-temporal: alternating the policy by tile as the segmented scans do
-// (kTileStoreNT) made them slower (TCU_FULL_AUTO 2^28 / 2^30: 201 / 762 us against 213-225 / 792-864 us with one
-// store in two, three or four through the cache; events around the call).
-template <bool NT, int J>
-constexpr bool kFullScanStoreNT = NT;
-
 constexpr unsigned long long kFlagAggregate = 1ull << 32;
 constexpr unsigned long long kFlagPrefix = 2ull << 32;
 
@@ -45,7 +39,10 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned *words, size_t
 // every partition's slot; the rest of a slot is never read.
 __global__ __launch_bounds__(256) void zero_look_back_kernel(unsigned *ws, size_t parts, unsigned desc_shift) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i == 0) ws[0] = 0u;
+  if (i == 0) {
+    ws[0] = 0u;
+    ws[1] = 0u;  // waits that gave up (WaitPolicy::expired)
+  }
   if (i < parts) {
     unsigned *slot = ws + 64 + 2 * (i << desc_shift);
     slot[0] = 0u;
@@ -88,23 +85,33 @@ constexpr unsigned long long kPublished = 1ull << 32;
 // descriptors (shift 0) put 16 partitions into one 128-byte line that hundreds of waiting waves poll while
 // its owners keep storing into it; one descriptor per 256 bytes (shift 5) took the full-array scan of 2^28
 // halves from 212 to 191 us.
+// expired: device word (may be null) that counts the waits that gave up, so that a caller can tell without
+// looking for NaN in the output; the workspace-taking entry points pass word 1 of the workspace.
 struct WaitPolicy {
   unsigned poll_limit;
   unsigned mute_partition;
   unsigned desc_shift;
+  unsigned *expired;
 };
+// called by every lane of the wave whose wait expired
+TCU_DEVICE void note_expired_wait(const WaitPolicy &wait, int lane) {
+  if (lane == 0 && wait.expired != nullptr) atomic_add_u32(wait.expired, 1u);
+}
 constexpr unsigned kDefaultPollLimit = 1u << 20;
 constexpr unsigned kDescShift = 5;
 
 
 // sum over lanes of the published values at p[lane], lane < count (count <= 64); false if a
 // value never showed up
-TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, int lane, float *sum, unsigned poll_limit) {
+TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, int lane, float *sum, const WaitPolicy &wait) {
   unsigned long long d = kPublished;
   for (unsigned polls = 0;; polls++) {
     if ((unsigned)lane < count) d = atomic_load_u64(p + lane);
     if (ballot((d >> 32) == 1ull) == ~0ull) break;
-    if (polls >= poll_limit) return false;
+    if (polls >= wait.poll_limit) {
+      note_expired_wait(wait, lane);
+      return false;
+    }
     spin_pause();
   }
   const float v = (unsigned)lane < count ? __uint_as_float((unsigned)d) : 0.0f;
@@ -151,14 +158,14 @@ __global__ __launch_bounds__(kMaxBlock) void full_reduce_kernel(const half8_t *_
   if (b != first + members - 1) return;  // wave-uniform: only a group's last block goes on
   const float failed = __builtin_nanf("");  // a published value never became visible
   float gs;
-  if (!gather_published(partials + first, members, lane, &gs, wait.poll_limit)) gs = failed;
+  if (!gather_published(partials + first, members, lane, &gs, wait)) gs = failed;
   if (lane == 0) atomic_store_u64(group_sum + g, kPublished | __float_as_uint(gs));
   if (g != n_groups - 1) return;  // wave-uniform: only the last block of the grid goes on
   float t = 0.0f;
   for (unsigned base = 0; base < n_groups; base += 64) {
     const unsigned count = n_groups - base < 64 ? n_groups - base : 64;
     float part;
-    if (!gather_published(group_sum + base, count, lane, &part, wait.poll_limit)) part = failed;
+    if (!gather_published(group_sum + base, count, lane, &part, wait)) part = failed;
     t += part;
   }
   if (lane == 0) out[0] = t != t ? (uint16_t)0x7e00u : f16_bits(t);
@@ -183,7 +190,10 @@ TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long 
     const int first_prefix = is_prefix ? __builtin_ctzll(is_prefix) : 64;
     const unsigned long long needed = first_prefix >= 63 ? ~0ull : ((2ull << first_prefix) - 1ull);
     if (is_empty & needed) {
-      if (polls++ >= wait.poll_limit) return __builtin_nanf("");  // never spin without bound
+      if (polls++ >= wait.poll_limit) {  // never spin without bound
+        note_expired_wait(wait, lane);
+        return __builtin_nanf("");
+      }
       spin_pause();
       continue;
     }
@@ -211,7 +221,8 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   const int WPB = (int)(blockDim.x >> 6);
   unsigned long long *desc = reinterpret_cast<unsigned long long *>(ws + 64);
   ScanOperands ops;
-  if constexpr (MFMA) ops = make_scan_operands(lane);
+  if constexpr (MFMA) ops = make_scan_operands<6>(lane);
+  const int chunk_lane = MFMA ? matrix_chunk_of_lane(lane) : lane;
 
   if (!static_order) {
     if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
@@ -221,7 +232,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   const size_t t0 = ((size_t)part * WPB + wave) * U;
 
   half8_t v[U];
-  load_tiles<U, NT>(v, in, t0 * kTileChunks, n_chunks, lane);
+  load_tiles<U, NT>(v, in, t0 * kTileChunks, n_chunks, chunk_lane);
   float acc = 0.0f;
 #pragma unroll
   for (int j = 0; j < U; j++) acc = sum8(v[j], acc);
@@ -255,7 +266,7 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   static_for<U>([&](auto J) {
     constexpr int j = decltype(J)::value;
     float tile_total;
-    scan_tile<6, MFMA, kFullScanStoreNT<NT, j>>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    scan_tile<6, MFMA, NT>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
     carry += tile_total;
   });
 }
@@ -329,14 +340,14 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_lds_kernel(const half8_t 
   static_for<U>([&](auto J) {
     constexpr int j = decltype(J)::value;
     float tile_total;
-    scan_tile<6, false, kFullScanStoreNT<NT, j>>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    scan_tile<6, false, NT>(v[j], carry, ops, lane, out, (t0 + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
     carry += tile_total;
   });
   static_for<ULDS>([&](auto J) {
     constexpr int j = decltype(J)::value;
     float tile_total;
     const half8_t h = *reinterpret_cast<const half8_t *>(mine + j * kTileHalves + lane * 8);
-    scan_tile<6, false, kFullScanStoreNT<NT, U + j>>(h, carry, ops, lane, out, (t0 + U + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
+    scan_tile<6, false, NT>(h, carry, ops, lane, out, (t0 + U + j) * kTileChunks, n_chunks, nullptr, 0, 0, &tile_total);
     carry += tile_total;
   });
 }

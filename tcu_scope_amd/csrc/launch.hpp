@@ -6,6 +6,7 @@
 #include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <mutex>
 
 namespace tcu {
@@ -45,7 +46,13 @@ inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void
 // request into a real allocation of a millisecond or more.  The block may be used by work
 // enqueued on `stream` between stream_alloc and stream_free.  The pool is that of the stream's
 // device (of the current device for the default stream).
+// how many times the library has asked for temporary device memory (process-wide; tcu_temporary_allocations)
+inline std::atomic<unsigned long> &stream_alloc_count() {
+  static std::atomic<unsigned long> n{0};
+  return n;
+}
 inline void *stream_alloc(size_t bytes, void *stream) {
+  stream_alloc_count()++;
   constexpr int kMaxDevices = 64;
   static hipMemPool_t pools[kMaxDevices] = {};
   static std::mutex pools_mutex;

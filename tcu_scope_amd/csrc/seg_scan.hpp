@@ -9,18 +9,21 @@
 // Flavour MFMA = false does 1 and 3 with packed fp16 dot products in the owning lane and
 // 2 with DPP row shifts / broadcasts (the counterpart of the reference's cub::WarpScan /
 // cub::BlockScan rows, src/prefixsum/seg_cub_warp.cu:17-27, seg_cub_block.cu:13-51).
-// Flavour MFMA = true takes the tile as the B operand of v_mfma_f32_16x16x32_f16:
-//   1. D0 = P * X with P[m][k] = [k/8 == m%4]: every lane of column n gets the four
-//      totals of chunks n, 16+n, 32+n, 48+n;
-//   3. D1 = U1 * X + C1 and D2 = U2 * X + C2 with block upper-triangular ones
-//      U1[m][k] = [k/8 == m/8][k%8 <= m%8], U2[m][k] = [k/8 == 2 + m/8][k%8 <= m%8] and the
-//      carries E broadcast in the accumulator inputs C1/C2 — scan == multiplication by a
-//      triangular ones matrix with the cross-tile carry entering through the accumulator,
-//      the formulation of reference src/prefixsum/kernel.cuh:48-83 (seg 16), :87-150
-//      (16n), :303-363 (256: L*A*O + A*U), :442-506 (256n, carry via fill_fragment);
-//   2. stays on DPP, on the four replicated totals.
-// Lane (n, g) of D1/D2 holds 4 consecutive outputs of chunk (n, g/2) / (n, 2 + g/2); two
-// v_permlane16_swap turn that into one 128-bit store per lane.
+// Flavour MFMA = true is the scan as a product with constant triangular matrices, the formulation of reference
+// src/prefixsum/kernel.cuh:48-83 (seg 16: A * U), :303-363 (seg 256: L * A * O + A * U) and :442-506 (256n: the
+// carry enters through the accumulator), on v_mfma_f32_16x16x32_f16.  The tile is read as 16 runs of 32 consecutive
+// halves: lane (n, b) = (lane % 16, lane / 16) holds chunk 4 n + b, which makes the tile the 32 x 16 B operand
+// X[k][n] = x[32 n + k] (and, in the same registers, its transpose as a 16 x 32 A operand).
+//   3. D1 = A1 * X + C, D2 = A2 * X + C with A1[m][k] = [k <= m], A2[m][k] = [k <= 16 + m] (for 16-half segments
+//      A2[m][k] = [16 <= k <= 16 + m]): D1[m][n], D2[m][n] are the inclusive prefixes at positions m and 16 + m of
+//      run n -- U^T * X, the transpose of the reference's A * U;
+//   1./2. for segments of more than one run, the carries C: Q = X^T * J (J all ones) gives every run's total (the
+//      reference's "* O"), T * R with R[n'][n] = [n' < n, same segment] the sum of the runs in front of run n inside
+//      its segment (the reference's strictly triangular "L *"), with what entered the tile as that product's own
+//      accumulator input.  T holds the totals as operands: fp32 totals split into two fp16 parts (hi + lo, 22 bits)
+//      that sit in different k slots, so that the product is formed from exact 0/1 weights and loses nothing that the
+//      fp16 result could show.  No DPP, no LDS; four lane swaps put the 16-byte pieces of the result back into the
+//      lanes that loaded them.
 #pragma once
 
 #include "seg_reduce.hpp"
@@ -94,24 +97,35 @@ TCU_DEVICE uint4_t chunk_scan_packed(half8_t v, float e) {
   return r;
 }
 
-// Constant A operands of the MFMA flavour (see the header comment).
+// The chunk of its tile that a lane holds in the matrix flavour (see the header comment); the DPP flavour and the
+// reductions use chunk == lane.
+TCU_DEVICE int matrix_chunk_of_lane(int lane) { return 4 * (lane & 15) + (lane >> 4); }
+
+// Constant operands of the matrix flavour (see the header comment), built from the lane id.
 struct ScanOperands {
-  half8_t totals;  // P
-  half8_t tri_lo;  // U1
-  half8_t tri_hi;  // U2
+  half8_t tri_lo;  // A1
+  half8_t tri_hi;  // A2
+  half8_t ones;    // J
+  half8_t strict;  // R, rows in the order of the k slots of T: blocks 0 / 1 = hi / lo parts of totals 0..7, blocks 2 / 3 of totals 8..15
 };
+template <int LPS_LOG2>
 TCU_DEVICE ScanOperands make_scan_operands(int lane) {
   const int m = lane & 15, b = lane >> 4;
+  constexpr int RPS = LPS_LOG2 >= 3 ? (1 << (LPS_LOG2 - 2)) : 1;  // runs of 32 halves per segment (inside a tile)
   ScanOperands o;
-  o.totals = splat8(b == (m & 3) ? 1.0f : 0.0f);
-  half8_t lo, hi;
+  half8_t lo, hi, st;
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    lo[i] = (half_t)((b == (m >> 3) && i <= (m & 7)) ? 1.0f : 0.0f);
-    hi[i] = (half_t)((b == 2 + (m >> 3) && i <= (m & 7)) ? 1.0f : 0.0f);
+  for (int e = 0; e < 8; e++) {
+    const int k = 8 * b + e;
+    lo[e] = (half_t)(k <= m ? 1.0f : 0.0f);
+    hi[e] = (half_t)((k <= 16 + m && (LPS_LOG2 > 1 || k >= 16)) ? 1.0f : 0.0f);
+    const int run = 8 * (b >> 1) + e;  // the run whose total sits in slot k of T; as a B operand this lane is column m
+    st[e] = (half_t)((run < m && run / RPS == m / RPS) ? 1.0f : 0.0f);
   }
   o.tri_lo = lo;
   o.tri_hi = hi;
+  o.ones = splat8(1.0f);
+  o.strict = st;
   return o;
 }
 
@@ -141,58 +155,58 @@ TCU_DEVICE void scan_tile(half8_t v, float carry, const ScanOperands &ops, int l
       }
     }
   } else {
+    // lane (n, g): v = chunk 4 n + g of the tile (matrix_chunk_of_lane)
     const int n = lane & 15, g = lane >> 4;
-    const float4_t zero = {0, 0, 0, 0};
-    const float4_t T = mfma_16x16x32(ops.totals, v, zero);  // T[i] = total of chunk 16*i + n
-    float e[4];
-    if constexpr (LPS_LOG2 <= 4) {
-#pragma unroll
-      for (int i = 0; i < 4; i++) e[i] = row_group_exclusive_scan<LPS_LOG2>(T[i], n);
-      *tile_total = 0.0f;
-      if (totals != nullptr && g == 0 && (n & (LPS - 1)) == LPS - 1) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const size_t s = tile_seg0 + (size_t)((16 * i + n) >> LPS_LOG2);
-          if (s < num_segments) totals[s] = f16_bits(e[i] + T[i]);
-        }
-      }
-    } else {
-      float rowsum[4];
+    float4_t c = {0, 0, 0, 0};
+    if constexpr (LPS_LOG2 >= 3) {
+      // totals of the 16 runs: lane (*, g) gets those of runs 4 g .. 4 g + 3
+      const float4_t q = mfma_16x16x32(v, ops.ones, c);
+      // the same as an A operand: rows g = 0, 1 take the totals of runs 0..7, rows 2, 3 those of runs 8..15
+      unsigned ta[4], tb[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        e[i] = row_group_exclusive_scan<4>(T[i], n);
-        rowsum[i] = readlane(e[i] + T[i], 15);
+        ta[i] = tb[i] = __float_as_uint(q[i]);
+        permlane16_swap(ta[i], tb[i]);  // ta = total of run 8 (g / 2) + i, tb = of run 8 (g / 2) + 4 + i
       }
-      if constexpr (LPS_LOG2 == 5) {
-        e[1] += rowsum[0];
-        e[3] += rowsum[2];
-        *tile_total = 0.0f;
-        if (totals != nullptr && lane < 2) {
-          const size_t s = tile_seg0 + (size_t)lane;
-          if (s < num_segments) totals[s] = f16_bits(lane == 0 ? rowsum[0] + rowsum[1] : rowsum[2] + rowsum[3]);
+      half8_t t;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const float x = __uint_as_float(i < 4 ? ta[i] : tb[i - 4]);
+        const half_t hi = (half_t)x;
+        const half_t lo = (half_t)(x - (float)hi);
+        t[i] = (g & 1) ? lo : hi;
+      }
+      const float in = LPS_LOG2 == 6 ? carry : 0.0f;
+      c = mfma_16x16x32(t, ops.strict, float4_t{in, in, in, in});  // every row: what precedes run n inside its segment
+    }
+    const float4_t d1 = mfma_16x16x32(ops.tri_lo, v, c);
+    const float4_t d2 = mfma_16x16x32(ops.tri_hi, v, c);
+    if constexpr (LPS_LOG2 == 6) {
+      *tile_total = readlane(d2[3], 63) - carry;  // the last prefix of the tile is what enters the next one
+    } else {
+      *tile_total = 0.0f;
+      if (totals != nullptr && g == 3) {  // lane (n, 3) holds the last prefix of both halves of run n
+        if constexpr (LPS_LOG2 == 1) {
+          const size_t s = tile_seg0 + 2 * (size_t)n;
+          if (s < num_segments) totals[s] = f16_bits(d1[3]);
+          if (s + 1 < num_segments) totals[s + 1] = f16_bits(d2[3]);
+        } else {
+          constexpr int RPS = LPS_LOG2 >= 3 ? (1 << (LPS_LOG2 - 2)) : 1;
+          const size_t s = tile_seg0 + (size_t)(n / RPS);
+          if ((n % RPS) == RPS - 1 && s < num_segments) totals[s] = f16_bits(d2[3]);
         }
-      } else {
-        const float r01 = rowsum[0] + rowsum[1];
-        e[0] += carry;
-        e[1] += carry + rowsum[0];
-        e[2] += carry + r01;
-        e[3] += carry + (r01 + rowsum[2]);
-        *tile_total = r01 + (rowsum[2] + rowsum[3]);
       }
     }
-    const float c1 = g < 2 ? e[0] : e[1];
-    const float c2 = g < 2 ? e[2] : e[3];
-    const float4_t d1 = mfma_16x16x32(ops.tri_lo, v, float4_t{c1, c1, c1, c1});
-    const float4_t d2 = mfma_16x16x32(ops.tri_hi, v, float4_t{c2, c2, c2, c2});
+    // lane (n, g) holds positions 4 g .. 4 g + 3 (d1) and 16 + 4 g .. (d2) of run n; it stores positions 8 g .. 8 g + 7
     unsigned a_lo = pack_f16x2(d1[0], d1[1]), a_hi = pack_f16x2(d1[2], d1[3]);
     unsigned b_lo = pack_f16x2(d2[0], d2[1]), b_hi = pack_f16x2(d2[2], d2[3]);
+    permlane32_swap(a_lo, b_lo);
+    permlane32_swap(a_hi, b_hi);
     permlane16_swap(a_lo, b_lo);
     permlane16_swap(a_hi, b_hi);
-    // rows 0..3 now hold chunks n, 32+n, 16+n, 48+n
-    const int dst = n + 16 * (((g & 1) << 1) | (g >> 1));
-    const size_t c = chunk_base + dst;
+    const size_t cidx = chunk_base + (size_t)matrix_chunk_of_lane(lane);
     const uint4_t r = {a_lo, a_hi, b_lo, b_hi};
-    if (c < n_chunks) store_chunk<NT>(out + c, r);
+    if (cidx < n_chunks) store_chunk<NT>(out + cidx, r);
   }
 }
 
@@ -210,14 +224,15 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_wave_kernel(const half8_t 
   if (tile0 * kTileChunks >= n_chunks) return;
   const size_t tmask = ((size_t)1 << tiles_per_seg_log2) - 1;
   ScanOperands ops;
-  if constexpr (MFMA) ops = make_scan_operands(lane);
+  if constexpr (MFMA) ops = make_scan_operands<LPS_LOG2>(lane);
+  const int chunk_lane = MFMA ? matrix_chunk_of_lane(lane) : lane;  // the chunk of a tile this lane loads
   constexpr int SEGS_PER_TILE = 64 >> LPS_LOG2;
 
   float carry = 0.0f;
   for (unsigned it = 0; it < iters; it++) {
     const size_t t_it = tile0 + (size_t)it * U;
     half8_t v[U];
-    load_tiles<U, NT != 0>(v, in, t_it * kTileChunks, n_chunks, lane);
+    load_tiles<U, NT != 0>(v, in, t_it * kTileChunks, n_chunks, chunk_lane);
     static_for<U>([&](auto J) {
       constexpr int j = decltype(J)::value;
       const size_t t = t_it + j;
@@ -252,7 +267,8 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
   const int G = (int)waves_per_seg, Q = WPB / G;  // waves per segment, segments in flight
   const int q = wave / G, wg = wave % G;           // this wave's group, and its place in the group
   ScanOperands ops;
-  if constexpr (MFMA) ops = make_scan_operands(lane);
+  if constexpr (MFMA) ops = make_scan_operands<6>(lane);
+  const int chunk_lane = MFMA ? matrix_chunk_of_lane(lane) : lane;
   unsigned parity = 0;
   const size_t piece = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run);
   for (unsigned sb = 0; sb < segs_per_block; sb += (unsigned)Q) {
@@ -267,7 +283,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_block_kernel(const half8_t
     for (size_t step0 = 0; step0 < tiles_per_seg; step0 += (size_t)G * U) {
       const size_t t0 = step0 + (size_t)wg * U;  // first tile of this wave (may lie past the segment)
       half8_t v[U];
-      load_tiles<U, NT != 0>(v, in, (tile_base + t0) * kTileChunks, t0 < tiles_per_seg ? lim : 0, lane);
+      load_tiles<U, NT != 0>(v, in, (tile_base + t0) * kTileChunks, t0 < tiles_per_seg ? lim : 0, chunk_lane);
       // pass 1: this wave's total
       float acc = 0.0f;
 #pragma unroll
@@ -332,7 +348,7 @@ __global__ __launch_bounds__(256) void add_partial_sums_kernel(uint4_t *out, con
   half8_t v = load_chunk<NT>(reinterpret_cast<const half8_t *>(out + c));
   uint4_t r = {pack_f16x2((float)v[0] + ps, (float)v[1] + ps), pack_f16x2((float)v[2] + ps, (float)v[3] + ps), pack_f16x2((float)v[4] + ps, (float)v[5] + ps),
                pack_f16x2((float)v[6] + ps, (float)v[7] + ps)};
-  store_chunk_alternating<NT>(out + c, r);
+  store_chunk<NT>(out + c, r);
 }
 __global__ __launch_bounds__(256) void add_partial_sums_generic_kernel(uint16_t *out, const uint16_t *partial_sums, size_t n, size_t segment_size, int shifted) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -396,10 +412,7 @@ __global__ __launch_bounds__(256) void seg_scan_offsets_kernel(const uint16_t *i
     carry += lane_group_sum<G_LOG2>(t);
     const uint4_t packed = chunk_scan_packed(v, start);
     if (full) {
-      if constexpr (G_LOG2 >= 4)
-        store_chunk_alternating<NT>(out8 + c, packed);
-      else  // few lanes per segment: 176 us with every store non-temporal, 190 us alternating (N = 2^28, 16 halves per segment)
-        store_chunk<NT>(out8 + c, packed);
+      store_chunk<NT>(out8 + c, packed);
     } else if (any) {
 #pragma unroll
       for (int i = 0; i < 8; i++)
@@ -514,7 +527,7 @@ __global__ __launch_bounds__(kMaxBlock) void seg_scan_offsets_sliced_kernel(cons
     const uint4_t packed = chunk_scan_packed(v, carry + before + excl);
     carry += all;
     if (full) {
-      store_chunk_alternating<NT>(reinterpret_cast<uint4_t *>(out) + c, packed);
+      store_chunk<NT>(reinterpret_cast<uint4_t *>(out) + c, packed);
     } else if (any) {
       const size_t lo = c * 8;
 #pragma unroll

@@ -138,34 +138,19 @@ TCU_DEVICE void store_chunk(uint4_t *p, uint4_t v) {
     *p = v;
 }
 
-// Streaming kernels that write as much as they read (the scans) alternate their stores: tile 0, 2, ... of a wave go
-// out non-temporal, tile 1, 3, ... through the cache, while all loads stay non-temporal.  Measured on the segmented
-// scan of 2^28 halves (HIP events around the call, every assignment of the two policies to the 2 or 4 tiles of a wave):
-// all stores non-temporal 171 us (2 tiles per wave) / 176 us (4), all through the cache 173 / 188, every other one
-// 153-156 / 162, three of four through the cache 188; alternating the LOADS instead (stores non-temporal) 155 / 170,
-// alternating both 172 / 180.  The two kinds of store drain through different paths, and using both is worth 9 %.
-// Kernels that only read gain nothing from mixing their loads (segmented reduction: 72-82 us with all loads
-// non-temporal, 73-104 us with every other one through the cache), and the look-back scans lose (full_array.hpp).
-// The NT template argument of the scan kernels and of the copy probe names one of three policies (all loads are
-// non-temporal unless it is 0): 0 = every access through the cache, 1 = the alternation above (a bool `true`
-// converts to it), 2 = every store non-temporal.
+// Store policies of the scan kernels and of the copy probe (the value of their NT template argument; all loads are
+// non-temporal unless it is 0): 0 = every access through the cache, 1 = tile 0, 2, ... of a wave stored
+// non-temporally and tile 1, 3, ... through the cache, 2 = every store non-temporal (the default).
+// What the alternation buys depends on where the output goes.  Segmented scan of 2^28 halves, kernel times: with ONE
+// 512 MiB output buffer that every launch rewrites, alternating stores run at 143-146 us against 160-169 us for
+// all non-temporal -- the cached half of the output is exactly the 256 MiB of the memory-side cache, stays there
+// dirty and is overwritten by the next launch before it has to be written to HBM.  With three or five output
+// buffers taken in turn (or one 2 GiB output at 2^30 halves), i.e. when every byte written has to reach HBM, the
+// same kernels take 161-174 us alternating and 160-169 us all non-temporal, and 172-182 us all cached.  Policy 1
+// is therefore kept for callers whose output is consumed from that cache, and is not the default.
 constexpr int kStoreCached = 0, kStoreAlternate = 1, kStoreStream = 2;
 template <int NT, int J>
 constexpr bool kTileStoreNT = NT == kStoreStream || (NT == kStoreAlternate && J % 2 == 0);
-
-// The same alternation where a tile's place in its wave is not known at compile time: the odd 1 KiB blocks of the
-// output go through the cache.  Written as assembly because the compiler merges two stores that differ only in
-// their cache policy into one store without the hint.
-template <bool NT>
-TCU_DEVICE void store_chunk_alternating(uint4_t *p, uint4_t v) {
-  if constexpr (!(NT && TCU_STORE_NT)) {
-    *p = v;
-  } else if ((reinterpret_cast<uintptr_t>(p) >> 10) & 1u) {
-    asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(p), "v"(v) : "memory");
-  } else {
-    asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(p), "v"(v) : "memory");
-  }
-}
 
 // f(Int<0>{}), f(Int<1>{}), ..., f(Int<N-1>{}): a loop whose index is a compile-time constant in the body
 template <int V>

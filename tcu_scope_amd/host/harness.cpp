@@ -1,5 +1,7 @@
 #include "harness.hpp"
 
+#include "../../include/tcu_scope_dev.h"  // --tcu_option
+
 #include <algorithm>
 #include <chrono>
 #include <cmath>

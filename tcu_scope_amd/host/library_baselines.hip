@@ -186,6 +186,35 @@ BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_26)->UseManualT
 BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
 BENCHMARK(CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_30)->UseManualTime();
 
+// The reference builds every CUB baseline twice: against its patched copy of CUB (fp16 shuffle specialisations,
+// CUB_HALF_OPTIMIZATION) and, under the ORIGINAL_CUB_* names, against the unpatched one
+// (src/reduction/cub_original.cu:106, seg_cub_device_original.cu:131-148, src/prefixsum/cub_original.cu:98).  The
+// library this build compares with is hipCUB as ROCm ships it, i.e. unpatched: the ORIGINAL_* device-wide names run
+// the same calls as their twins above.
+static void ORIGINAL_CUB_FULL_REDUCTION(benchmark::State &state) { CUB_FULL_REDUCTION(state); }
+static void ORIGINAL_CUB_FULL_PREFIXSUM(benchmark::State &state) { CUB_FULL_PREFIXSUM(state); }
+static void ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION(benchmark::State &state) { run_device_segmented_reduction(state); }
+static void ORIGINAL_CUB_DEVICE_TUNE_SEGMENTED_REDUCTION(benchmark::State &state) { run_device_segmented_reduction(state); }
+BENCHMARK(ORIGINAL_CUB_FULL_REDUCTION)->ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_FULL_PREFIXSUM)->ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_16_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_32_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_64_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_128_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_256_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_512_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_1024_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_2048_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_4096_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_8192_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_SEGMENTED_REDUCTION)->SEG_16384_ARGS()->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_14)->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_18)->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_22)->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_26)->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
+BENCHMARK(ORIGINAL_CUB_DEVICE_TUNE_SEGMENTED_REDUCTION)->Apply(Tuning16_x_30)->UseManualTime();
+
 // ---- rocBLAS ------------------------------------------------------------------------------------
 namespace {
 rocblas_handle blas() {

@@ -99,6 +99,13 @@ static void CUB_BLOCK_SEGMENTED_PREFIXSUM(benchmark::State &state) {
 }
 RUN_CUB_WARP(CUB_WARP_SEGMENTED_PREFIXSUM);
 RUN_CUB_BLOCK(CUB_BLOCK_SEGMENTED_PREFIXSUM, BLOCK_SCAN_RAKING);
+// the reference's twins on its unpatched copy of CUB (src/prefixsum/seg_cub_warp_original.cu, seg_cub_block_original.cu)
+template <int THREADS_PER_BLOCK, int LOGICAL_WARP_SIZE>
+static void ORIGINAL_CUB_WARP_SEGMENTED_PREFIXSUM(benchmark::State &state) { CUB_WARP_SEGMENTED_PREFIXSUM<THREADS_PER_BLOCK, LOGICAL_WARP_SIZE>(state); }
+template <int THREADS_PER_BLOCK, int ITEMS_PER_THREAD, int ALGORITHM>
+static void ORIGINAL_CUB_BLOCK_SEGMENTED_PREFIXSUM(benchmark::State &state) { CUB_BLOCK_SEGMENTED_PREFIXSUM<THREADS_PER_BLOCK, ITEMS_PER_THREAD, ALGORITHM>(state); }
+RUN_CUB_WARP(ORIGINAL_CUB_WARP_SEGMENTED_PREFIXSUM);
+RUN_CUB_BLOCK(ORIGINAL_CUB_BLOCK_SEGMENTED_PREFIXSUM, BLOCK_SCAN_RAKING);
 
 // ---- full-array prefix sum -----------------------------------------------------------------
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>

@@ -2,6 +2,8 @@
 // streaming kernels that give the machine's copy / read / write ceilings for a launch
 // shape, and launch-shape sweeps of the segmented kernels (kernel family, 1 KiB tiles in
 // flight per wave, waves per block) from which the AUTO launch shapes were chosen.
+// Not part of `bench`: `make bench_probes` builds a second executable that has these names as well.
+#include "../../include/tcu_scope_dev.h"
 #include "args.hpp"
 #include "harness.hpp"
 
@@ -13,22 +15,21 @@ namespace {
 void run_stream_probe(benchmark::State &state, int mode, int tiles_per_wave, int waves_per_block) {
   try {
     const size_t num_elements = state.range(0), bytes = num_elements * 2;
-    // two source/destination pairs alternate so that no launch is served from the Infinity Cache
-    const int nbuf = bytes <= ((size_t)1 << 30) ? 2 : 1;
-    DeviceBuffer src[2] = {DeviceBuffer(bytes), DeviceBuffer(nbuf == 2 ? bytes : 16)};
-    DeviceBuffer dst[2] = {DeviceBuffer(bytes), DeviceBuffer(nbuf == 2 ? bytes : 16)};
-    for (int i = 0; i < nbuf; i++) {
-      harness::fill_input(src[i].get(), num_elements, harness::flags().seed + i);
-      TCU_CHECK(tcu_fill_f16(dst[i].get(), 0.0f, num_elements, nullptr));
-    }
+    // two sources alternate and four destinations take turns, so that no launch is served from the memory-side
+    // cache or overwrites lines an earlier launch left dirty in it
+    const int nbuf = 2, ndst = 4;
+    DeviceBuffer src[2] = {DeviceBuffer(bytes), DeviceBuffer(bytes)};
+    DeviceBuffer dst[4] = {DeviceBuffer(bytes), DeviceBuffer(bytes), DeviceBuffer(bytes), DeviceBuffer(bytes)};
+    for (int i = 0; i < nbuf; i++) harness::fill_input(src[i].get(), num_elements, harness::flags().seed + i);
+    for (int i = 0; i < ndst; i++) TCU_CHECK(tcu_fill_f16(dst[i].get(), 0.0f, num_elements, nullptr));
     TCU_CHECK(tcu_stream_probe(dst[0].get(), src[0].get(), bytes, mode, tiles_per_wave, waves_per_block, nullptr));
     PRINT_IF_ERROR(hipDeviceSynchronize());
     EventPair ev;
     size_t it = 0;
     for (auto _ : state) {
-      const int b = (int)(it++ % nbuf);
+      const size_t i = it++;
       ev.start();
-      TCU_CHECK(tcu_stream_probe(dst[b].get(), src[b].get(), bytes, mode, tiles_per_wave, waves_per_block, nullptr));
+      TCU_CHECK(tcu_stream_probe(dst[i % ndst].get(), src[i % nbuf].get(), bytes, mode, tiles_per_wave, waves_per_block, nullptr));
       const float ms = ev.stop_ms();
       state.PauseTiming();
       state.SetIterationTime(ms / 1000);
@@ -106,20 +107,3 @@ SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_MFMA_16N_BLOCK);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_MFMA_256N_BLOCK);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_WAVE_SHUFFLE);
 SHAPE_FAMILY(TCU_SHAPE_SEGMENTED_PREFIXSUM, TCU_VARIANT_BLOCK_LDS);
-
-// ---- segmented reduction through an offsets array (the hand-written counterpart of the
-// CUB_DEVICE_SEGMENTED_REDUCTION library baseline; same offsets, same argument tuples) ------------
-static void TCU_OFFSETS_SEGMENTED_REDUCTION(benchmark::State &state) { harness::run_seg_reduce_offsets(state, true, "TCU_OFFSETS_SEGMENTED_REDUCTION"); }
-// without the length hint: a whole wave per segment
-static void TCU_OFFSETS_NOHINT_SEGMENTED_REDUCTION(benchmark::State &state) { harness::run_seg_reduce_offsets(state, false, "TCU_OFFSETS_NOHINT_SEGMENTED_REDUCTION"); }
-BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
-BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_256_ARGS()->UseManualTime();
-BENCHMARK(TCU_OFFSETS_SEGMENTED_REDUCTION)->SEG_4096_ARGS()->UseManualTime();
-BENCHMARK(TCU_OFFSETS_NOHINT_SEGMENTED_REDUCTION)->Apply(Tuning16_x_28)->UseManualTime();
-// inclusive prefix sums inside the segments of the same offsets array
-static void TCU_OFFSETS_SEGMENTED_PREFIXSUM(benchmark::State &state) { harness::run_seg_scan_offsets(state, "TCU_OFFSETS_SEGMENTED_PREFIXSUM"); }
-BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->Apply(Tuning16_x_28)->UseManualTime();
-BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->SEG_16_ARGS()->UseManualTime();
-BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->SEG_256_ARGS()->UseManualTime();
-BENCHMARK(TCU_OFFSETS_SEGMENTED_PREFIXSUM)->SEG_2048_ARGS()->UseManualTime();

@@ -110,6 +110,14 @@ static void CUB_BLOCK_SEGMENTED_REDUCTION(benchmark::State &state) {
 }
 RUN_CUB_WARP(CUB_WARP_SEGMENTED_REDUCTION);
 RUN_CUB_BLOCK(CUB_BLOCK_SEGMENTED_REDUCTION, BLOCK_REDUCE_RAKING);
+// The reference's twins on its unpatched copy of CUB (src/reduction/seg_cub_warp_original.cu, seg_cub_block_original.cu):
+// the patch only changes how the library adds halves, which has no counterpart here, so the names run the same kernels.
+template <int THREADS_PER_BLOCK, int LOGICAL_WARP_SIZE>
+static void ORIGINAL_CUB_WARP_SEGMENTED_REDUCTION(benchmark::State &state) { CUB_WARP_SEGMENTED_REDUCTION<THREADS_PER_BLOCK, LOGICAL_WARP_SIZE>(state); }
+template <int THREADS_PER_BLOCK, int ITEMS_PER_THREAD, int ALGORITHM>
+static void ORIGINAL_CUB_BLOCK_SEGMENTED_REDUCTION(benchmark::State &state) { CUB_BLOCK_SEGMENTED_REDUCTION<THREADS_PER_BLOCK, ITEMS_PER_THREAD, ALGORITHM>(state); }
+RUN_CUB_WARP(ORIGINAL_CUB_WARP_SEGMENTED_REDUCTION);
+RUN_CUB_BLOCK(ORIGINAL_CUB_BLOCK_SEGMENTED_REDUCTION, BLOCK_REDUCE_RAKING);
 
 // ---- full-array reduction --------------------------------------------------------------------
 template <int SEGMENT_SIZE, int WARPS_PER_BLOCK>

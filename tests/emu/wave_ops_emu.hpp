@@ -365,10 +365,6 @@ template <bool NT>
 inline void store_chunk(uint4_t *p, uint4_t v) {
   *p = v;
 }
-template <bool NT>
-inline void store_chunk_alternating(uint4_t *p, uint4_t v) {
-  *p = v;
-}
 constexpr int kStoreCached = 0, kStoreAlternate = 1, kStoreStream = 2;
 template <int NT, int J>
 constexpr bool kTileStoreNT = NT == kStoreStream || (NT == kStoreAlternate && J % 2 == 0);

@@ -112,7 +112,11 @@ def test_a_wait_that_expires_gives_nan_not_wrong_numbers(tcu, oracle):
         tcu.set_option("test_mute_partition", mute)
         # (strategy, segment_size, waves) -> halves per partition
         for strategy, seg, w, part in [(S.SINGLE_PASS, 0, 0, 65536), (S.SINGLE_PASS, 8192, 4, 8192), (S.AUTO, 0, 0, 98304), (S.SINGLE_PASS | tcu.FULL_MFMA, 0, 0, 65536)]:
-            got = to_host(tcu.full_scan(xd, strategy, seg, w))
+            ws = torch.zeros(tcu.binding.full_workspace_bytes("scan", n, strategy, seg, w) // 4, dtype=torch.int32, device="cuda")
+            got = to_host(tcu.full_scan(xd, strategy, seg, w, workspace=ws))
+            # word 1 of the workspace counts the waits that gave up: the partition behind the silent one for certain,
+            # later ones only if their own limit ran out before that partition published its NaN prefix
+            assert 1 <= int(ws[1].item()) <= (n + part - 1) // part - mute, f"scan strategy={int(strategy):#x}: expired waits {int(ws[1].item())}"
             good = mute * part
             expect_ok(oracle, got[:good], ref[:good], n, f"scan strategy={int(strategy):#x}: partitions before the silent one")
             assert np.isnan(got[good:].view(np.float16)).all(), f"scan strategy={int(strategy):#x}: data after a wait that expired must be NaN"
@@ -135,7 +139,9 @@ def test_a_wait_that_expires_gives_nan_not_wrong_numbers(tcu, oracle):
         tcu.set_option("test_mute_partition", 0)
         tcu.set_option("lookback_poll_limit", -1)
     # and with the defaults restored the same calls are right again
-    expect_ok(oracle, to_host(tcu.full_scan(xd, S.SINGLE_PASS)), ref, n, "scan after the options were reset")
+    ws = torch.ones(tcu.binding.full_workspace_bytes("scan", n, S.SINGLE_PASS) // 4, dtype=torch.int32, device="cuda")
+    expect_ok(oracle, to_host(tcu.full_scan(xd, S.SINGLE_PASS, workspace=ws)), ref, n, "scan after the options were reset")
+    assert int(ws[1].item()) == 0  # no wait gave up
     expect_ok(oracle, to_host(tcu.full_reduce(xd, S.SINGLE_PASS)), ref[-1:], n, "reduce after the options were reset")
 
 
@@ -395,6 +401,20 @@ def test_gemm_8192(tcu, oracle):
         ref = oracle.gemm_f64(A, B, M, N, K, row0=r, rows=1)
         bad, worst, first = oracle.check_f32_rel(D[r].cpu().numpy(), ref, 1e-2, float(np.sqrt(K)))
         assert bad == 0, (r, bad, worst, first)
+        # the configuration's 1e-2 at the scale of an output (sqrt(K) = 90) would let a dropped product through: fp32
+        # accumulation of K products of fp16 values keeps every output within 1e-4 * sqrt(K) of the fp64 product
+        bad, worst, first = oracle.check_f32_rel(D[r].cpu().numpy(), ref, 1e-4, float(np.sqrt(K)))
+        assert bad == 0, ("tight", r, bad, worst, first)
+    # exact: small integers as inputs ({0, 1, 2}, the reference's rand() % 3 fill, src/gemm/wmma.cu:110-127) make every
+    # fp32 partial sum exact (outputs <= 4 * 8192 < 2^24), so the default kernel must give the fp64 product bit for bit
+    Ai = tcu.generate(M * K, 14, tcu.Dist.SMALLINT).view(M, K)
+    Bi = tcu.generate(N * K, 15, tcu.Dist.SMALLINT).view(N, K)
+    Di = tcu.gemm(Ai, Bi)
+    torch.cuda.synchronize()
+    Aih, Bih = to_host(Ai).ravel(), to_host(Bi).ravel()
+    for r in rows[::3]:
+        ref = oracle.gemm_f64(Aih, Bih, M, N, K, row0=r, rows=1)
+        assert np.array_equal(Di[r].cpu().numpy().astype(np.float64), np.asarray(ref).ravel()), ("exact integers", r)
     # fp16 C and D with the benchmark's alpha and beta (reference src/gemm/wmma.cu:679-680)
     Ch = tcu.generate(M * N, 13, tcu.Dist.NORMAL).view(M, N)
     C32 = to_host(Ch).ravel().view(np.float16).astype(np.float32)

@@ -79,6 +79,28 @@ def test_exact_grid_inputs_bitwise(tcu, oracle, seg):
         assert np.array_equal(to_host(tcu.seg_scan(xd, seg, variant=v)), want_scan), f"scan {v.name}"
 
 
+def test_cpu_reference_configuration(tcu, oracle):
+    """The configuration the reference's CPU path is quoted on: N = 2^20 halves, uniform [-1, 1) from seed 0,
+    contiguous segments of 16 (65536 segments), fp32 accumulation, one fp16 result per segment.  Every family that
+    takes 16-half segments against the fp64 sums within the stated tolerance, and against the CPU path itself
+    (fp32 running sum, one rounding): sums of 16 halves of magnitude below 1 are exact in fp32 in any order, so the
+    two must agree bit for bit."""
+    n, seg = 1 << 20, 16
+    nseg = n // seg
+    x = oracle.generate_f16(n, 0, oracle.DIST_UNIFORM)
+    ref64 = oracle.seg_reduce_f64(x, nseg, seg)
+    cpu_path = oracle.seg_reduce_ref(x, nseg, seg)
+    expect_ok(oracle, cpu_path, ref64, seg, "the CPU path itself")
+    xd = to_dev(x)
+    dev = tcu.generate(n, 0, tcu.Dist.UNIFORM)  # the device generator gives the same input
+    assert np.array_equal(to_host(dev), x)
+    for v in (tcu.Variant.AUTO, tcu.Variant.MFMA_16, tcu.Variant.MFMA_16N, tcu.Variant.WAVE_SHUFFLE, tcu.Variant.MFMA_16N_BLOCK, tcu.Variant.BLOCK_LDS):
+        got = to_host(tcu.seg_reduce(xd, seg, variant=v))
+        assert got.size == 65536
+        expect_ok(oracle, got, ref64, seg, f"configuration 1 {v.name}")
+        assert np.array_equal(got, cpu_path), f"configuration 1 {v.name}: differs from the CPU path"
+
+
 def test_reference_fixture_constant_fill(tcu, oracle):
     """The reference fills its inputs with (half)0.001f; closed forms seg*c and (i+1)*c."""
     import torch

@@ -53,6 +53,37 @@ def _both(tcu, oracle, x16, seg, what, exact):
         assert (np.abs(a - b) <= bound).all(), what + ": the two entry points disagree beyond the tolerance"
 
 
+def test_noalloc_allocates_nothing(tcu, oracle):
+    """The property the entry point is named for, on its look-back path (the only path of tcu_seg_scan_f16 that takes
+    temporary memory): the library's count of temporary allocations and the device's free memory do not move across
+    the call -- made before any other call of this test has warmed the library's memory pool -- while the same
+    call through tcu_seg_scan_f16 does take temporary memory.  On a side stream as well, whose device the scratch
+    array is looked up for."""
+    import torch
+
+    n, seg = 1 << 22, 1 << 21
+    g = oracle.generate_f16(n, 39, oracle.DIST_GRID)
+    xd = to_dev(g)
+    out = torch.empty(n, dtype=torch.float16, device="cuda")
+    want = oracle.seg_scan_f64(g, n // seg, seg).astype(np.float16).view(np.uint16)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):  # the stream's first launch sets up its queue: not part of what is measured
+        out.zero_()
+    torch.cuda.synchronize()
+    for stream in (None, side):
+        allocations, free = tcu.temporary_allocations(), torch.cuda.mem_get_info()[0]
+        tcu.seg_scan_noalloc(xd, seg, out, stream=stream)
+        torch.cuda.synchronize()
+        assert tcu.temporary_allocations() == allocations, "tcu_seg_scan_f16_noalloc took temporary device memory"
+        assert torch.cuda.mem_get_info()[0] == free, "free device memory changed across tcu_seg_scan_f16_noalloc"
+        assert np.array_equal(to_host(out), want)
+        out.zero_()
+    allocations = tcu.temporary_allocations()
+    tcu.seg_scan(xd, seg, out=out)
+    assert tcu.temporary_allocations() == allocations + 1  # the counter does see the allocating entry point
+    assert np.array_equal(to_host(out), want)
+
+
 def test_noalloc_matches_seg_scan_on_two_calls_in_a_row(tcu, oracle):
     # first call: 2^24 halves in 4 segments of 2^22 (256 partitions); second call: 2^22 halves in 2 segments of
     # 2^21 (64 partitions) - fewer descriptors than the first call left behind
