@@ -163,13 +163,17 @@ def main():
     main_buffers = Buffers(n, inputs, red_outs, scan_outs)
     current = [main_buffers]
 
+    turns = {"reduce": 0, "scan": 0}  # launches of each kind so far: a kind's output buffers are taken in turn by its own launches
+
     def launch(i, kind, seg):
         b = current[0]
         x = b.inputs[i % len(b.inputs)]
+        turn = turns[kind] if i else 0  # launch 0 (the checks read its output) writes the first buffer
+        turns[kind] += 1
         if kind == "reduce":
-            tcu.seg_reduce(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=b.red_outs[i % len(b.red_outs)], stream=stream)
+            tcu.seg_reduce(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=b.red_outs[turn % len(b.red_outs)], stream=stream)
         else:
-            tcu.seg_scan(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=b.scan_outs[i % len(b.scan_outs)], stream=stream)
+            tcu.seg_scan(x, seg, variant=variant, tiles_per_wave=args.tiles_per_wave, waves_per_block=args.waves_per_block, out=b.scan_outs[turn % len(b.scan_outs)], stream=stream)
 
     # families do not cover every size (MFMA_16 is 16 only, ...): such launches are left out and said so
     skipped = []

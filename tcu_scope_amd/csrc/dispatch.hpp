@@ -154,9 +154,8 @@ inline int validate_segmented(const char *what, const void *in, const void *out,
   return TCU_OK;
 }
 
-// Launch shapes measured on MI355X at N = 2^28 (timings in profiles/): for each segment
-// size the family and (tiles per wave, waves per block) that moved the most bytes per
-// second.  MFMA and DPP flavours tie within run-to-run noise at every size (the kernels
+// Launch shapes measured on MI355X (timings in profiles/): for each segment size and element
+// count the family and (tiles per wave, waves per block) that moved the most bytes per second.  MFMA and DPP flavours tie within run-to-run noise at every size (the kernels
 // are bound by HBM, not by issue slots), so AUTO takes the DPP flavour.
 struct Plan {
   bool block;  // block-per-segment kernel
@@ -168,24 +167,42 @@ inline unsigned xcd_run_for(const Plan &plan, bool plan_shape) {
   if (options().xcd_run >= 0) return (unsigned)options().xcd_run;
   return plan_shape ? plan.c : 0u;
 }
-inline Plan auto_plan_reduce(size_t S) {
+// N = num_segments * S.  The shapes were measured at N = 2^24, 2^26, 2^28 and 2^30 (randomised sweeps over family,
+// tiles per wave, waves per block and XCD run length with the outputs of the launches taken in turn;
+// profiles/seg_launch_shape_sweeps.md).  From 2^26 elements on one table serves every N but for the entries marked;
+// below 2^25 a launch lasts 6-13 us and is bound by how fast blocks start, so fewer and larger blocks win.
+inline Plan auto_plan_reduce(size_t S, size_t N) {
+  if (N < ((size_t)1 << 25)) {
+    if (S <= 1024) return {false, 2, 1, 128};
+    if (S == 2048) return {false, 2, 1, 8};
+    if (S == 4096) return {false, 4, 4, 0};
+    if (S == 8192) return {false, 8, 1, 512};
+    if (S == 16384) return {true, 4, 16, 0};
+  }
   if (S <= 512) return {false, 2, 1, 512};
   if (S == 1024) return {true, 2, 1, 64};
-  if (S == 2048) return {false, 1, 1, 0};
+  if (S == 2048) return {true, 2, 4, 128};
   if (S == 4096) return {true, 2, 4, 64};
-  if (S == 8192) return {true, 2, 8, 64};
+  if (S == 8192) return {true, 2, 8, 0};
   if (S == 16384) return {true, 2, 8, 64};
   if (S == 65536 || S == 131072) return {true, 2, 16, 32};
   if (S == 262144) return {true, 4, 8, 0};
   if (S > 262144) return {true, 2, 8, 0};
   return {true, 1, 8, 0};
 }
-inline Plan auto_plan_scan(size_t S) {
+inline Plan auto_plan_scan(size_t S, size_t N) {
+  if (N < ((size_t)1 << 25)) {
+    if (S <= 512) return {false, 1, 1, 512};
+    if (S == 1024) return {false, 8, 4, 512};
+    if (S == 2048) return {false, 8, 8, 8};
+    if (S == 4096) return {false, 8, 4, 32};
+    if (S == 8192 || S == 16384) return {true, 8, 8, 8};
+  }
   if (S <= 512) return {false, 2, 1, 512};
-  if (S == 1024) return {false, 2, 2, 256};
+  if (S == 1024) return {true, 1, 1, 128};
   if (S == 2048) return {true, 2, 2, 256};
-  if (S == 4096) return {true, 2, 4, 128};
-  if (S == 8192) return {true, 2, 8, 32};
+  if (S == 4096) return N <= ((size_t)1 << 26) ? Plan{true, 2, 8, 0} : Plan{true, 2, 4, 128};
+  if (S == 8192) return N >= ((size_t)1 << 30) ? Plan{true, 2, 16, 32} : Plan{true, 2, 8, 32};
   if (S == 16384) return {true, 4, 8, 8};
   if (S == 32768) return {true, 8, 8, 16};
   if (S == 65536 || S == 131072) return {true, 4, 16, 32};
@@ -299,21 +316,54 @@ inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned b
 // few bytes per partition of temporary device memory, taken in stream order.
 constexpr size_t kHugeReduceSegment = (size_t)1 << 20, kHugeScanSegment = (size_t)1 << 21, kHugePartHalves = 65536;
 
-// partitions of 65536 halves per XCD in the partition-sum launches (xcd_run_piece)
-inline unsigned partition_sums_run() { return options().xcd_run >= 0 ? (unsigned)options().xcd_run : 0u; }
+// The partition sums (full-array reduction, segments of 2^20 halves and more) take the launch shape that the
+// segmented reduction of 4096-half segments measures fastest: blocks of 4 waves x 2 tiles, every XCD on 128
+// consecutive partitions (0.95-0.97 of 8 TB/s at 2^28 / 2^30 halves; blocks of 16 waves x 8 tiles in launch order,
+// the shape of the look-back scan, gave 0.83-0.85).  One fp32 partial per 4096 halves.
+constexpr int kSumTiles = 2, kSumWaves = 4;
+constexpr size_t kSumPartHalves = (size_t)kSumTiles * kSumWaves * kTileHalves;
+inline unsigned partition_sums_run() { return options().xcd_run >= 0 ? (unsigned)options().xcd_run : 128u; }
+// out[j] = fp16(sum of the pps partials of segment j), j < num_segments.  A block adds up to kSumLevel partials;
+// longer rows of partials are first cut into pieces of kSumLevel whose fp32 sums are written behind the partials
+// (one block walking 262144 partials takes 21 us, two levels 8 us), so `partials` has room for
+// sum_partials_floats(num_segments, pps) floats.
+constexpr size_t kSumLevel = 4096;
+inline size_t sum_partials_floats(size_t num_segments, size_t pps) {
+  const size_t parts = num_segments * pps;
+  return pps > 2 * kSumLevel ? parts + num_segments * ((pps + kSumLevel - 1) / kSumLevel) : parts;
+}
+inline void launch_sum_of_partials(void *stream, float *partials, uint16_t *out, size_t num_segments, size_t pps) {
+  const size_t parts = num_segments * pps;
+  if (pps > 2 * kSumLevel && pps % kSumLevel == 0) {  // whole pieces per segment: the pieces of all segments in one launch
+    float *second = partials + parts;
+    const size_t pieces = pps / kSumLevel;
+    launch(segment_of_partials_kernel<float>, (unsigned)(num_segments * pieces), 1024u, stream, static_cast<const float *>(partials), second, kSumLevel, parts);
+    launch(segment_of_partials_kernel<uint16_t>, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(second), out, pieces, num_segments * pieces);
+  } else if (pps > 2 * kSumLevel && num_segments == 1) {
+    float *second = partials + parts;
+    const size_t pieces = (pps + kSumLevel - 1) / kSumLevel;
+    launch(segment_of_partials_kernel<float>, (unsigned)pieces, 1024u, stream, static_cast<const float *>(partials), second, kSumLevel, parts);
+    launch(segment_of_partials_kernel<uint16_t>, 1u, 1024u, stream, static_cast<const float *>(second), out, pieces, pieces);
+  } else {
+    launch(segment_of_partials_kernel<uint16_t>, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(partials), out, pps, parts);
+  }
+}
+inline void launch_partition_sums(bool nt, size_t parts, void *stream, const half8_t *in, float *partials, size_t n_chunks) {
+  if (nt)
+    launch(partition_sums_kernel<kSumTiles, true>, (unsigned)parts, (unsigned)kSumWaves * 64u, stream, in, partials, n_chunks, partition_sums_run());
+  else
+    launch(partition_sums_kernel<kSumTiles, false>, (unsigned)parts, (unsigned)kSumWaves * 64u, stream, in, partials, n_chunks, partition_sums_run());
+}
 
 inline int seg_reduce_huge(const half8_t *in, uint16_t *out, size_t num_segments, size_t S, bool nt, void *stream) {
   const char *what = "tcu_seg_reduce_f16";
-  const size_t pps = S / kHugePartHalves, parts = num_segments * pps;
+  const size_t pps = S / kSumPartHalves, parts = num_segments * pps;
   if (parts > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-  float *partials = static_cast<float *>(stream_alloc(parts * sizeof(float), stream));
+  float *partials = static_cast<float *>(stream_alloc(sum_partials_floats(num_segments, pps) * sizeof(float), stream));
   if (!partials) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partition sums");
   const size_t n_chunks = num_segments * S / 8;
-  if (nt)
-    launch(partition_sums_kernel<8, true>, (unsigned)parts, 1024u, stream, in, partials, n_chunks, partition_sums_run());
-  else
-    launch(partition_sums_kernel<8, false>, (unsigned)parts, 1024u, stream, in, partials, n_chunks, partition_sums_run());
-  launch(segment_of_partials_kernel, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(partials), out, pps);
+  launch_partition_sums(nt, parts, stream, in, partials, n_chunks);
+  launch_sum_of_partials(stream, partials, out, num_segments, pps);
   stream_free(partials, stream);
   return TCU_OK;
 }
@@ -372,7 +422,7 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
   }
   if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeReduceSegment) return seg_reduce_huge(in, out, num_segments, S, nt, stream);
   const size_t n_chunks = N / 8;
-  const Plan plan = auto_plan_reduce(S);
+  const Plan plan = auto_plan_reduce(S, N);
   // A segment shorter than a tile cannot be shared by the waves of a block: below 512 halves the block families
   // run the kernels whose waves take whole tiles, at the block's launch shape (waves per block x tiles per wave)
   const bool use_block = S >= kTileHalves && (variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant));
@@ -438,7 +488,7 @@ inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t nu
       launch(seg_reduce_offsets_sliced_kernel<OFF, true>, (unsigned)blocks, 1024u, stream, in, partials, begin, end, (unsigned)slices, vector);
     else
       launch(seg_reduce_offsets_sliced_kernel<OFF, false>, (unsigned)blocks, 1024u, stream, in, partials, begin, end, (unsigned)slices, vector);
-    launch(segment_of_partials_kernel, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(partials), out, slices);
+    launch(segment_of_partials_kernel<uint16_t>, (unsigned)num_segments, 1024u, stream, static_cast<const float *>(partials), out, slices, blocks);
     stream_free(partials, stream);
     return TCU_OK;
   }
@@ -564,7 +614,7 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
   }
   if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeScanSegment) return seg_scan_huge(what, in, out, totals, num_segments, S, nt, stream, scratch);
   const size_t n_chunks = N / 8;
-  const Plan plan = auto_plan_scan(S);
+  const Plan plan = auto_plan_scan(S, N);
   const bool use_block = S >= kTileHalves && (variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant));  // as in the reduction
   const bool plan_fits = variant == TCU_VARIANT_AUTO || plan.block == use_block;
   const int wpb = waves_per_block ? waves_per_block : (plan_fits ? plan.w : (use_block ? 4 : 1));
@@ -742,8 +792,7 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
   const bool mfma = (strategy & TCU_FULL_MFMA) != 0;
   strategy &= ~TCU_FULL_MFMA;
   if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
-  // AUTO with the default partition: partition sums, then one small block adds them (measured
-  // 81 us at 2^28 against 86 us for the single kernel, whose workspace must be zeroed first)
+  // AUTO with the default partition: partition sums, then one block adds them
   const bool two_level = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && !mfma;
   if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
   const bool nt = options().nontemporal;
@@ -758,7 +807,10 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
     const size_t groups = (grid + kFullReduceGroup - 1) / kFullReduceGroup;
     const size_t counter_words = 64 + ((groups + 1) & ~(size_t)1);
     const size_t words = counter_words + 2 * (grid + groups);
-    const size_t need = round_up(4 * words, kWorkspaceAlign);
+    // the two-launch form keeps one float per 4096 halves in the workspace
+    const size_t sum_parts = (n + kSumPartHalves - 1) / kSumPartHalves;
+    const size_t sum_floats = sum_partials_floats(1, sum_parts ? sum_parts : 1);
+    const size_t need = round_up(two_level && sum_floats > words ? 4 * sum_floats : 4 * words, kWorkspaceAlign);
     if (!d_ws) {
       *ws_bytes = need;
       return TCU_OK;
@@ -771,13 +823,11 @@ inline int full_reduce_dispatch(const void *d_in, void *d_out, size_t n, void *d
       return TCU_OK;
     }
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
-    if (two_level) {  // p is 16 waves of 8 tiles; the workspace (sized for the single kernel) holds one float per partition
+    if (two_level) {
+      if (sum_parts > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
       float *partials = static_cast<float *>(d_ws);
-      if (nt)
-        launch(partition_sums_kernel<8, true>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks, partition_sums_run());
-      else
-        launch(partition_sums_kernel<8, false>, (unsigned)grid, 1024u, stream, static_cast<const half8_t *>(d_in), partials, n_chunks, partition_sums_run());
-      launch(segment_of_partials_kernel, 1u, 1024u, stream, static_cast<const float *>(partials), static_cast<uint16_t *>(d_out), grid);
+      launch_partition_sums(nt, sum_parts ? sum_parts : 1, stream, static_cast<const half8_t *>(d_in), partials, n_chunks);
+      launch_sum_of_partials(stream, partials, static_cast<uint16_t *>(d_out), 1, sum_parts ? sum_parts : 1);
       return TCU_OK;
     }
     unsigned *ws = static_cast<unsigned *>(d_ws);

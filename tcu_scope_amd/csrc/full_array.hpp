@@ -211,7 +211,7 @@ TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long 
 // segments of parts_per_segment whole partitions each, scanned independently (segments far
 // larger than what one block can walk), and `totals`, if given, receives every segment's sum.
 template <int U, bool MFMA, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order, unsigned parts_per_segment, uint16_t *totals,
+__global__ __launch_bounds__(kMaxBlock, 8) void full_scan_kernel(const half8_t *in, uint4_t *out, size_t n_chunks, unsigned *ws, int static_order, unsigned parts_per_segment, uint16_t *totals,
                                                                WaitPolicy wait) {
   __shared__ float wave_total[kMaxWaves];
   __shared__ unsigned s_part;
@@ -220,8 +220,6 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   const int wave = wave_in_block();
   const int WPB = (int)(blockDim.x >> 6);
   unsigned long long *desc = reinterpret_cast<unsigned long long *>(ws + 64);
-  ScanOperands ops;
-  if constexpr (MFMA) ops = make_scan_operands<6>(lane);
   const int chunk_lane = MFMA ? matrix_chunk_of_lane(lane) : lane;
 
   if (!static_order) {
@@ -263,6 +261,8 @@ __global__ __launch_bounds__(kMaxBlock) void full_scan_kernel(const half8_t *in,
   __syncthreads();
   float carry = s_prefix;
   for (int w = 0; w < wave; w++) carry += wave_total[w];
+  ScanOperands ops;  // built here, behind the wait: the tiles held in registers leave no room for constants before it
+  if constexpr (MFMA) ops = make_scan_operands<6>(lane);
   static_for<U>([&](auto J) {
     constexpr int j = decltype(J)::value;
     float tile_total;
@@ -374,13 +374,16 @@ __global__ __launch_bounds__(kMaxBlock) void partition_sums_kernel(const half8_t
     partial_out[part] = s;
   }
 }
-// second level: block j (1024 threads) adds the parts_per_segment partials of segment j in a
-// fixed order (four independent strided streams per thread, then lanes, then waves) and writes
-// the fp16 result
-__global__ __launch_bounds__(1024) void segment_of_partials_kernel(const float *__restrict__ partial_in, uint16_t *__restrict__ out, size_t parts_per_segment) {
+// second level: block j (1024 threads) adds the parts_per_segment partials of segment j (fewer for a last block
+// that reaches total_parts) in a fixed order (four independent strided streams per thread, then lanes, then
+// waves) and writes the result: fp16 (OUT = uint16_t), or fp32 for a further level (OUT = float)
+template <typename OUT>
+__global__ __launch_bounds__(1024) void segment_of_partials_kernel(const float *__restrict__ partial_in, OUT *__restrict__ out, size_t parts_per_segment, size_t total_parts) {
   __shared__ float partial[16];
   const int lane = lane_id(), wave = wave_in_block();
-  const float *p = partial_in + (size_t)blockIdx.x * parts_per_segment;
+  const size_t first = (size_t)blockIdx.x * parts_per_segment;
+  if (first + parts_per_segment > total_parts) parts_per_segment = total_parts > first ? total_parts - first : 0;
+  const float *p = partial_in + first;
   float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
   size_t i = threadIdx.x;
   for (; i + 3 * 1024 < parts_per_segment; i += 4 * 1024) {
@@ -396,7 +399,10 @@ __global__ __launch_bounds__(1024) void segment_of_partials_kernel(const float *
   if (threadIdx.x == 0) {
     float s = 0.0f;
     for (int w = 0; w < 16; w++) s += partial[w];
-    out[blockIdx.x] = f16_bits(s);
+    if constexpr (sizeof(OUT) == 4)
+      out[blockIdx.x] = s;
+    else
+      out[blockIdx.x] = f16_bits(s);
   }
 }
 
