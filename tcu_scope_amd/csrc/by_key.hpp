@@ -432,4 +432,292 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
   }
 }
 
+
+// ---- the reduction without a chain: four launches, no waits, sums added in index order ------------------------
+//
+// What makes the one-pass kernel above slow as a reduction is that a run's sum cannot be written before the
+// number of runs in front of it is known, so every block holds its partition (keys parked in LDS, values in
+// registers) while that count travels down the chain.  Here the count comes first:
+//   1. key_heads_kernel    reads the keys once: a bit per element (1 = starts a run), the number of run starts per
+//                          partition of kKeyPartElems elements, and the keys of the first kKeyListCap run starts
+//                          of every partition, side by side in a list;
+//   2. key_count_prefix_kernel  exclusive prefix of the counts (one block);
+//   3. reduce_by_heads_kernel   reads the values and the bits: a run that starts after another run start of the same
+//                          partition has its sum written where it belongs (prefix + position in the partition), the
+//                          keys move from the list to keys_out; what precedes a partition's first run start
+//                          ("lead") and what follows its last ("tail", the whole partition without a run start) go
+//                          to two floats per partition;
+//   4. close_boundary_runs_kernel  a segmented scan of the tails over the partitions (one block) gives every run
+//                          that crosses a partition boundary its sum: tails back to the partition it started in +
+//                          the lead of the partition it ends in.
+// A partition is one wave's work in launches 1 and 3 (8 tiles), so both are grids of small blocks that depend on
+// nothing.  The bits of a partition are kept lane-major: lane l owns 8 bytes, byte j = its chunk of tile j.
+
+constexpr int kKeyPartTiles = 8;
+constexpr size_t kKeyPartElems = (size_t)kKeyPartTiles * kTileChunks * 8;  // 4096
+constexpr unsigned kKeyListCap = (unsigned)(kKeyPartElems / 8);           // run starts of a partition whose keys are parked
+
+// workspace of the four launches, in 8-byte units: bits | list | counts (parts + 1, u32) | lead | tail (fp32)
+struct KeyReduceLayout {
+  size_t parts, bits_at, list_at, counts_at, lead_at, tail_at, total;  // offsets and total in bytes
+};
+inline KeyReduceLayout key_reduce_layout(size_t n, size_t key_bytes) {
+  KeyReduceLayout l;
+  l.parts = (n + kKeyPartElems - 1) / kKeyPartElems;
+  auto up = [](size_t b) { return (b + 255) & ~(size_t)255; };
+  l.bits_at = 0;
+  l.list_at = up(l.parts * 64 * 8);
+  l.counts_at = l.list_at + up(l.parts * kKeyListCap * key_bytes);
+  l.lead_at = l.counts_at + up((l.parts + 1) * 4);
+  l.tail_at = l.lead_at + up(l.parts * 4);
+  l.total = l.tail_at + up(l.parts * 4);
+  return l;
+}
+
+template <typename KEY, int G, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void key_heads_kernel(const KEY *__restrict__ keys, size_t n, size_t parts, unsigned long long *__restrict__ bits, unsigned *__restrict__ counts,
+                                                              KEY *__restrict__ list, unsigned xcd_run) {
+  static_assert(kKeyPartTiles % G == 0, "tiles are loaded in groups of G");
+  const int lane = lane_id();
+  const size_t p = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave_in_block();
+  if (p >= parts) return;  // wave-uniform; the kernel has no barrier
+  const size_t base = p * kKeyPartElems;
+  unsigned long long mine = 0ull;
+  unsigned seen = 0;  // run starts of the partition in the tiles before
+  KEY last_of_tile = 0;
+#pragma unroll
+  for (int g = 0; g < kKeyPartTiles; g += G) {
+    KEY k[G][8];
+#pragma unroll
+    for (int j = 0; j < G; j++) {
+      const size_t e0 = base + ((size_t)(g + j) * kTileChunks + lane) * 8;
+      if (e0 + 8 <= n) {
+        constexpr int Q = (int)sizeof(KEY) / 2;  // 16-byte pieces per chunk of keys
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+          const uint4_t a = __builtin_bit_cast(uint4_t, load_chunk<NT>(reinterpret_cast<const half8_t *>(keys + e0) + q));
+          if constexpr (sizeof(KEY) == 4) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) k[j][4 * q + i] = (KEY)a[i];
+          } else {
+            k[j][2 * q] = (KEY)(((uint64_t)a[1] << 32) | a[0]);
+            k[j][2 * q + 1] = (KEY)(((uint64_t)a[3] << 32) | a[2]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) k[j][i] = e0 + i < n ? keys[e0 + i] : (KEY)0;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < G; j++) {
+      const size_t e0 = base + ((size_t)(g + j) * kTileChunks + lane) * 8;
+      const int valid = e0 >= n ? 0 : (n - e0 >= 8 ? 8 : (int)(n - e0));
+      KEY pk = key_of_previous_lane(k[j][7]);
+      if (lane == 0) {
+        if (g + j > 0)
+          pk = last_of_tile;
+        else if (e0 > 0 && e0 < n)
+          pk = keys[e0 - 1];
+      }
+      last_of_tile = key_of_lane(k[j][7], 63);
+      unsigned heads = 0;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const KEY before = i ? k[j][i - 1] : pk;
+        if (i < valid && (k[j][i] != before || e0 + i == 0)) heads |= 1u << i;
+      }
+      mine |= (unsigned long long)heads << (8 * (g + j));
+      const unsigned hc = (unsigned)__builtin_popcount(heads);
+      const unsigned he = wave_exclusive_count(hc);
+      if (list != nullptr && heads != 0u && seen + he < kKeyListCap) {
+        unsigned m = seen + he;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          if (((heads >> i) & 1u) && m < kKeyListCap) list[p * kKeyListCap + m] = k[j][i];
+          m += (heads >> i) & 1u;
+        }
+      }
+      seen += readlane_u32(he + hc, 63);
+    }
+  }
+  bits[p * 64 + lane] = mine;
+  if (lane == 0) counts[p] = seen;
+}
+
+// counts[0 .. parts) -> their exclusive prefix, counts[parts] = the total.  One block of 16 waves; a wave takes a
+// contiguous stretch, 64 entries at a time.
+__global__ __launch_bounds__(1024) void key_count_prefix_kernel(unsigned *counts, size_t parts) {
+  __shared__ unsigned wave_total[kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const size_t steps = (parts + 1023) / 1024, first = (size_t)wave * steps * 64;
+  unsigned total = 0;
+  for (size_t s = 0; s < steps; s++) {
+    const size_t i = first + s * 64 + lane;
+    total += i < parts ? counts[i] : 0u;
+  }
+  total += wave_exclusive_count(total);  // inclusive: the wave's total in lane 63
+  if (lane == 63) wave_total[wave] = total;
+  __syncthreads();
+  unsigned run = 0;
+  for (int w = 0; w < wave; w++) run += wave_total[w];
+  for (size_t s = 0; s < steps; s++) {
+    const size_t i = first + s * 64 + lane;
+    const unsigned c = i < parts ? counts[i] : 0u;
+    const unsigned e = wave_exclusive_count(c);
+    if (i < parts) counts[i] = run + e;
+    run += readlane_u32(e + c, 63);
+  }
+  if (wave == kMaxWaves - 1 && lane == 0) counts[parts] = run;
+}
+
+template <typename KEY, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void reduce_by_heads_kernel(const uint16_t *__restrict__ in, const unsigned long long *__restrict__ bits, const unsigned *__restrict__ prefix,
+                                                                    const KEY *__restrict__ keys, const KEY *__restrict__ list, uint16_t *__restrict__ out, KEY *__restrict__ keys_out,
+                                                                    float *__restrict__ lead, float *__restrict__ tail, size_t n, size_t parts, unsigned xcd_run) {
+  const int lane = lane_id();
+  const size_t p = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave_in_block();
+  if (p >= parts) return;  // wave-uniform; the kernel has no barrier
+  const size_t base = p * kKeyPartElems;
+  half8_t v[kKeyPartTiles];
+#pragma unroll
+  for (int j = 0; j < kKeyPartTiles; j++) {
+    const size_t e0 = base + ((size_t)j * kTileChunks + lane) * 8;
+    if (e0 + 8 <= n) {
+      v[j] = load_chunk<NT>(reinterpret_cast<const half8_t *>(in + e0));
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[j][i] = e0 + i < n ? __builtin_bit_cast(half_t, in[e0 + i]) : (half_t)0.0f;
+    }
+  }
+  const unsigned long long mine = bits[p * 64 + lane];
+  const unsigned first_run = prefix[p], runs = prefix[p + 1] - first_run;
+  // the keys of the runs that start here: from the list, as far as it goes
+  if (keys_out) {
+    const unsigned parked = runs < kKeyListCap ? runs : kKeyListCap;
+    for (unsigned m = (unsigned)lane; m < parked; m += 64u) keys_out[(size_t)first_run + m] = list[p * kKeyListCap + m];
+  }
+  unsigned wf = 0, seen = 0;  // the partition so far: a run start seen / how many
+  float wv = 0.0f;            //   ... and the sum since the last of them (or since the partition's start)
+#pragma unroll
+  for (int j = 0; j < kKeyPartTiles; j++) {
+    const unsigned heads = (unsigned)(mine >> (8 * j)) & 0xffu;
+    const size_t e0 = base + ((size_t)j * kTileChunks + lane) * 8;
+    const unsigned hc = (unsigned)__builtin_popcount(heads);
+    const unsigned hb = seen + wave_exclusive_count(hc);  // run starts of the partition before this chunk
+    // the chunk, element by element: the second and further run starts of the chunk close a run that began in it
+    float run = 0.0f, before_first = 0.0f;
+    unsigned m = hb;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if ((heads >> i) & 1u) {
+        if (m == hb) {
+          before_first = run;
+        } else {
+          out[(size_t)first_run + m - 1] = f16_bits(run);
+        }
+        if (keys_out && m >= kKeyListCap) keys_out[(size_t)first_run + m] = keys[e0 + i];
+        m++;
+        run = (float)v[j][i];
+      } else {
+        run += (float)v[j][i];
+      }
+    }
+    const unsigned F = heads ? 1u : 0u;
+    unsigned fe;
+    float ve;
+    wave_exclusive_seg_scan(F, run, fe, ve);
+    // what precedes this lane's chunk inside the partition
+    unsigned lf = fe;
+    float lv = ve;
+    seg_combine(wf, wv, lf, lv);
+    if (heads != 0u) {  // the chunk's first run start closes the run that came in
+      if (hb == 0u)
+        lead[p] = lv + before_first;  // it came in from outside the partition: closed by the last launch
+      else
+        out[(size_t)first_run + hb - 1] = f16_bits(lv + before_first);
+    }
+    unsigned fi = F;
+    float vi = run;
+    seg_combine(fe, ve, fi, vi);
+    unsigned tf = readlane_u32(fi, 63);
+    float tv = readlane(vi, 63);
+    seg_combine(wf, wv, tf, tv);
+    wf = tf;
+    wv = tv;
+    seen = readlane_u32(hb + hc, 63);
+  }
+  if (lane == 0) tail[p] = wv;
+}
+
+// One block.  Over the partitions, under the operator of the top of this file with flag = "a run starts in the
+// partition" and value = tail: the exclusive scan at partition p is what the run that comes into p has gathered
+// before p.  That run ends at p's first run start (its sum goes to out[prefix[p] - 1], with p's lead) or runs on;
+// the one that reaches the end of the array is the last run.
+__global__ __launch_bounds__(1024) void close_boundary_runs_kernel(const unsigned *__restrict__ prefix, const float *__restrict__ lead, const float *__restrict__ tail,
+                                                                   uint16_t *__restrict__ out, unsigned long long *num_runs, size_t parts) {
+  __shared__ unsigned wave_f[kMaxWaves];
+  __shared__ float wave_v[kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const size_t steps = (parts + 1023) / 1024, first = (size_t)wave * steps * 64;
+  unsigned wf = 0;
+  float wv = 0.0f;
+  for (size_t s = 0; s < steps; s++) {
+    const size_t i = first + s * 64 + lane;
+    const unsigned F = i < parts && prefix[i + 1] > prefix[i] ? 1u : 0u;
+    const float V = i < parts ? tail[i] : 0.0f;
+    unsigned fe;
+    float ve;
+    wave_exclusive_seg_scan(F, V, fe, ve);
+    unsigned fi = F;
+    float vi = V;
+    seg_combine(fe, ve, fi, vi);
+    unsigned tf = readlane_u32(fi, 63);
+    float tv = readlane(vi, 63);
+    seg_combine(wf, wv, tf, tv);
+    wf = tf;
+    wv = tv;
+  }
+  if (lane == 0) {
+    wave_f[wave] = wf;
+    wave_v[wave] = wv;
+  }
+  __syncthreads();
+  unsigned cf = 0;
+  float cv = 0.0f;
+  for (int w = 0; w < wave; w++) {
+    unsigned f = wave_f[w];
+    float v = wave_v[w];
+    seg_combine(cf, cv, f, v);
+    cf = f;
+    cv = v;
+  }
+  for (size_t s = 0; s < steps; s++) {
+    const size_t i = first + s * 64 + lane;
+    const unsigned before = i < parts ? prefix[i] : 0u;
+    const unsigned F = i < parts && prefix[i + 1] > before ? 1u : 0u;
+    const float V = i < parts ? tail[i] : 0.0f;
+    unsigned fe;
+    float ve;
+    wave_exclusive_seg_scan(F, V, fe, ve);
+    unsigned lf = fe;
+    float lv = ve;
+    seg_combine(cf, cv, lf, lv);
+    if (F && before > 0u) out[(size_t)before - 1] = f16_bits(lv + lead[i]);
+    unsigned fi = F;
+    float vi = V;
+    seg_combine(fe, ve, fi, vi);
+    unsigned tf = readlane_u32(fi, 63);
+    float tv = readlane(vi, 63);
+    seg_combine(cf, cv, tf, tv);
+    cf = tf;
+    cv = tv;
+  }
+  if (wave == kMaxWaves - 1 && lane == 0) {  // the last wave's stretch reaches the end of the partitions (or is empty)
+    const unsigned total = prefix[parts];
+    if (total > 0u) out[(size_t)total - 1] = f16_bits(cv);
+    if (num_runs) *num_runs = total;
+  }
+}
+
 }  // namespace tcu

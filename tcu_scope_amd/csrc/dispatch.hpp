@@ -51,6 +51,8 @@ struct Options {
   int xcd_run = -1;            // consecutive pieces of work per XCD (xcd_run_piece): -1 = the measured value for the size, 0 = none, C > 0 = C
   unsigned lookback_poll_limit = kDefaultPollLimit;  // polls of an unpublished value before a single-pass kernel gives up (results become NaN)
   unsigned test_mute_partition = 0;                  // tests only: partition test_mute_partition - 1 of a single-pass kernel publishes nothing
+  bool by_key_reduce_chain = false;  // reduction by key: the one-pass look-back kernel instead of the four launches that wait for nothing
+  int by_key_waves = 0;              // waves per block of the two big launches of the reduction by key (0 = default)
 };
 inline Options &options() {
   static Options o;
@@ -72,6 +74,8 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_strip_lds") o.gemv_strip_lds = value != 0;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
+  else if (n == "by_key_reduce_chain") o.by_key_reduce_chain = value != 0;
+  else if (n == "by_key_waves") o.by_key_waves = value < 0 ? 0 : (value > kMaxWaves ? kMaxWaves : value);
   else if (n == "gemm_staged_epilogue") o.gemm_staged_epilogue = value != 0;
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
   else if (n == "compute_units") o.compute_units = value < 1 ? 1 : value;
@@ -951,7 +955,9 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
   const size_t parts = (n + kByKeyPartition - 1) / kByKeyPartition;
   const unsigned shift = desc_shift_for(parts) ? desc_shift_for(parts) : 1;  // a slot holds the value and the count descriptor: at least 16 bytes
   const size_t words = look_back_words(parts, shift);
-  const size_t need = round_up(4 * words, kWorkspaceAlign);
+  // the reduction's workspace serves either of its forms (the option may change between the query and the call)
+  const KeyReduceLayout lay = key_reduce_layout(n, sizeof(KEY));
+  const size_t need = round_up(reduce && lay.total > 4 * words ? lay.total : 4 * words, kWorkspaceAlign);
   if (!d_ws) {
     *ws_bytes = need;
     return TCU_OK;
@@ -965,6 +971,32 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
   if (!aligned16(d_keys) || !aligned16(d_in) || (!reduce && !aligned16(d_out))) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": keys, values and the scan's output must be 16-byte aligned");
   if ((reinterpret_cast<uintptr_t>(d_out) & 1u) || (reinterpret_cast<uintptr_t>(d_keys_out) & (sizeof(KEY) - 1)) || (reinterpret_cast<uintptr_t>(d_num_runs) & 7u))
     return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": misaligned output pointer");
+  if (reduce && !options().by_key_reduce_chain) {
+    if (!aligned16(d_ws)) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": the workspace must be 16-byte aligned");
+    char *w = static_cast<char *>(d_ws);
+    unsigned long long *bits = reinterpret_cast<unsigned long long *>(w + lay.bits_at);
+    KEY *list = d_keys_out ? reinterpret_cast<KEY *>(w + lay.list_at) : nullptr;
+    unsigned *counts = reinterpret_cast<unsigned *>(w + lay.counts_at);
+    float *lead = reinterpret_cast<float *>(w + lay.lead_at), *tail = reinterpret_cast<float *>(w + lay.tail_at);
+    const unsigned waves = options().by_key_waves > 0 ? (unsigned)options().by_key_waves : 1u;
+    const size_t blocks = (lay.parts + waves - 1) / waves;
+    if (blocks > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    const unsigned run = options().xcd_run >= 0 ? (unsigned)options().xcd_run : 0u;
+    const KEY *keys = static_cast<const KEY *>(d_keys);
+    constexpr int G = sizeof(KEY) == 4 ? 8 : 4;
+    if (options().nontemporal) launch(key_heads_kernel<KEY, G, true>, (unsigned)blocks, waves * 64u, stream, keys, n, lay.parts, bits, counts, list, run);
+    else launch(key_heads_kernel<KEY, G, false>, (unsigned)blocks, waves * 64u, stream, keys, n, lay.parts, bits, counts, list, run);
+    launch(key_count_prefix_kernel, 1u, 1024u, stream, counts, lay.parts);
+    if (options().nontemporal)
+      launch(reduce_by_heads_kernel<KEY, true>, (unsigned)blocks, waves * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<const unsigned long long *>(bits), static_cast<const unsigned *>(counts), keys,
+             static_cast<const KEY *>(list), static_cast<uint16_t *>(d_out), static_cast<KEY *>(d_keys_out), lead, tail, n, lay.parts, run);
+    else
+      launch(reduce_by_heads_kernel<KEY, false>, (unsigned)blocks, waves * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<const unsigned long long *>(bits), static_cast<const unsigned *>(counts), keys,
+             static_cast<const KEY *>(list), static_cast<uint16_t *>(d_out), static_cast<KEY *>(d_keys_out), lead, tail, n, lay.parts, run);
+    launch(close_boundary_runs_kernel, 1u, 1024u, stream, static_cast<const unsigned *>(counts), static_cast<const float *>(lead), static_cast<const float *>(tail), static_cast<uint16_t *>(d_out),
+           static_cast<unsigned long long *>(d_num_runs), lay.parts);
+    return TCU_OK;
+  }
   unsigned *ws = static_cast<unsigned *>(d_ws);
   launch(zero_look_back_kernel, (unsigned)((parts + 255) / 256), 256u, stream, ws, parts, shift);
   const int so = options().static_order ? 1 : 0;

@@ -25,7 +25,7 @@
 #define __device__
 #define __forceinline__ inline
 #define __shared__ static
-#define __launch_bounds__(x)
+#define __launch_bounds__(...)
 #define TCU_DEVICE inline
 
 namespace emu {
