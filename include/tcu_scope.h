@@ -163,8 +163,9 @@ int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments,
 
 /* Segments given by a key array: a segment is a run of equal consecutive keys (d_keys: n signed integers of
  * key_bits = 32 or 64 bits in device memory; n < 2^32).  d_keys, d_in and the scan's d_out must be 16-byte
- * aligned.  Workspace: the two-phase protocol of the full-array entry points below (256 bytes per 32768
- * elements + 256).  One pass over keys and values (decoupled look-back on (head flag, value) pairs).
+ * aligned.  Workspace: the two-phase protocol of the full-array entry points below (16-byte aligned; the scan:
+ * 256 bytes per 32768 elements + 256; the reduction: n/8 bytes of run-start bits + one key per 8 elements + 12
+ * bytes per 4096 elements, about 0.63 n bytes with 32-bit keys and 1.13 n with 64-bit keys).
  *
  * tcu_seg_scan_by_key_f16: d_out[i] = fp16( sum of d_in[j .. i] ), j = the first element of i's run.  In place
  * (d_out == d_in) is allowed.  Hand-written counterpart of thrust::inclusive_scan_by_key(keys, keys + n, in, out)
@@ -174,8 +175,10 @@ int tcu_seg_scan_offsets_f16(const void *d_in, void *d_out, size_t num_segments,
  * d_keys_out[r] = its key; *d_num_runs (a 64-bit unsigned in device memory, may be NULL) receives the number of
  * runs, which is what thrust::reduce_by_key(keys, keys + n, in, keys_out, out) returns as the end of its output
  * (src/reduction/seg_thrust.cu:50-51).  d_out and d_keys_out need room for as many entries as there are runs
- * (at most n) and must not overlap d_in or d_keys.  A look-back wait that expires (see "lookback_poll_limit")
- * leaves ~0 in *d_num_runs and NaN in the sums that depended on it. */
+ * (at most n) and must not overlap d_in or d_keys.  The scan is one pass over keys and values with a decoupled
+ * look-back on (head flag, value) pairs.  The reduction is five launches none of which waits for another block: the
+ * keys are read once (run-start bits and counts), the values once; sums are added in index order, so the same
+ * input gives the same bits every time. */
 int tcu_seg_scan_by_key_f16(const void *d_keys, const void *d_in, void *d_out, size_t n, int key_bits, void *d_workspace, size_t *workspace_bytes, void *stream);
 int tcu_seg_reduce_by_key_f16(const void *d_keys, const void *d_in, void *d_keys_out, void *d_out, void *d_num_runs, size_t n, int key_bits, void *d_workspace, size_t *workspace_bytes, void *stream);
 

@@ -24,6 +24,11 @@ extern "C" {
  *                     reach HBM; a scan whose output must reach HBM (outputs taken in turn, or 2 GiB of output) runs
  *                     1-3 % slower with it
  *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
+ *   "by_key_reduce_chain" 0/1, default 0: tcu_seg_reduce_by_key_f16 as one pass with a decoupled look-back (the form of the
+ *                     scan by key; a wait that expires leaves ~0 in *d_num_runs and NaN in the sums that depended on it)
+ *                     instead of the five launches that wait for nothing
+ *   "by_key_waves"    waves per block of the two large launches of tcu_seg_reduce_by_key_f16 (1 .. 16; 0 = default 1)
+ *   "by_key_key_tiles" KiB of keys a wave of its first launch has in flight: 4, 8 or 16 (0 = default 16)
  *   "scan_lds_tiles"  0/1, default 1: full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves)
  *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step
  *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more);

@@ -3,20 +3,22 @@
 // src/prefixsum/seg_thrust.cu:46-47) and one sum per run (thrust::reduce_by_key,
 // src/reduction/seg_thrust.cu:50-51), fp16 values, fp32 accumulation, one rounding to fp16.
 //
-// One pass over keys and values.  The scan operator on pairs (head flag, value)
+// by_key_kernel: one pass over keys and values.  The scan operator on pairs (head flag, value)
 //     (f1, v1) (+) (f2, v2) = (f1 | f2, f2 ? v2 : v1 + v2)
 // is associative, so the whole array is scanned like the full-array prefix sum: a lane scans
 // its 8 elements serially, the 64 chunk summaries of a tile are scanned across the lanes with
 // DPP, tiles are chained in the wave, waves meet in LDS, blocks (partitions of
 // blockDim/64 * U tiles, handed out by a ticket) meet through decoupled look-back on 64-bit
 // descriptors {status + 4 * flag, fp32 value}: a predecessor whose aggregate carries a head
-// flag ends the look-back just as a published prefix does.  The reduction also counts the heads
+// flag ends the look-back just as a published prefix does.  As a reduction it also counts the heads
 // (a second, integer look-back) to know where a run's sum goes, and writes a run's sum at the
 // head of the NEXT run (the value carried up to that head), so no element ever needs its
 // successor's key; the last run is written by the lane that holds the last element.
-//
 // Every wait is bounded (WaitPolicy): a look-back that gives up yields NaN sums (and, for the
 // reduction, counts of 0xffffffff that keep later partitions from writing anything).
+//
+// The reduction's default form is the sequence of launches in the second half of this file, which waits
+// for nothing; by_key_kernel<..., REDUCE = true> stays selectable.
 #pragma once
 
 #include "full_array.hpp"
@@ -433,7 +435,7 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
 }
 
 
-// ---- the reduction without a chain: four launches, no waits, sums added in index order ------------------------
+// ---- the reduction without a chain: five launches, no waits, sums added in index order ------------------------
 //
 // What makes the one-pass kernel above slow as a reduction is that a run's sum cannot be written before the
 // number of runs in front of it is known, so every block holds its partition (keys parked in LDS, values in
@@ -441,25 +443,28 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
 //   1. key_heads_kernel    reads the keys once: a bit per element (1 = starts a run), the number of run starts per
 //                          partition of kKeyPartElems elements, and the keys of the first kKeyListCap run starts
 //                          of every partition, side by side in a list;
-//   2. key_count_prefix_kernel  exclusive prefix of the counts (one block);
+//   2. key_group_prefix_kernel  the run starts in front of every group of 64 partitions (one block);
 //   3. reduce_by_heads_kernel   reads the values and the bits: a run that starts after another run start of the same
-//                          partition has its sum written where it belongs (prefix + position in the partition), the
-//                          keys move from the list to keys_out; what precedes a partition's first run start
-//                          ("lead") and what follows its last ("tail", the whole partition without a run start) go
-//                          to two floats per partition;
-//   4. close_boundary_runs_kernel  a segmented scan of the tails over the partitions (one block) gives every run
-//                          that crosses a partition boundary its sum: tails back to the partition it started in +
-//                          the lead of the partition it ends in.
-// A partition is one wave's work in launches 1 and 3 (8 tiles), so both are grids of small blocks that depend on
-// nothing.  The bits of a partition are kept lane-major: lane l owns 8 bytes, byte j = its chunk of tile j.
+//                          partition has its sum written where it belongs (runs in front of the group + in front of
+//                          the partition + in the partition), the keys move from the list to keys_out; what precedes
+//                          a partition's first run start ("lead") and what follows its last ("tail", the whole
+//                          partition without a run start) go to two floats per partition;
+//   4. key_group_tails_kernel, 5. close_boundary_runs_kernel  a segmented scan of the tails over the partitions
+//                          gives every run that crosses a partition boundary its sum: tails back to the partition it
+//                          started in + the lead of the partition it ends in.
+// A partition is one wave's work in launches 1 and 3 (8 tiles of values), so both are grids of small blocks that
+// depend on nothing; launches 2, 4 and 5 touch a few bytes per partition.  The bits of a partition are kept
+// lane-major for launch 3: lane l owns 8 bytes, byte j = its chunk of tile j.
+// Measured (2^28 elements, 32-bit keys): launch 1 165-187 us (0.86 of the HBM peak as long as it writes nothing;
+// the bits, 3 % of its bytes, cost 10 %), launch 3 82-120 us, the three small ones 21 us together.
 
 constexpr int kKeyPartTiles = 8;
 constexpr size_t kKeyPartElems = (size_t)kKeyPartTiles * kTileChunks * 8;  // 4096
 constexpr unsigned kKeyListCap = (unsigned)(kKeyPartElems / 8);           // run starts of a partition whose keys are parked
 
-// workspace of the four launches, in 8-byte units: bits | list | counts (parts + 1, u32) | lead | tail (fp32)
+// workspace: bits | list | counts (u32) | lead | tail (fp32) per partition; prefix (groups + 1), flag, tail per group of 64 partitions
 struct KeyReduceLayout {
-  size_t parts, bits_at, list_at, counts_at, lead_at, tail_at, total;  // offsets and total in bytes
+  size_t parts, groups, bits_at, list_at, counts_at, lead_at, tail_at, gprefix_at, gflag_at, gtail_at, total;  // offsets and total in bytes
 };
 inline KeyReduceLayout key_reduce_layout(size_t n, size_t key_bytes) {
   KeyReduceLayout l;
@@ -468,72 +473,91 @@ inline KeyReduceLayout key_reduce_layout(size_t n, size_t key_bytes) {
   l.bits_at = 0;
   l.list_at = up(l.parts * 64 * 8);
   l.counts_at = l.list_at + up(l.parts * kKeyListCap * key_bytes);
-  l.lead_at = l.counts_at + up((l.parts + 1) * 4);
+  l.groups = (l.parts + 63) / 64;
+  l.lead_at = l.counts_at + up(l.parts * 4);
   l.tail_at = l.lead_at + up(l.parts * 4);
-  l.total = l.tail_at + up(l.parts * 4);
+  l.gprefix_at = l.tail_at + up(l.parts * 4);
+  l.gflag_at = l.gprefix_at + up((l.groups + 1) * 4);
+  l.gtail_at = l.gflag_at + up(l.groups * 4);
+  l.total = l.gtail_at + up(l.groups * 4);
   return l;
 }
 
-template <typename KEY, int G, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void key_heads_kernel(const KEY *__restrict__ keys, size_t n, size_t parts, unsigned long long *__restrict__ bits, unsigned *__restrict__ counts,
-                                                              KEY *__restrict__ list, unsigned xcd_run) {
-  static_assert(kKeyPartTiles % G == 0, "tiles are loaded in groups of G");
-  const int lane = lane_id();
-  const size_t p = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave_in_block();
-  if (p >= parts) return;  // wave-uniform; the kernel has no barrier
+// One partition's keys -> its bits, its number of run starts and its list.  WHOLE: the partition lies inside the array.
+// The keys are read 16 bytes per lane with the lanes side by side (whole cache lines per instruction): a "key tile" is
+// 1 KiB of keys, a lane holds KPL = 4 (32-bit) or 2 (64-bit) consecutive ones.  The bits are wanted by the byte, one
+// byte per 8 consecutive elements: LPB = 8 / KPL neighbouring lanes put theirs together (quad permutes), and the first
+// lane of each such set gathers the bytes of the value tile's lane it stands for (see reduce_partition_by_heads).
+template <typename KEY, int G_ASKED, bool NT, bool WHOLE>
+TCU_DEVICE void key_heads_of_partition(const KEY *__restrict__ keys, size_t n, size_t p, int lane, unsigned long long *__restrict__ bits, unsigned *__restrict__ counts, KEY *__restrict__ list) {
+  constexpr int KPL = 16 / (int)sizeof(KEY);
+  constexpr int KT_ELEMS = 64 * KPL;                        // elements per key tile
+  constexpr int KTS = (int)(kKeyPartElems / KT_ELEMS);      // key tiles per partition: 16 or 32
+  constexpr int KTPT = kTileChunks * 8 / KT_ELEMS;          // key tiles per tile of values: 2 or 4
+  constexpr int LPB = 8 / KPL;
+  constexpr int G = G_ASKED < KTS ? G_ASKED : KTS;  // key tiles in flight
+  static_assert(KTS % G == 0, "key tiles are loaded in groups of G");
   const size_t base = p * kKeyPartElems;
-  unsigned long long mine = 0ull;
-  unsigned seen = 0;  // run starts of the partition in the tiles before
+  unsigned long long word[KTPT];
+#pragma unroll
+  for (int r = 0; r < KTPT; r++) word[r] = 0ull;
+  unsigned seen = 0;  // run starts of the partition in the key tiles before
   KEY last_of_tile = 0;
 #pragma unroll
-  for (int g = 0; g < kKeyPartTiles; g += G) {
-    KEY k[G][8];
+  for (int g = 0; g < KTS; g += G) {
+    KEY k[G][KPL];
 #pragma unroll
     for (int j = 0; j < G; j++) {
-      const size_t e0 = base + ((size_t)(g + j) * kTileChunks + lane) * 8;
-      if (e0 + 8 <= n) {
-        constexpr int Q = (int)sizeof(KEY) / 2;  // 16-byte pieces per chunk of keys
+      const size_t e0 = base + ((size_t)(g + j) * 64 + lane) * KPL;
+      if (WHOLE || e0 + KPL <= n) {
+        const uint4_t a = __builtin_bit_cast(uint4_t, load_chunk<NT>(reinterpret_cast<const half8_t *>(keys + e0)));
+        if constexpr (sizeof(KEY) == 4) {
 #pragma unroll
-        for (int q = 0; q < Q; q++) {
-          const uint4_t a = __builtin_bit_cast(uint4_t, load_chunk<NT>(reinterpret_cast<const half8_t *>(keys + e0) + q));
-          if constexpr (sizeof(KEY) == 4) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) k[j][4 * q + i] = (KEY)a[i];
-          } else {
-            k[j][2 * q] = (KEY)(((uint64_t)a[1] << 32) | a[0]);
-            k[j][2 * q + 1] = (KEY)(((uint64_t)a[3] << 32) | a[2]);
-          }
+          for (int i = 0; i < 4; i++) k[j][i] = (KEY)a[i];
+        } else {
+          k[j][0] = (KEY)(((uint64_t)a[1] << 32) | a[0]);
+          k[j][1] = (KEY)(((uint64_t)a[3] << 32) | a[2]);
         }
       } else {
 #pragma unroll
-        for (int i = 0; i < 8; i++) k[j][i] = e0 + i < n ? keys[e0 + i] : (KEY)0;
+        for (int i = 0; i < KPL; i++) k[j][i] = e0 + i < n ? keys[e0 + i] : (KEY)0;
       }
     }
 #pragma unroll
     for (int j = 0; j < G; j++) {
-      const size_t e0 = base + ((size_t)(g + j) * kTileChunks + lane) * 8;
-      const int valid = e0 >= n ? 0 : (n - e0 >= 8 ? 8 : (int)(n - e0));
-      KEY pk = key_of_previous_lane(k[j][7]);
+      const int kt = g + j;
+      const size_t e0 = base + ((size_t)kt * 64 + lane) * KPL;
+      KEY pk = key_of_previous_lane(k[j][KPL - 1]);
       if (lane == 0) {
-        if (g + j > 0)
+        if (kt > 0)
           pk = last_of_tile;
-        else if (e0 > 0 && e0 < n)
-          pk = keys[e0 - 1];
+        else
+          pk = e0 > 0 ? keys[e0 - 1] : (KEY)~k[j][0];  // the first element of the array starts a run
       }
-      last_of_tile = key_of_lane(k[j][7], 63);
-      unsigned heads = 0;
+      last_of_tile = key_of_lane(k[j][KPL - 1], 63);
+      unsigned heads = 0;  // bit i = element i differs from the one before
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const KEY before = i ? k[j][i - 1] : pk;
-        if (i < valid && (k[j][i] != before || e0 + i == 0)) heads |= 1u << i;
+      for (int i = KPL - 1; i >= 0; i--) heads = heads + heads + (k[j][i] != (i ? k[j][i - 1] : pk) ? 1u : 0u);
+      if constexpr (!WHOLE) {
+        const int valid = e0 >= n ? 0 : (n - e0 >= (size_t)KPL ? KPL : (int)(n - e0));
+        heads &= (1u << valid) - 1u;
       }
-      mine |= (unsigned long long)heads << (8 * (g + j));
+      if (ballot(heads != 0u) == 0ull) continue;  // wave-uniform: most key tiles of long runs
+      unsigned byte = heads;
+      if constexpr (LPB == 2) {
+        byte |= dpp_u32<0xF5>(0u, heads) << 4;  // quad_perm:[1,1,3,3]: the odd neighbour's bits
+      } else {
+        byte |= dpp_u32<0x55>(0u, heads) << 2;  // quad_perm:[1,1,1,1]
+        byte |= dpp_u32<0xAA>(0u, heads) << 4;  // quad_perm:[2,2,2,2]
+        byte |= dpp_u32<0xFF>(0u, heads) << 6;  // quad_perm:[3,3,3,3]
+      }
+      word[kt % KTPT] |= (unsigned long long)byte << (8 * (kt / KTPT));
       const unsigned hc = (unsigned)__builtin_popcount(heads);
       const unsigned he = wave_exclusive_count(hc);
       if (list != nullptr && heads != 0u && seen + he < kKeyListCap) {
         unsigned m = seen + he;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
+        for (int i = 0; i < KPL; i++) {
           if (((heads >> i) & 1u) && m < kKeyListCap) list[p * kKeyListCap + m] = k[j][i];
           m += (heads >> i) & 1u;
         }
@@ -541,59 +565,145 @@ __global__ __launch_bounds__(kMaxBlock) void key_heads_kernel(const KEY *__restr
       seen += readlane_u32(he + hc, 63);
     }
   }
-  bits[p * 64 + lane] = mine;
+  // A partition without a run start writes no bits (nobody reads them: see reduce_partition_by_heads).  The bits are
+  // 3 % of the bytes of this launch and cost 12 % of its time (writes among the reads; 10 % when non-temporal).
+  if (seen != 0u && lane % LPB == 0) {
+#pragma unroll
+    for (int r = 0; r < KTPT; r++) {
+      unsigned long long *at = bits + p * 64 + r * (64 / LPB) + lane / LPB;
+      if constexpr (NT) __builtin_nontemporal_store(word[r], at);
+      else *at = word[r];
+    }
+  }
   if (lane == 0) counts[p] = seen;
 }
 
-// counts[0 .. parts) -> their exclusive prefix, counts[parts] = the total.  One block of 16 waves; a wave takes a
-// contiguous stretch, 64 entries at a time.
-__global__ __launch_bounds__(1024) void key_count_prefix_kernel(unsigned *counts, size_t parts) {
-  __shared__ unsigned wave_total[kMaxWaves];
-  const int lane = lane_id(), wave = wave_in_block();
-  const size_t steps = (parts + 1023) / 1024, first = (size_t)wave * steps * 64;
-  unsigned total = 0;
-  for (size_t s = 0; s < steps; s++) {
-    const size_t i = first + s * 64 + lane;
-    total += i < parts ? counts[i] : 0u;
-  }
-  total += wave_exclusive_count(total);  // inclusive: the wave's total in lane 63
-  if (lane == 63) wave_total[wave] = total;
-  __syncthreads();
-  unsigned run = 0;
-  for (int w = 0; w < wave; w++) run += wave_total[w];
-  for (size_t s = 0; s < steps; s++) {
-    const size_t i = first + s * 64 + lane;
-    const unsigned c = i < parts ? counts[i] : 0u;
-    const unsigned e = wave_exclusive_count(c);
-    if (i < parts) counts[i] = run + e;
-    run += readlane_u32(e + c, 63);
-  }
-  if (wave == kMaxWaves - 1 && lane == 0) counts[parts] = run;
-}
-
-template <typename KEY, bool NT>
-__global__ __launch_bounds__(kMaxBlock) void reduce_by_heads_kernel(const uint16_t *__restrict__ in, const unsigned long long *__restrict__ bits, const unsigned *__restrict__ prefix,
-                                                                    const KEY *__restrict__ keys, const KEY *__restrict__ list, uint16_t *__restrict__ out, KEY *__restrict__ keys_out,
-                                                                    float *__restrict__ lead, float *__restrict__ tail, size_t n, size_t parts, unsigned xcd_run) {
-  const int lane = lane_id();
+template <typename KEY, int G, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void key_heads_kernel(const KEY *__restrict__ keys, size_t n, size_t parts, unsigned long long *__restrict__ bits, unsigned *__restrict__ counts,
+                                                              KEY *__restrict__ list, unsigned xcd_run) {
   const size_t p = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave_in_block();
   if (p >= parts) return;  // wave-uniform; the kernel has no barrier
+  if ((p + 1) * kKeyPartElems <= n)
+    key_heads_of_partition<KEY, G, NT, true>(keys, n, p, lane_id(), bits, counts, list);
+  else
+    key_heads_of_partition<KEY, G, NT, false>(keys, n, p, lane_id(), bits, counts, list);
+}
+
+// Scan over the 1024 threads of a block of what each of them has gathered: exclusive prefix of a count ...
+TCU_DEVICE unsigned block_exclusive_count(unsigned mine, unsigned *wave_total, int lane, int wave) {
+  const unsigned e = wave_exclusive_count(mine);
+  if (lane == 63) wave_total[wave] = e + mine;
+  __syncthreads();
+  unsigned before = 0;
+  for (int w = 0; w < wave; w++) before += wave_total[w];
+  return before + e;
+}
+// ... and of a (flag, value) pair under the operator at the top of this file
+TCU_DEVICE void block_exclusive_seg_scan(unsigned F, float V, unsigned *wave_f, float *wave_v, int lane, int wave, unsigned &Fe, float &Ve) {
+  unsigned fe, fi = F;
+  float ve, vi = V;
+  wave_exclusive_seg_scan(F, V, fe, ve);
+  seg_combine(fe, ve, fi, vi);
+  if (lane == 63) {
+    wave_f[wave] = fi;
+    wave_v[wave] = vi;
+  }
+  __syncthreads();
+  unsigned cf = 0;
+  float cv = 0.0f;
+  for (int w = 0; w < wave; w++) {
+    unsigned f = wave_f[w];
+    float v = wave_v[w];
+    seg_combine(cf, cv, f, v);
+    cf = f;
+    cv = v;
+  }
+  seg_combine(cf, cv, fe, ve);
+  Fe = fe;
+  Ve = ve;
+}
+
+// The partitions are taken in groups of 64: a wave reads a group's counts in one load.
+// group_prefix[g] = the run starts in front of group g, g = 0 .. groups.
+// One block of 16 waves; a wave takes a contiguous stretch of the groups, adds up each of them and keeps the sum of
+// the stretch's i-th group in lane i % 64 of register i / 64 (at most kMaxGroupRows registers: 2^20 partitions).
+constexpr int kMaxGroupRows = 16;
+__global__ __launch_bounds__(1024) void key_group_prefix_kernel(const unsigned *__restrict__ counts, unsigned *__restrict__ group_prefix, size_t parts, size_t groups) {
+  __shared__ unsigned wave_total[kMaxWaves];
+  const int lane = lane_id(), wave = wave_in_block();
+  const size_t per_wave = (groups + kMaxWaves - 1) / kMaxWaves, first = (size_t)wave * per_wave;
+  const size_t mine = first >= groups ? 0 : (groups - first < per_wave ? groups - first : per_wave);  // groups of this wave
+  unsigned row[kMaxGroupRows];
+#pragma unroll
+  for (int r = 0; r < kMaxGroupRows; r++) {
+    row[r] = 0u;
+    if ((size_t)r * 64 < mine) {
+      for (int gl0 = 0; gl0 < 64; gl0 += 16) {  // 16 loads in flight, then their sums
+        unsigned c[16];
+#pragma unroll
+        for (int b = 0; b < 16; b++) {
+          const size_t i = (first + (size_t)r * 64 + gl0 + b) * 64 + lane;
+          c[b] = (size_t)r * 64 + gl0 + b < mine && i < parts ? counts[i] : 0u;
+        }
+#pragma unroll
+        for (int b = 0; b < 16; b++) {
+          const unsigned sum = readlane_u32(c[b] + wave_exclusive_count(c[b]), 63);
+          if (lane == gl0 + b) row[r] = sum;
+        }
+      }
+    }
+  }
+  unsigned stretch = 0;
+#pragma unroll
+  for (int r = 0; r < kMaxGroupRows; r++) stretch += row[r];
+  unsigned before = block_exclusive_count(stretch, wave_total, lane, wave);  // lanes of a wave: their sums of all rows, in lane order - not the order of the groups
+  // so only the waves' totals are taken from it: what lies in front of this wave's stretch
+  before = readlane_u32(before, 0);
+#pragma unroll
+  for (int r = 0; r < kMaxGroupRows; r++) {
+    if ((size_t)r * 64 < mine) {
+      const unsigned e = wave_exclusive_count(row[r]);
+      const size_t gl = (size_t)r * 64 + lane;
+      if (gl < mine) group_prefix[first + gl] = before + e;
+      before += readlane_u32(e + row[r], 63);
+    }
+  }
+  if (first + mine == groups && mine > 0 && lane == 0) group_prefix[groups] = before;  // the wave whose stretch ends the groups
+  if (groups == 0 && threadIdx.x == 0) group_prefix[0] = 0u;
+}
+// run starts in front of partition p: those in front of its group + those of the group's partitions before it
+TCU_DEVICE unsigned runs_before_partition(const unsigned *__restrict__ counts, const unsigned *__restrict__ group_prefix, size_t p, int lane, unsigned *own) {
+  const size_t first = p & ~(size_t)63;
+  const unsigned c = first + lane <= p ? counts[first + lane] : 0u;  // the partitions of p's group up to p: all exist
+  const unsigned e = wave_exclusive_count(c);
+  const int at = (int)(p - first);
+  *own = readlane_u32(c, at);
+  return group_prefix[p >> 6] + readlane_u32(e, at);
+}
+
+// One partition's values and bits -> the sums of the runs that start and end in it, the keys of the runs that
+// start in it, its lead and its tail.
+template <typename KEY, bool NT, bool WHOLE>
+TCU_DEVICE void reduce_partition_by_heads(const uint16_t *__restrict__ in, const unsigned long long *__restrict__ bits, const unsigned *__restrict__ counts, const unsigned *__restrict__ group_prefix, const KEY *__restrict__ keys,
+                                          const KEY *__restrict__ list, uint16_t *__restrict__ out, KEY *__restrict__ keys_out, float *__restrict__ lead, float *__restrict__ tail, size_t n, size_t p,
+                                          int lane) {
   const size_t base = p * kKeyPartElems;
   half8_t v[kKeyPartTiles];
 #pragma unroll
   for (int j = 0; j < kKeyPartTiles; j++) {
     const size_t e0 = base + ((size_t)j * kTileChunks + lane) * 8;
-    if (e0 + 8 <= n) {
+    if (WHOLE || e0 + 8 <= n) {
       v[j] = load_chunk<NT>(reinterpret_cast<const half8_t *>(in + e0));
     } else {
 #pragma unroll
       for (int i = 0; i < 8; i++) v[j][i] = e0 + i < n ? __builtin_bit_cast(half_t, in[e0 + i]) : (half_t)0.0f;
     }
   }
-  const unsigned long long mine = bits[p * 64 + lane];
-  const unsigned first_run = prefix[p], runs = prefix[p + 1] - first_run;
-  // the keys of the runs that start here: from the list, as far as it goes
-  if (keys_out) {
+  unsigned runs;
+  const unsigned first_run = runs_before_partition(counts, group_prefix, p, lane, &runs);
+  const unsigned long long mine = runs ? bits[p * 64 + lane] : 0ull;  // wave-uniform
+  const bool keys_beyond_list = keys_out != nullptr && runs > kKeyListCap;  // wave-uniform
+  if (keys_out) {  // the keys of the runs that start here: from the list, as far as it goes
     const unsigned parked = runs < kKeyListCap ? runs : kKeyListCap;
     for (unsigned m = (unsigned)lane; m < parked; m += 64u) keys_out[(size_t)first_run + m] = list[p * kKeyListCap + m];
   }
@@ -602,24 +712,35 @@ __global__ __launch_bounds__(kMaxBlock) void reduce_by_heads_kernel(const uint16
 #pragma unroll
   for (int j = 0; j < kKeyPartTiles; j++) {
     const unsigned heads = (unsigned)(mine >> (8 * j)) & 0xffu;
+    if (ballot(heads != 0u) == 0ull) {  // wave-uniform: no run starts in this tile
+      wv += readlane(lane_group_sum<6>(sum8(v[j], 0.0f)), 63);
+      continue;
+    }
     const size_t e0 = base + ((size_t)j * kTileChunks + lane) * 8;
     const unsigned hc = (unsigned)__builtin_popcount(heads);
     const unsigned hb = seen + wave_exclusive_count(hc);  // run starts of the partition before this chunk
-    // the chunk, element by element: the second and further run starts of the chunk close a run that began in it
     float run = 0.0f, before_first = 0.0f;
-    unsigned m = hb;
+    if (ballot(hc > 1u) == 0ull) {  // wave-uniform: at most one run start per chunk, nothing to write from inside a chunk
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      if ((heads >> i) & 1u) {
-        if (m == hb) {
-          before_first = run;
-        } else {
-          out[(size_t)first_run + m - 1] = f16_bits(run);
+      for (int i = 0; i < 8; i++) {
+        const bool h = (heads >> i) & 1u;
+        before_first = h ? run : before_first;
+        run = (h ? 0.0f : run) + (float)v[j][i];
+      }
+      if (keys_beyond_list && heads != 0u && hb >= kKeyListCap) keys_out[(size_t)first_run + hb] = keys[e0 + __builtin_ctz(heads)];
+    } else {  // the second and further run starts of a chunk close a run that began in it
+      unsigned m = hb;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        if ((heads >> i) & 1u) {
+          if (m == hb)
+            before_first = run;
+          else
+            out[(size_t)first_run + m - 1] = f16_bits(run);
+          if (keys_beyond_list && m >= kKeyListCap) keys_out[(size_t)first_run + m] = keys[e0 + i];
+          m++;
+          run = 0.0f;
         }
-        if (keys_out && m >= kKeyListCap) keys_out[(size_t)first_run + m] = keys[e0 + i];
-        m++;
-        run = (float)v[j][i];
-      } else {
         run += (float)v[j][i];
       }
     }
@@ -627,8 +748,7 @@ __global__ __launch_bounds__(kMaxBlock) void reduce_by_heads_kernel(const uint16
     unsigned fe;
     float ve;
     wave_exclusive_seg_scan(F, run, fe, ve);
-    // what precedes this lane's chunk inside the partition
-    unsigned lf = fe;
+    unsigned lf = fe;  // what precedes this lane's chunk inside the partition
     float lv = ve;
     seg_combine(wf, wv, lf, lv);
     if (heads != 0u) {  // the chunk's first run start closes the run that came in
@@ -650,73 +770,71 @@ __global__ __launch_bounds__(kMaxBlock) void reduce_by_heads_kernel(const uint16
   if (lane == 0) tail[p] = wv;
 }
 
-// One block.  Over the partitions, under the operator of the top of this file with flag = "a run starts in the
-// partition" and value = tail: the exclusive scan at partition p is what the run that comes into p has gathered
-// before p.  That run ends at p's first run start (its sum goes to out[prefix[p] - 1], with p's lead) or runs on;
-// the one that reaches the end of the array is the last run.
-__global__ __launch_bounds__(1024) void close_boundary_runs_kernel(const unsigned *__restrict__ prefix, const float *__restrict__ lead, const float *__restrict__ tail,
-                                                                   uint16_t *__restrict__ out, unsigned long long *num_runs, size_t parts) {
-  __shared__ unsigned wave_f[kMaxWaves];
-  __shared__ float wave_v[kMaxWaves];
-  const int lane = lane_id(), wave = wave_in_block();
-  const size_t steps = (parts + 1023) / 1024, first = (size_t)wave * steps * 64;
-  unsigned wf = 0;
-  float wv = 0.0f;
-  for (size_t s = 0; s < steps; s++) {
-    const size_t i = first + s * 64 + lane;
-    const unsigned F = i < parts && prefix[i + 1] > prefix[i] ? 1u : 0u;
-    const float V = i < parts ? tail[i] : 0.0f;
-    unsigned fe;
-    float ve;
-    wave_exclusive_seg_scan(F, V, fe, ve);
-    unsigned fi = F;
-    float vi = V;
-    seg_combine(fe, ve, fi, vi);
-    unsigned tf = readlane_u32(fi, 63);
-    float tv = readlane(vi, 63);
-    seg_combine(wf, wv, tf, tv);
-    wf = tf;
-    wv = tv;
+template <typename KEY, bool NT>
+__global__ __launch_bounds__(kMaxBlock) void reduce_by_heads_kernel(const uint16_t *__restrict__ in, const unsigned long long *__restrict__ bits, const unsigned *__restrict__ counts, const unsigned *__restrict__ group_prefix,
+                                                                    const KEY *__restrict__ keys, const KEY *__restrict__ list, uint16_t *__restrict__ out, KEY *__restrict__ keys_out,
+                                                                    float *__restrict__ lead, float *__restrict__ tail, size_t n, size_t parts, unsigned xcd_run) {
+  const size_t p = xcd_run_piece(blockIdx.x, gridDim.x, xcd_run) * (blockDim.x >> 6) + wave_in_block();
+  if (p >= parts) return;  // wave-uniform; the kernel has no barrier
+  if ((p + 1) * kKeyPartElems <= n)
+    reduce_partition_by_heads<KEY, NT, true>(in, bits, counts, group_prefix, keys, list, out, keys_out, lead, tail, n, p, lane_id());
+  else
+    reduce_partition_by_heads<KEY, NT, false>(in, bits, counts, group_prefix, keys, list, out, keys_out, lead, tail, n, p, lane_id());
+}
+
+// The runs that cross a partition boundary.  Under the operator of the top of this file with flag = "a run starts in
+// the partition" and value = tail, the exclusive scan at partition p is what the run that comes into p has gathered
+// before p.  That run ends at p's first run start (its sum goes in front of p's first own run, with p's lead) or
+// runs on; the one that reaches the end of the array is the last run.  Two small launches with one wave per group of
+// 64 partitions: the groups' summaries; then every wave walks back over the summaries of the groups before its own to
+// the nearest one in which a run starts - one step when runs are shorter than 2^18 elements - and scans its group.
+__global__ __launch_bounds__(kMaxBlock) void key_group_tails_kernel(const unsigned *__restrict__ counts, const float *__restrict__ tail, unsigned *__restrict__ group_flag, float *__restrict__ group_tail,
+                                                                    size_t parts, size_t groups) {
+  const size_t g = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  if (g >= groups) return;
+  const int lane = lane_id();
+  const size_t i = g * 64 + lane;
+  unsigned F = i < parts && counts[i] > 0u ? 1u : 0u, fe;
+  float V = i < parts ? tail[i] : 0.0f, ve;
+  wave_exclusive_seg_scan(F, V, fe, ve);
+  seg_combine(fe, ve, F, V);
+  if (lane == 63) {
+    group_flag[g] = F;
+    group_tail[g] = V;
   }
-  if (lane == 0) {
-    wave_f[wave] = wf;
-    wave_v[wave] = wv;
+}
+__global__ __launch_bounds__(kMaxBlock) void close_boundary_runs_kernel(const unsigned *__restrict__ counts, const unsigned *__restrict__ group_prefix, const float *__restrict__ lead,
+                                                                        const float *__restrict__ tail, const unsigned *__restrict__ group_flag, const float *__restrict__ group_tail,
+                                                                        uint16_t *__restrict__ out, unsigned long long *num_runs, size_t parts, size_t groups) {
+  const size_t g = (size_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block();
+  if (g >= groups) return;
+  const int lane = lane_id();
+  // what comes into the group: the groups before it, from the nearest back to the first one in which a run starts
+  float carry = 0.0f;
+  for (long long base = (long long)g - 1; base >= 0; base -= 64) {
+    const long long at = base - lane;
+    const unsigned f = at >= 0 ? group_flag[at] : 1u;
+    const unsigned long long stops = ballot(f != 0u);
+    const int first_stop = stops ? __builtin_ctzll(stops) : 64;
+    float v = at >= 0 && lane <= first_stop ? group_tail[at] : 0.0f;
+    carry += readlane(lane_group_sum<6>(v), 63);
+    if (first_stop < 64) break;
   }
-  __syncthreads();
-  unsigned cf = 0;
-  float cv = 0.0f;
-  for (int w = 0; w < wave; w++) {
-    unsigned f = wave_f[w];
-    float v = wave_v[w];
-    seg_combine(cf, cv, f, v);
-    cf = f;
-    cv = v;
-  }
-  for (size_t s = 0; s < steps; s++) {
-    const size_t i = first + s * 64 + lane;
-    const unsigned before = i < parts ? prefix[i] : 0u;
-    const unsigned F = i < parts && prefix[i + 1] > before ? 1u : 0u;
-    const float V = i < parts ? tail[i] : 0.0f;
-    unsigned fe;
-    float ve;
-    wave_exclusive_seg_scan(F, V, fe, ve);
-    unsigned lf = fe;
-    float lv = ve;
-    seg_combine(cf, cv, lf, lv);
-    if (F && before > 0u) out[(size_t)before - 1] = f16_bits(lv + lead[i]);
-    unsigned fi = F;
-    float vi = V;
-    seg_combine(fe, ve, fi, vi);
-    unsigned tf = readlane_u32(fi, 63);
-    float tv = readlane(vi, 63);
-    seg_combine(cf, cv, tf, tv);
-    cf = tf;
-    cv = tv;
-  }
-  if (wave == kMaxWaves - 1 && lane == 0) {  // the last wave's stretch reaches the end of the partitions (or is empty)
-    const unsigned total = prefix[parts];
-    if (total > 0u) out[(size_t)total - 1] = f16_bits(cv);
-    if (num_runs) *num_runs = total;
+  const size_t i = g * 64 + lane;
+  const unsigned c = i < parts ? counts[i] : 0u;
+  unsigned F = c > 0u ? 1u : 0u, fe;
+  float V = i < parts ? tail[i] : 0.0f, ve;
+  wave_exclusive_seg_scan(F, V, fe, ve);
+  seg_combine(0u, carry, fe, ve);  // ve: what the run that comes into this partition has gathered
+  const unsigned before = group_prefix[g] + wave_exclusive_count(c);
+  if (F && before > 0u) out[(size_t)before - 1] = f16_bits(ve + lead[i]);
+  if (g + 1 == groups) {  // the run that reaches the end of the array
+    seg_combine(fe, ve, F, V);
+    const unsigned total = group_prefix[groups];
+    if (lane == 63) {
+      if (total > 0u) out[(size_t)total - 1] = f16_bits(V);
+      if (num_runs) *num_runs = total;
+    }
   }
 }
 

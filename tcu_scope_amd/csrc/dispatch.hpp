@@ -53,6 +53,7 @@ struct Options {
   unsigned test_mute_partition = 0;                  // tests only: partition test_mute_partition - 1 of a single-pass kernel publishes nothing
   bool by_key_reduce_chain = false;  // reduction by key: the one-pass look-back kernel instead of the four launches that wait for nothing
   int by_key_waves = 0;              // waves per block of the two big launches of the reduction by key (0 = default)
+  int by_key_key_tiles = 0;          // KiB of keys a wave of its first launch has in flight: 4, 8 or 16 (0 = default)
 };
 inline Options &options() {
   static Options o;
@@ -75,6 +76,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
   else if (n == "by_key_reduce_chain") o.by_key_reduce_chain = value != 0;
+  else if (n == "by_key_key_tiles") o.by_key_key_tiles = value == 4 || value == 8 || value == 16 ? value : 0;
   else if (n == "by_key_waves") o.by_key_waves = value < 0 ? 0 : (value > kMaxWaves ? kMaxWaves : value);
   else if (n == "gemm_staged_epilogue") o.gemm_staged_epilogue = value != 0;
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
@@ -976,25 +978,39 @@ inline int by_key_typed(const char *what, bool reduce, const void *d_keys, const
     char *w = static_cast<char *>(d_ws);
     unsigned long long *bits = reinterpret_cast<unsigned long long *>(w + lay.bits_at);
     KEY *list = d_keys_out ? reinterpret_cast<KEY *>(w + lay.list_at) : nullptr;
-    unsigned *counts = reinterpret_cast<unsigned *>(w + lay.counts_at);
-    float *lead = reinterpret_cast<float *>(w + lay.lead_at), *tail = reinterpret_cast<float *>(w + lay.tail_at);
+    unsigned *counts = reinterpret_cast<unsigned *>(w + lay.counts_at), *gprefix = reinterpret_cast<unsigned *>(w + lay.gprefix_at),
+             *gflag = reinterpret_cast<unsigned *>(w + lay.gflag_at);
+    float *lead = reinterpret_cast<float *>(w + lay.lead_at), *tail = reinterpret_cast<float *>(w + lay.tail_at), *gtail = reinterpret_cast<float *>(w + lay.gtail_at);
     const unsigned waves = options().by_key_waves > 0 ? (unsigned)options().by_key_waves : 1u;
     const size_t blocks = (lay.parts + waves - 1) / waves;
     if (blocks > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
     const unsigned run = options().xcd_run >= 0 ? (unsigned)options().xcd_run : 0u;
+    const unsigned group_blocks = (unsigned)((lay.groups + 3) / 4);  // the launches with a wave per group: 4 waves per block
     const KEY *keys = static_cast<const KEY *>(d_keys);
-    constexpr int G = sizeof(KEY) == 4 ? 8 : 4;
-    if (options().nontemporal) launch(key_heads_kernel<KEY, G, true>, (unsigned)blocks, waves * 64u, stream, keys, n, lay.parts, bits, counts, list, run);
-    else launch(key_heads_kernel<KEY, G, false>, (unsigned)blocks, waves * 64u, stream, keys, n, lay.parts, bits, counts, list, run);
-    launch(key_count_prefix_kernel, 1u, 1024u, stream, counts, lay.parts);
+    const unsigned *ccounts = counts, *cgprefix = gprefix;
+    uint16_t *out = static_cast<uint16_t *>(d_out);
+    const int in_flight = options().by_key_key_tiles ? options().by_key_key_tiles : 16;  // KiB of keys a wave has in flight
+#define TCU_KEY_HEADS(G_, NT_) launch(key_heads_kernel<KEY, G_, NT_>, (unsigned)blocks, waves * 64u, stream, keys, n, lay.parts, bits, counts, list, run)
+    if (options().nontemporal) {
+      if (in_flight == 4) TCU_KEY_HEADS(4, true);
+      else if (in_flight == 8) TCU_KEY_HEADS(8, true);
+      else TCU_KEY_HEADS(16, true);
+    } else {
+      if (in_flight == 4) TCU_KEY_HEADS(4, false);
+      else if (in_flight == 8) TCU_KEY_HEADS(8, false);
+      else TCU_KEY_HEADS(16, false);
+    }
+#undef TCU_KEY_HEADS
+    launch(key_group_prefix_kernel, 1u, 1024u, stream, ccounts, gprefix, lay.parts, lay.groups);
     if (options().nontemporal)
-      launch(reduce_by_heads_kernel<KEY, true>, (unsigned)blocks, waves * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<const unsigned long long *>(bits), static_cast<const unsigned *>(counts), keys,
-             static_cast<const KEY *>(list), static_cast<uint16_t *>(d_out), static_cast<KEY *>(d_keys_out), lead, tail, n, lay.parts, run);
+      launch(reduce_by_heads_kernel<KEY, true>, (unsigned)blocks, waves * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<const unsigned long long *>(bits), ccounts, cgprefix, keys,
+             static_cast<const KEY *>(list), out, static_cast<KEY *>(d_keys_out), lead, tail, n, lay.parts, run);
     else
-      launch(reduce_by_heads_kernel<KEY, false>, (unsigned)blocks, waves * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<const unsigned long long *>(bits), static_cast<const unsigned *>(counts), keys,
-             static_cast<const KEY *>(list), static_cast<uint16_t *>(d_out), static_cast<KEY *>(d_keys_out), lead, tail, n, lay.parts, run);
-    launch(close_boundary_runs_kernel, 1u, 1024u, stream, static_cast<const unsigned *>(counts), static_cast<const float *>(lead), static_cast<const float *>(tail), static_cast<uint16_t *>(d_out),
-           static_cast<unsigned long long *>(d_num_runs), lay.parts);
+      launch(reduce_by_heads_kernel<KEY, false>, (unsigned)blocks, waves * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<const unsigned long long *>(bits), ccounts, cgprefix, keys,
+             static_cast<const KEY *>(list), out, static_cast<KEY *>(d_keys_out), lead, tail, n, lay.parts, run);
+    launch(key_group_tails_kernel, group_blocks, 256u, stream, ccounts, static_cast<const float *>(tail), gflag, gtail, lay.parts, lay.groups);
+    launch(close_boundary_runs_kernel, group_blocks, 256u, stream, ccounts, cgprefix, static_cast<const float *>(lead), static_cast<const float *>(tail), static_cast<const unsigned *>(gflag),
+           static_cast<const float *>(gtail), out, static_cast<unsigned long long *>(d_num_runs), lay.parts, lay.groups);
     return TCU_OK;
   }
   unsigned *ws = static_cast<unsigned *>(d_ws);

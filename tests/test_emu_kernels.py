@@ -458,15 +458,19 @@ def test_segments_given_by_keys(emu, oracle, bits):
         want_scan = oracle.seg_scan_by_key_f64(keys, x).astype(np.float16).view(np.uint16)
         want_keys, want_sums = oracle.seg_reduce_by_key_f64(keys, x)
         want_sums = want_sums.astype(np.float16).view(np.uint16)
-        for static_order in (0, 1):
+        # the reduction in four launches that wait for nothing (one wave and four waves per block), then both
+        # operations on the one-pass look-back kernel with tickets and in block-index order
+        for static_order, chain, waves in ((0, 0, 0), (0, 0, 4), (0, 1, 0), (1, 1, 0)):
             emu.emu_set_option(b"static_order", static_order)
+            emu.emu_set_option(b"by_key_reduce_chain", chain)
+            emu.emu_set_option(b"by_key_waves", waves)
             d_keys, d_x = copy_in(keys, kt), copy_in(x)
             need = sz(0)
             assert emu.emu_seg_scan_by_key_f16(None, None, None, n, bits, None, ctypes.byref(need)) == 0
             ws = aligned(need.value, np.uint8, 0xAB)
             out = aligned(n, np.uint16, 0xFFFF)
             assert emu.emu_seg_scan_by_key_f16(d_keys.ctypes.data, d_x.ctypes.data, out.ctypes.data, n, bits, ws.ctypes.data, ctypes.byref(need)) == 0, emu.emu_last_error()
-            assert np.array_equal(out, want_scan), (n, mean_run, static_order)
+            assert np.array_equal(out, want_scan), (n, mean_run, static_order, chain)
             # in place
             assert emu.emu_seg_scan_by_key_f16(d_keys.ctypes.data, d_x.ctypes.data, d_x.ctypes.data, n, bits, ws.ctypes.data, ctypes.byref(need)) == 0
             assert np.array_equal(d_x[:n], want_scan)
@@ -479,7 +483,13 @@ def test_segments_given_by_keys(emu, oracle, bits):
             assert r == want_keys.size, (n, mean_run)
             assert np.array_equal(sums[:r], want_sums) and np.array_equal(keys_out[:r], want_keys.astype(kt))
             assert np.all(sums[r:] == 0xFFFF)  # nothing written past the runs
+            # without the keys
+            sums2 = aligned(n, np.uint16, 0xFFFF)
+            assert emu.emu_seg_reduce_by_key_f16(d_keys.ctypes.data, d_x.ctypes.data, None, sums2.ctypes.data, None, n, bits, ws.ctypes.data, ctypes.byref(need)) == 0, emu.emu_last_error()
+            assert np.array_equal(sums2, sums)
     emu.emu_set_option(b"static_order", 0)
+    emu.emu_set_option(b"by_key_reduce_chain", 0)
+    emu.emu_set_option(b"by_key_waves", 0)
     # empty input: no launch needed, the run count is cleared
     need, runs = sz(1 << 20), aligned(1, np.uint64, 99)
     ws = aligned(1 << 12, np.uint8)

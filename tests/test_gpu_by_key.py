@@ -63,19 +63,30 @@ def test_by_key_against_the_oracle(tcu, oracle, bits):
         tcu.seg_scan_by_key(kd, buf, out=buf)  # in place
         if exact and np.array_equal(wg.astype(np.float16).astype(np.float64), wg):
             assert np.array_equal(to_host(buf), wg.astype(np.float16).view(np.uint16)), what
-        # reduction
+        # reduction: the four launches that wait for nothing (one and four waves per block), then the one-pass look-back kernel
         want_keys, ref_sums = oracle.seg_reduce_by_key_f64(keys, x)
-        keys_out, sums, num = tcu.seg_reduce_by_key(kd, xd)
-        r = int(num.item())
-        assert r == want_keys.size == starts.size, what
-        assert np.array_equal(keys_out[:r].cpu().numpy(), want_keys.astype(kt)), what
-        gs = to_host(sums)[:r].view(np.float16).astype(np.float64)
-        bad = np.abs(gs - ref_sums) > allow_for(ref_sums, lens)
-        assert not bad.any(), (what, int(bad.sum()))
         _, wsum = oracle.seg_reduce_by_key_f64(keys, g)
-        if np.abs(wg).max() < 2048:  # exact fp32 partial sums in any order: one rounding, fixed bit for bit
-            _, gsum, _ = tcu.seg_reduce_by_key(kd, gd)
-            assert np.array_equal(to_host(gsum)[:r], wsum.astype(np.float16).view(np.uint16)), what
+        try:
+            for chain, waves in ((0, 0), (0, 4), (1, 0)):
+                tcu.set_option("by_key_reduce_chain", chain)
+                tcu.set_option("by_key_waves", waves)
+                what = (n, mean_run, bits, chain, waves)
+                keys_out, sums, num = tcu.seg_reduce_by_key(kd, xd)
+                r = int(num.item())
+                assert r == want_keys.size == starts.size, what
+                assert np.array_equal(keys_out[:r].cpu().numpy(), want_keys.astype(kt)), what
+                gs = to_host(sums)[:r].view(np.float16).astype(np.float64)
+                bad = np.abs(gs - ref_sums) > allow_for(ref_sums, lens)
+                assert not bad.any(), (what, int(bad.sum()))
+                if not chain:  # sums added in index order at every level: the same bits every time
+                    _, again, _ = tcu.seg_reduce_by_key(kd, xd)
+                    assert np.array_equal(to_host(again)[:r], to_host(sums)[:r]), what
+                if np.abs(wg).max() < 2048:  # exact fp32 partial sums in any order: one rounding, fixed bit for bit
+                    _, gsum, _ = tcu.seg_reduce_by_key(kd, gd)
+                    assert np.array_equal(to_host(gsum)[:r], wsum.astype(np.float16).view(np.uint16)), what
+        finally:
+            tcu.set_option("by_key_reduce_chain", 0)
+            tcu.set_option("by_key_waves", 0)
 
 
 def test_by_key_equals_the_fixed_size_kernels_at_full_size(tcu, oracle):
@@ -154,6 +165,12 @@ def test_by_key_arguments_and_expired_waits(tcu, oracle):
         ok = ~affected
         bad = np.abs(got[ok] - ref[ok]) > allow_for(ref[ok], np.repeat(lens, lens)[ok])
         assert not bad.any()
+        # the reduction's default form waits for nothing, so a silent partition means nothing to it
+        keys_out, sums, num = tcu.seg_reduce_by_key(kd, xd)
+        want_keys, ref_sums = oracle.seg_reduce_by_key_f64(keys, xh)
+        assert int(num.item()) == want_keys.size
+        assert not (np.abs(to_host(sums)[:want_keys.size].view(np.float16).astype(np.float64) - ref_sums) > allow_for(ref_sums, lens)).any()
+        tcu.set_option("by_key_reduce_chain", 1)  # its one-pass look-back form
         keys_out, sums, num = tcu.seg_reduce_by_key(kd, xd)
         assert int(num.item()) == -1  # all ones: unknown
         done = int((starts < mute * PART).sum()) - 1  # runs closed by the partitions that could still count
@@ -164,5 +181,6 @@ def test_by_key_arguments_and_expired_waits(tcu, oracle):
     finally:
         tcu.set_option("test_mute_partition", 0)
         tcu.set_option("lookback_poll_limit", -1)
+        tcu.set_option("by_key_reduce_chain", 0)
     got = to_host(tcu.seg_scan_by_key(kd, xd)).view(np.float16).astype(np.float64)
     assert not (np.abs(got - ref) > allow_for(ref, np.repeat(lens, lens))).any()
