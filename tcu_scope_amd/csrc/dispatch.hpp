@@ -51,6 +51,7 @@ struct Options {
   int xcd_run = -1;            // consecutive pieces of work per XCD (xcd_run_piece): -1 = the measured value for the size, 0 = none, C > 0 = C
   unsigned lookback_poll_limit = kDefaultPollLimit;  // polls of an unpublished value before a single-pass kernel gives up (results become NaN)
   unsigned test_mute_partition = 0;                  // tests only: partition test_mute_partition - 1 of a single-pass kernel publishes nothing
+  bool offsets_scan_chain = true;   // scan over offsets, expected segments beyond 65536 halves: one pass with look-back between a segment's slices instead of slice sums + a second read
   bool by_key_reduce_chain = false;  // reduction by key: the one-pass look-back kernel instead of the four launches that wait for nothing
   int by_key_waves = 0;              // waves per block of the two big launches of the reduction by key (0 = default)
   int by_key_key_tiles = 0;          // KiB of keys a wave of its first launch has in flight: 4, 8 or 16 (0 = default)
@@ -75,6 +76,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_strip_lds") o.gemv_strip_lds = value != 0;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
+  else if (n == "offsets_scan_chain") o.offsets_scan_chain = value != 0;
   else if (n == "by_key_reduce_chain") o.by_key_reduce_chain = value != 0;
   else if (n == "by_key_key_tiles") o.by_key_key_tiles = value == 4 || value == 8 || value == 16 ? value : 0;
   else if (n == "by_key_waves") o.by_key_waves = value < 0 ? 0 : (value > kMaxWaves ? kMaxWaves : value);
@@ -666,6 +668,10 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
 
 // ----- segmented inclusive prefix sum over an offsets array -----------------------------------
 
+// rounds of 1024 chunks a slice of the chained kernel keeps in registers: 8 for the 65536 halves a slice is cut to,
+// one more for segments that start off a chunk boundary or run up to an eighth over the expected length
+constexpr int kOffsetsChainRounds = 9;
+
 template <typename OFF>
 inline int seg_scan_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_segments, const OFF *begin, const OFF *end, size_t expected, void *stream) {
   // expected length of 1024 halves and more: a block per run of at most about 65536 halves of one
@@ -683,6 +689,21 @@ inline int seg_scan_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_
     const unsigned threads = expected < 2048 ? 64 : expected < 8192 ? 128 : expected <= 8192 ? 512 : 1024;
     const size_t blocks = num_segments * slices;
     if (blocks > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_scan_offsets_f16: grid exceeds the launch limit");
+    if (slices > 1 && options().offsets_scan_chain) {
+      // one pass: the slices of a segment meet through decoupled look-back (descriptors in stream-ordered temporary memory)
+      const unsigned shift = desc_shift_for(blocks);
+      const size_t words = look_back_words(blocks, shift);
+      unsigned *ws = static_cast<unsigned *>(stream_alloc(words * sizeof(unsigned), stream));
+      if (!ws) return fail(TCU_ERR_RUNTIME, "tcu_seg_scan_offsets_f16: no temporary device memory for the partition descriptors");
+      launch(zero_look_back_kernel, (unsigned)((blocks + 255) / 256), 256u, stream, ws, blocks, shift);
+      const int so = options().static_order ? 1 : 0;
+      if (ntl)
+        launch(seg_scan_offsets_chained_kernel<OFF, kOffsetsChainRounds, true>, (unsigned)blocks, 1024u, stream, in, out, begin, end, (unsigned)slices, vec, ws, so, wait_policy(shift, ws));
+      else
+        launch(seg_scan_offsets_chained_kernel<OFF, kOffsetsChainRounds, false>, (unsigned)blocks, 1024u, stream, in, out, begin, end, (unsigned)slices, vec, ws, so, wait_policy(shift, ws));
+      stream_free(ws, stream);
+      return TCU_OK;
+    }
     float *sums = nullptr;
     if (slices > 1) {
       sums = static_cast<float *>(stream_alloc(blocks * sizeof(float), stream));

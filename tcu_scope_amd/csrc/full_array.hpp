@@ -271,6 +271,141 @@ __global__ __launch_bounds__(kMaxBlock, 8) void full_scan_kernel(const half8_t *
   });
 }
 
+// The look-back scan over segments given by offsets: slice p of segment j (offsets_slice: the segment's aligned chunks
+// cut into `slices` equal stretches) is partition j * slices + p, and the look-back stops at the segment's first slice.
+// A slice of up to U rounds of blockDim chunks stays in registers between its sum and its scan, so every element is
+// read once; a longer one (the segment is far longer than the caller expected) is read twice by its block.
+// Same workspace layout as full_scan_kernel.
+template <typename OFF, int U, bool NT>
+__global__ __launch_bounds__(kMaxBlock, 8) void seg_scan_offsets_chained_kernel(const uint16_t *in, uint16_t *out, const OFF *__restrict__ begin, const OFF *__restrict__ end, unsigned slices, int vector,
+                                                                                unsigned *ws, int static_order, WaitPolicy wait) {
+  static_assert(U >= 2, "the streaming path keeps two rows of wave totals");
+  __shared__ float wave_total[U * kMaxWaves];  // [round][wave]; after the look-back: what precedes that wave's chunks of that round
+  __shared__ unsigned s_part;
+  __shared__ float s_prefix;
+  const int lane = lane_id(), wave = wave_in_block();
+  const int WPB = (int)(blockDim.x >> 6);
+  unsigned long long *desc = reinterpret_cast<unsigned long long *>(ws + 64);
+  if (!static_order) {
+    if (threadIdx.x == 0) s_part = atomic_add_u32(ws, 1u);
+    __syncthreads();
+  }
+  const unsigned part = static_order ? blockIdx.x : s_part;
+  const unsigned p = part % slices;
+  const OffsetsSlice s = offsets_slice(begin, end, part / slices, p, slices);
+  const bool resident = s.c_hi - s.c_lo <= (size_t)U * blockDim.x;  // block-uniform
+
+  half8_t v[U];
+  if (resident) {
+#pragma unroll
+    for (int r = 0; r < U; r++) {
+      const size_t c = s.c_lo + (size_t)r * blockDim.x + threadIdx.x;
+      v[r] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      bool whole;
+      if (c < s.c_hi) v[r] = offsets_masked_chunk<NT>(in, c, s.b, s.e, vector, &whole);
+    }
+#pragma unroll
+    for (int r = 0; r < U; r++) {
+      const float wt = lane_group_sum<6>(sum8(v[r], 0.0f));
+      if (lane == 63) wave_total[r * WPB + wave] = wt;
+    }
+  } else {
+    float acc = 0.0f;
+    for (size_t c = s.c_lo + threadIdx.x; c < s.c_hi; c += blockDim.x) {
+      bool whole;
+      acc = sum8(offsets_masked_chunk<false>(in, c, s.b, s.e, vector, &whole), acc);  // cached: read again below
+    }
+    acc = lane_group_sum<6>(acc);
+    if (lane == 63) wave_total[wave] = acc;
+  }
+  __syncthreads();
+
+  if (wave == 0) {
+    // exclusive scan of the totals in (round, wave) order, 64 at a time; the slice's sum falls out at the end
+    const int count = resident ? U * WPB : WPB;
+    float before[(U * kMaxWaves + 63) / 64];
+    float aggregate = 0.0f;
+#pragma unroll
+    for (int k = 0; k < (U * kMaxWaves + 63) / 64; k++) {
+      const int i = k * 64 + lane;
+      const float x = i < count ? wave_total[i] : 0.0f;
+      before[k] = aggregate + lane_group_exclusive_scan<6>(x, lane);
+      aggregate = readlane(before[k] + x, 63);
+    }
+    float prefix = 0.0f;
+    const bool muted = part + 1 == wait.mute_partition;
+    unsigned long long *mine = desc + ((size_t)part << wait.desc_shift);
+    if (p == 0) {
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagPrefix | __float_as_uint(aggregate));
+    } else {
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagAggregate | __float_as_uint(aggregate));
+      prefix = look_back(desc, (long long)part, (long long)part - p, lane, wait);
+      if (lane == 0 && !muted) atomic_store_u64(mine, kFlagPrefix | __float_as_uint(prefix + aggregate));
+    }
+    if (lane == 0) s_prefix = prefix;
+    if (resident) {
+#pragma unroll
+      for (int k = 0; k < (U * kMaxWaves + 63) / 64; k++) {
+        const int i = k * 64 + lane;
+        if (i < count) wave_total[i] = prefix + before[k];
+      }
+    }
+  }
+  __syncthreads();
+
+  if (resident) {
+#pragma unroll
+    for (int r = 0; r < U; r++) {
+      const size_t c = s.c_lo + (size_t)r * blockDim.x + threadIdx.x;
+      if (s.c_lo + (size_t)r * blockDim.x >= s.c_hi) break;  // block-uniform
+      const float e = lane_group_exclusive_scan<6>(sum8(v[r], 0.0f), lane);
+      const uint4_t packed = chunk_scan_packed(v[r], wave_total[r * WPB + wave] + e);
+      const size_t lo = c * 8;
+      if (c >= s.c_hi) continue;  // the round's last chunks lie beyond the slice
+      if (vector && lo >= s.b && lo + 8 <= s.e) {
+        store_chunk<NT>(reinterpret_cast<uint4_t *>(out) + c, packed);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+          if (lo + i >= s.b && lo + i < s.e) out[lo + i] = (uint16_t)(packed[i / 2] >> (16 * (i & 1)));
+      }
+    }
+    return;
+  }
+  float carry = s_prefix;
+  // the slice again, a round of blockDim chunks at a time (every thread runs the same number of rounds: barriers inside)
+  unsigned parity = 0;
+  for (size_t c0 = s.c_lo; c0 < s.c_hi; c0 += blockDim.x) {
+    const size_t c = c0 + threadIdx.x;
+    const bool any = c < s.c_hi;
+    bool whole = false;
+    half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (any) x = offsets_masked_chunk<NT>(in, c, s.b, s.e, vector, &whole);
+    const float t = sum8(x, 0.0f);
+    const float e = lane_group_exclusive_scan<6>(t, lane);
+    const float wt = lane_group_sum<6>(t);
+    if (lane == 63) wave_total[parity * WPB + wave] = wt;
+    __syncthreads();
+    float before = 0.0f, all = 0.0f;
+    for (int w = 0; w < WPB; w++) {
+      const float y = wave_total[parity * WPB + w];
+      if (w < wave) before += y;
+      all += y;
+    }
+    parity ^= 1u;
+    const uint4_t packed = chunk_scan_packed(x, carry + before + e);
+    carry += all;
+    if (whole) {
+      store_chunk<NT>(reinterpret_cast<uint4_t *>(out) + c, packed);
+    } else if (any) {
+      const size_t lo = c * 8;
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        if (lo + i >= s.b && lo + i < s.e) out[lo + i] = (uint16_t)(packed[i / 2] >> (16 * (i & 1)));
+    }
+  }
+}
+
 // The look-back scan with more bytes in flight per wave slot.  A block of full_scan_kernel
 // waits about 30 % of its life for its predecessors' aggregates with its whole partition
 // parked in registers and nothing in flight; wave slots (32 per CU), not registers, cap what a

@@ -198,6 +198,25 @@ def test_segmented_scan_over_offsets(emu, oracle):
         out = aligned(n + 64, np.uint16, 0xFFFF)
         assert emu.emu_seg_scan_offsets_f16(xi.ctypes.data, out.ctypes.data, nseg, bi.ctypes.data, ei.ctypes.data, bits, expected) == 0, emu.emu_last_error()
         assert np.array_equal(out[:n], want) and np.all(out[n:] == 0xFFFF), (nseg, expected, bits)
+    # segments far longer than expected: slices that do not fit a block's registers are read twice by their block;
+    # and the slice sums + second read form of the same lengths
+    n2 = 200000
+    x2 = oracle.generate_f16(n2, 11, oracle.DIST_GRID)
+    x2i = copy_in(x2)
+    begin, end = np.array([3, 199000], np.int64), np.array([198999, 199990], np.int64)
+    w64 = oracle.seg_scan_offsets_f64(x2, begin, end)
+    inside = ~np.isnan(w64)
+    want = np.full(n2, 0xFFFF, np.uint16)
+    want[inside] = w64[inside].astype(np.float16).view(np.uint16)
+    bi, ei = copy_in(begin, np.int64), copy_in(end, np.int64)
+    for chain, static_order in ((1, 0), (1, 1), (0, 0)):
+        emu.emu_set_option(b"offsets_scan_chain", chain)
+        emu.emu_set_option(b"static_order", static_order)
+        out = aligned(n2 + 64, np.uint16, 0xFFFF)
+        assert emu.emu_seg_scan_offsets_f16(x2i.ctypes.data, out.ctypes.data, 2, bi.ctypes.data, ei.ctypes.data, 64, 65537) == 0, emu.emu_last_error()
+        assert np.array_equal(out[:n2], want) and np.all(out[n2:] == 0xFFFF), (chain, static_order)
+    emu.emu_set_option(b"offsets_scan_chain", 1)
+    emu.emu_set_option(b"static_order", 0)
     # uniform offsets from one array (begin = offsets, end = offsets + 1) == the fixed-size scan; in place
     seg, nseg = 200, 150
     off = copy_in((np.arange(nseg + 1) * seg).astype(np.int32), np.int32)

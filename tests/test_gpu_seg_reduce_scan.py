@@ -416,7 +416,11 @@ def test_segmented_scan_over_offsets(tcu, oracle):
         exact = np.nanmax(np.abs(wg)) < 4096
         for dtype in (torch.int32, torch.int64):
             bd, ed = torch.from_numpy(begin).to(dtype).cuda(), torch.from_numpy(end).to(dtype).cuda()
-            for expected in (0, 16, 40, 100, 1500, 5000) + ((1 << 16, 300000) if nseg <= 500 else ()):  # the last two: several blocks per segment
+            # the last two: several blocks per segment; 300000: slices that meet through look-back (slices longer than a
+            # block holds when nseg = 3), and once more (-300000) as slice sums + a second read
+            for expected in (0, 16, 40, 100, 1500, 5000) + ((1 << 16, 300000, -300000) if nseg <= 500 else ()):
+                tcu.set_option("offsets_scan_chain", 0 if expected < 0 else 1)
+                expected = abs(expected)
                 out = torch.full((n,), -7.0, dtype=torch.float16, device="cuda")
                 tcu.seg_scan_offsets(xd, bd, ed, expected_segment_size=expected, out=out)
                 got = to_host(out)
