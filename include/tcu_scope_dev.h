@@ -24,6 +24,8 @@ extern "C" {
  *                     reach HBM; a scan whose output must reach HBM (outputs taken in turn, or 2 GiB of output) runs
  *                     1-3 % slower with it
  *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
+ *   "offsets_scan_chain" 0/1, default 1: tcu_seg_scan_offsets_f16 with expected segments beyond 65536 halves in one pass (a
+ *                     segment's slices meet through decoupled look-back) instead of slice sums followed by a second read
  *   "by_key_reduce_chain" 0/1, default 0: tcu_seg_reduce_by_key_f16 as one pass with a decoupled look-back (the form of the
  *                     scan by key; a wait that expires leaves ~0 in *d_num_runs and NaN in the sums that depended on it)
  *                     instead of the five launches that wait for nothing
