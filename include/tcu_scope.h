@@ -21,7 +21,7 @@
  *     tcu_seg_reduce_f16 with segments of 2^20 halves and more and tcu_seg_scan_f16 from 2^21
  *     (reduction: 4 bytes per 4096 input halves, and a thousandth of that again for segments
  *     beyond 2^25; scan: 256 bytes per 65536 input halves), the *_offsets_f16 entry points with
- *     expected segment lengths of 2^17 and more (4 bytes per 65536 halves), and tcu_gemm_* when the
+ *     expected segment lengths beyond 65536 halves (reduction 4, scan up to 256 bytes per 65536 halves), and tcu_gemm_* when the
  *     last round of output tiles is sparsely filled (up to 128 MiB).  The full-array entry
  *     points work in the caller's workspace; tcu_seg_scan_f16_noalloc never allocates.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only
