@@ -128,6 +128,7 @@ def by_key_case(rng, emu, oracle):
     assert np.array_equal(out, want_scan), ("scan",) + tag
     runs = int(heads.sum())
     ko, so, nr = aligned(runs, dt, -1), aligned(runs, np.uint16, 0xFFFF), aligned(1, np.uint64, 0)
+    assert emu.emu_seg_reduce_by_key_f16(None, None, None, None, None, n, bits, None, ctypes.byref(need)) == 0  # the reduction's own workspace size
     ws = aligned(need.value, np.uint8, 0xAB)
     assert emu.emu_seg_reduce_by_key_f16(ki.ctypes.data, xi.ctypes.data, ko.ctypes.data, so.ctypes.data, nr.ctypes.data, n, bits, ws.ctypes.data, ctypes.byref(need)) == 0, emu.emu_last_error()
     starts = np.flatnonzero(heads)
