@@ -455,8 +455,9 @@ __global__ __launch_bounds__(kMaxBlock) void by_key_kernel(const KEY *__restrict
 // A partition is one wave's work in launches 1 and 3 (8 tiles of values), so both are grids of small blocks that
 // depend on nothing; launches 2, 4 and 5 touch a few bytes per partition.  The bits of a partition are kept
 // lane-major for launch 3: lane l owns 8 bytes, byte j = its chunk of tile j.
-// Measured (2^28 elements, 32-bit keys): launch 1 165-187 us (0.86 of the HBM peak as long as it writes nothing;
-// the bits, 3 % of its bytes, cost 10 %), launch 3 82-120 us, the three small ones 21 us together.
+// Measured (2^28 elements, 32-bit keys, runs of 16384 / 16 elements): launch 1 169 / 192 us (0.86 of the HBM peak as
+// long as it writes nothing; the bits, 3 % of its bytes, cost 10 %), launch 3 83 / 122 us, the three small ones 21 us
+// together; per call 265 / 334 us against 384 / 437 us for the one-pass kernel.
 
 constexpr int kKeyPartTiles = 8;
 constexpr size_t kKeyPartElems = (size_t)kKeyPartTiles * kTileChunks * 8;  // 4096
