@@ -118,6 +118,40 @@ def test_by_key_equals_the_fixed_size_kernels_at_full_size(tcu, oracle):
     assert torch.equal(sums[:1].view(torch.int16), tcu.full_reduce(g).view(torch.int16))
 
 
+def test_by_key_at_the_largest_size(tcu, oracle):
+    """n = 2^32 - 24, the most the by-key entry points take (runs are counted in 32 bits): 32-bit keys = index / 4099
+    (runs that start anywhere in a partition), exact-grid values; the scan against the fixed-size kernel wherever runs
+    and segments coincide is not available at this run length, so both results are checked through properties that do
+    not depend on the size: the reduction's sums equal the scan's value at every run's last element, the number of runs
+    and their keys are what the keys say, and a sample of runs is summed again with torch in fp64."""
+    import torch
+
+    free = torch.cuda.mem_get_info()[0]
+    if free < 80 << 30:
+        pytest.skip("needs 80 GiB of free device memory")
+    n, seg = (1 << 32) - 24, 4099
+    g = tcu.generate(n, 78, tcu.Dist.GRID)
+    keys = torch.empty(n, dtype=torch.int32, device="cuda")
+    step = 1 << 28
+    for lo in range(0, n, step):  # keys = index / seg without a 32 GiB index array
+        hi = min(n, lo + step)
+        keys[lo:hi] = (torch.arange(lo, hi, dtype=torch.int64, device="cuda") // seg).to(torch.int32)
+    runs = (n + seg - 1) // seg
+    keys_out, sums, num = tcu.seg_reduce_by_key(keys, g)
+    assert int(num.item()) == runs
+    assert torch.equal(keys_out[:runs], torch.arange(runs, dtype=torch.int32, device="cuda"))
+    scan = tcu.seg_scan_by_key(keys, g)
+    last = torch.arange(1, runs + 1, dtype=torch.int64, device="cuda") * seg - 1
+    last[-1] = n - 1
+    assert torch.equal(sums[:runs].view(torch.int16), scan[last].view(torch.int16))
+    for r in (0, 1, 65535, 65536, runs // 2, runs - 2, runs - 1):  # around partition and group boundaries, and both ends
+        lo, hi = r * seg, min(n, (r + 1) * seg)
+        want = g[lo:hi].double().sum().half()  # |sum| < 4099 / 2048: exact in fp64, one rounding
+        assert sums[r].view(torch.int16) == want.view(torch.int16), r
+        inside = g[lo:hi].double().cumsum(0).half()
+        assert torch.equal(scan[lo:hi].view(torch.int16), inside.view(torch.int16)), r
+
+
 def test_by_key_arguments_and_expired_waits(tcu, oracle):
     import ctypes
 
