@@ -488,7 +488,7 @@ inline int seg_reduce_offsets_typed(const uint16_t *in, uint16_t *out, size_t nu
   // block per segment adds them.  (A wave per segment: 158 us at 2^19, 57 ms for one 2^28 segment.)
   if (expected >= ((size_t)1 << 17)) {
     size_t slices = (expected + 65535) / 65536;
-    if (slices > 4096) slices = 4096;
+    if (slices > 65536) slices = 65536;  // one segment of 2^32 halves
     const size_t blocks = num_segments * slices;
     if (blocks > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, "tcu_seg_reduce_offsets_f16: grid exceeds the launch limit");
     float *partials = static_cast<float *>(stream_alloc(blocks * sizeof(float), stream));
@@ -684,7 +684,7 @@ inline int seg_scan_offsets_typed(const uint16_t *in, uint16_t *out, size_t num_
     const int vec = aligned16(in) && aligned16(out) ? 1 : 0;
     const bool ntl = options().nontemporal;
     size_t slices = (expected + 65535) / 65536;
-    if (slices > 4096) slices = 4096;
+    if (slices > 65536) slices = 65536;  // one segment of 2^32 halves
     // two to four rounds per block measure best (N = 2^28: S = 1024 with 64 threads 165 us, 180 with groups of 16
     // lanes; S = 2048 with 128 threads 164, with 256 184; S = 4096 with 128 threads 167.5, with 256 173)
     const unsigned threads = expected < 2048 ? 64 : expected < 8192 ? 128 : expected <= 8192 ? 512 : 1024;

@@ -440,6 +440,45 @@ def test_segmented_scan_over_offsets(tcu, oracle):
         assert np.array_equal(to_host(buf), oracle.seg_scan_f64(g, nseg, seg).astype(np.float16).view(np.uint16)), seg
 
 
+def test_offsets_one_segment_beyond_2_to_the_31(tcu, oracle):
+    """A segment of 2^31 + 11 halves that starts off a chunk boundary, 64-bit offsets, and a short one behind it: 32769
+    slices that meet through look-back.  The values repeat (-3 ... 3) / 2048, so every prefix is one of seven small
+    numbers and the whole output is checked against the closed form, chunk by chunk; nothing outside the segments is
+    written; the reduction over the same offsets gives the two closed-form sums."""
+    import torch
+
+    if torch.cuda.mem_get_info()[0] < 40 << 30:
+        pytest.skip("needs 40 GiB of free device memory")
+    n = (1 << 31) + 64
+    cycle = torch.tensor([-3, -2, -1, 0, 1, 2, 3], dtype=torch.float32, device="cuda") / 2048
+    upto = torch.cumsum(cycle, 0)  # sum of the first r + 1 values of a cycle; whole cycles add nothing
+    g = torch.empty(n, dtype=torch.float16, device="cuda")
+    step = 1 << 28
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        g[lo:hi] = cycle[torch.arange(lo, hi, dtype=torch.int64, device="cuda") % 7].half()
+    length = (1 << 31) + 11
+    begin = torch.tensor([5, 5 + length + 3], dtype=torch.int64, device="cuda")
+    end = torch.tensor([5 + length, n - 1], dtype=torch.int64, device="cuda")
+    out = torch.full((n,), -7.0, dtype=torch.float16, device="cuda")
+    tcu.seg_scan_offsets(g, begin, end, expected_segment_size=length, out=out)
+
+    def prefix(i, b):  # sum of g[b .. i]
+        return upto[i % 7] - (upto[(b - 1) % 7] if (b % 7) else 0.0)
+
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        i = torch.arange(lo, hi, dtype=torch.int64, device="cuda")
+        want = torch.full((hi - lo,), -7.0, dtype=torch.float32, device="cuda")
+        for b, e in ((5, 5 + length), (5 + length + 3, n - 1)):
+            inside = (i >= b) & (i < e)
+            want = torch.where(inside, prefix(i, b), want)
+        assert torch.equal(out[lo:hi].view(torch.int16), want.half().view(torch.int16)), lo
+    sums = tcu.seg_reduce_offsets(g, begin, end, expected_segment_size=length)
+    want = torch.stack([prefix(torch.tensor(int(e) - 1, device="cuda"), int(b)) for b, e in zip(begin.tolist(), end.tolist())]).half()
+    assert torch.equal(sums.view(torch.int16), want.view(torch.int16))
+
+
 def test_time_next_launch(tcu):
     """tcu_time_next_launch: the events are stamped by the kernel itself, only the next launch carries them, and the
     duration lies between what the bytes need at 8 TB/s and the wall-clock time of the call."""
