@@ -49,8 +49,9 @@ extern "C" {
 /* 2: entry points over offsets and key arrays, tcu_seg_scan_f16_noalloc, the TCU_FULL_MFMA flag, block variants from 16
  * halves per segment, 256 bytes of workspace per partition of the full-array scan (a cached size from version 1 is too
  * small), tcu_init fails when the scratch symbol cannot be resolved; the tuning switches and measurement aids moved to
- * tcu_scope_dev.h. */
-#define TCU_SCOPE_ABI_VERSION 2
+ * tcu_scope_dev.h.
+ * 3: tcu_gemv_col_major_f16_f32 / _f16; the workspace of tcu_seg_reduce_by_key_f16 grew (ask again: about 0.63 n bytes). */
+#define TCU_SCOPE_ABI_VERSION 3
 
 typedef enum {
   TCU_OK = 0,
@@ -219,13 +220,22 @@ int tcu_full_scan_f16(const void *d_in, void *d_out, size_t n, void *d_workspace
 /* y = alpha * A x + beta * y.  A: M x K row-major fp16, x: K fp16, y: M fp32.
  * Replaces compute_wmma_gemv_naive / compute_wmma_gemv_sharedmem (reference
  * src/gemv/wmma_naive.cu:29-94, wmma_sharedmem.cu:43-137); note the reference stores A
- * column-major and returns y as column 0 of an M x 16 matrix.
+ * column-major (tcu_gemv_col_major_* below take that layout) and returns y as column 0 of an M x 16 matrix.
  * variant: TCU_VARIANT_AUTO, TCU_VARIANT_WAVE_SHUFFLE (dot products + DPP),
  * TCU_VARIANT_MFMA_16N (16-row strips on MFMA with x as a replicated B operand, the
  * reference's formulation) or TCU_VARIANT_MFMA_256N (a 1 KiB tile of a row as the MFMA A
  * operand, the matching tile of x as the B operand, trace of the accumulated product: the
  * launch shapes and loads of the dot-product form with the arithmetic on the matrix unit). */
 int tcu_gemv_f16_f32(const void *d_A, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, int variant, void *stream);
+
+/* The same product with A column-major, element (m, k) at d_A[m + k * lda] (lda >= M, in elements): the layout in which
+ * the reference's own kernels and its cuBLAS baseline take A (src/gemv/wmma_naive.cu:33-36, 61: lda = M_GLOBAL,
+ * fragments loaded col_major), so a caller that holds the reference's buffers passes them as they are.  y: M values of
+ * fp32 (_f32) or fp16 (_f16).  Columns are read 1 KiB at a time and scaled by x[k]; the sums of stretches of K meet in
+ * M floats per stretch of stream-ordered temporary memory (up to 64 stretches) and are added in a fixed order.  K a
+ * multiple of 8, lda a multiple of 8 and 16-byte aligned A and x take the fast kernels, anything else a scalar one. */
+int tcu_gemv_col_major_f16_f32(const void *d_A, size_t lda, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, void *stream);
+int tcu_gemv_col_major_f16_f16(const void *d_A, size_t lda, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, void *stream);
 
 /* D = alpha * A B + beta * C.  A: M x K row-major fp16; B: K x N column-major fp16
  * (element (k,n) at d_B[n*K + k]); C, D: M x N row-major fp32 (C may equal D, may be

@@ -22,6 +22,7 @@ from .binding import (  # noqa: F401
     full_scan,
     gemm,
     gemv,
+    gemv_col_major,
     generate,
     init,
     lane_probe,

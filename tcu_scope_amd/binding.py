@@ -12,7 +12,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 EXPORTS = [
     "tcu_abi_version", "tcu_last_error", "tcu_init", "tcu_device_info", "tcu_set_option",
     "tcu_seg_reduce_f16", "tcu_seg_reduce_offsets_f16", "tcu_seg_scan_f16", "tcu_seg_scan_f16_noalloc", "tcu_seg_scan_offsets_f16", "tcu_seg_scan_by_key_f16", "tcu_seg_reduce_by_key_f16", "tcu_add_partial_sums_f16",
-    "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32", "tcu_gemv_f16_f16", "tcu_gemm_f16_f16",
+    "tcu_full_reduce_f16", "tcu_full_scan_f16", "tcu_gemv_f16_f32", "tcu_gemm_f16_f32", "tcu_gemv_f16_f16", "tcu_gemm_f16_f16", "tcu_gemv_col_major_f16_f32", "tcu_gemv_col_major_f16_f16",
     "tcu_fill_f16", "tcu_convert_f32_to_f16", "tcu_generate_f16", "tcu_stream_probe", "tcu_time_next_launch", "tcu_lane_probe", "tcu_temporary_allocations",
 ]
 
@@ -98,6 +98,8 @@ def lib():
         L.tcu_gemv_f16_f32.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci, vp]
         L.tcu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci, vp]
         L.tcu_gemv_f16_f16.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci, vp]
+        L.tcu_gemv_col_major_f16_f32.argtypes = [vp, sz, vp, vp, sz, sz, cf, cf, vp]
+        L.tcu_gemv_col_major_f16_f16.argtypes = [vp, sz, vp, vp, sz, sz, cf, cf, vp]
         L.tcu_gemm_f16_f16.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci, vp]
         L.tcu_fill_f16.argtypes = [vp, cf, sz, vp]
         L.tcu_convert_f32_to_f16.argtypes = [vp, vp, sz, vp]
@@ -332,6 +334,21 @@ def gemv(A, x, alpha=1.0, beta=0.0, y=None, variant=Variant.AUTO, stream=None, o
         y = torch.zeros(M, dtype=out_dtype or torch.float32, device=A.device)
     entry = _out_entry(y, "y", lib().tcu_gemv_f16_f32, lib().tcu_gemv_f16_f16)
     _check(entry(_ptr(A), _ptr(x), _ptr(y), M, K, alpha, beta, int(variant), _stream(stream)))
+    return y
+
+
+def gemv_col_major(At, x, alpha=1.0, beta=0.0, y=None, stream=None, out_dtype=None):
+    """y = alpha*A@x + beta*y with A column-major: `At` is the (K, M) fp16 tensor whose row k is column k of A (rows may be
+    further apart than M elements: lda = At.stride(0)); x (K,) fp16, y (M,) fp32 or fp16 (tcu_gemv_col_major_f16_f32 / _f16)."""
+    torch = _torch()
+    _need_f16(x, "x")
+    if At.dtype != torch.float16 or not At.is_cuda or At.dim() != 2 or At.stride(1) != 1:
+        raise ValueError("At must be a CUDA float16 matrix that holds the columns of A contiguously (stride 1 along its second dimension)")
+    K, M = At.shape
+    if y is None:
+        y = torch.zeros(M, dtype=out_dtype or torch.float32, device=At.device)
+    entry = _out_entry(y, "y", lib().tcu_gemv_col_major_f16_f32, lib().tcu_gemv_col_major_f16_f16)
+    _check(entry(ctypes.c_void_p(At.data_ptr()), At.stride(0) if K > 1 else M, _ptr(x), _ptr(y), M, K, alpha, beta, _stream(stream)))
     return y
 
 

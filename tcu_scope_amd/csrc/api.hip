@@ -199,6 +199,16 @@ int tcu_gemv_f16_f16(const void *d_A, const void *d_x, void *d_y, size_t M, size
   return after_launch("tcu_gemv_f16_f16", before, tcu::hgemv_dispatch(d_A, d_x, d_y, M, K, alpha, beta, variant, stream));
 }
 
+int tcu_gemv_col_major_f16_f32(const void *d_A, size_t lda, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_gemv_col_major_f16_f32", before, tcu::gemv_col_major_dispatch<float>("tcu_gemv_col_major_f16_f32", d_A, lda, d_x, d_y, M, K, alpha, beta, stream));
+}
+
+int tcu_gemv_col_major_f16_f16(const void *d_A, size_t lda, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, void *stream) {
+  const unsigned long before = tcu::launch_count();
+  return after_launch("tcu_gemv_col_major_f16_f16", before, tcu::gemv_col_major_dispatch<tcu::half_t>("tcu_gemv_col_major_f16_f16", d_A, lda, d_x, d_y, M, K, alpha, beta, stream));
+}
+
 int tcu_gemm_f16_f16(const void *d_A, const void *d_B, const void *d_C, void *d_D, size_t M, size_t N, size_t K, float alpha, float beta, int variant, void *stream) {
   const unsigned long before = tcu::launch_count();
   return after_launch("tcu_gemm_f16_f16", before, tcu::hgemm_dispatch(d_A, d_B, d_C, d_D, M, N, K, alpha, beta, variant, stream));

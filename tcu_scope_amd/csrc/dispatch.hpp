@@ -43,6 +43,7 @@ struct Options {
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
+  int gemv_col_shape = 42;     // column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2)
   bool gemv_strip_lds = true;  // strip GEMV (TCU_VARIANT_MFMA_16N): stage the strip through LDS where K is a multiple of 512
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
   int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
@@ -73,6 +74,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_rows") o.gemv_rows = value;
   else if (n == "gemv_tiles") o.gemv_tiles = value;
   else if (n == "gemv_waves") o.gemv_waves = value;
+  else if (n == "gemv_col_shape") o.gemv_col_shape = value;
   else if (n == "gemv_strip_lds") o.gemv_strip_lds = value != 0;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
@@ -1162,6 +1164,54 @@ inline int gemv_dispatch_typed(const char *what, const void *A, const void *x, v
     launch(gemv_dot_kernel<ROWS, UK, false, OUT>, (unsigned)grid, block, stream, a, xv, yy, M, K / 8, alpha, beta);
   return TCU_OK;
 }
+// A column-major (tcu_gemv_col_major_f16_f32 / _f16)
+template <typename OUT>
+inline int gemv_col_major_dispatch(const char *what, const void *A, size_t lda, const void *x, void *y, size_t M, size_t K, float alpha, float beta, void *stream) {
+  if (M == 0) return TCU_OK;
+  if (!y || (K && (!A || !x))) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": null device pointer");
+  if (lda < M) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": lda must be at least M");
+  const uint16_t *a = static_cast<const uint16_t *>(A);
+  OUT *yy = static_cast<OUT *>(y);
+  const bool vec_ok = K > 0 && K % 8 == 0 && lda % 8 == 0 && aligned16(A) && aligned16(x);
+  if (!vec_ok) {
+    const size_t grid = (M + 255) / 256;
+    if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    launch(gemv_col_generic_kernel<OUT>, (unsigned)grid, 256u, stream, a, lda, static_cast<const uint16_t *>(x), yy, M, K, alpha, beta);
+    return TCU_OK;
+  }
+  // slabs of 512 rows; K is cut into stretches so that about 2048 blocks run and a wave still takes two rounds or more
+  // (16384 x 16384: 32 slabs x 64 stretches of 256 columns)
+  const int shape = options().gemv_col_shape;  // waves per block * 10 + groups of 8 columns per wave and round
+  const unsigned waves = shape / 10 == 8 ? 8u : 4u, groups = shape % 10 == 1 ? 1u : 2u;
+  const size_t round = (size_t)8 * groups * waves;  // columns per round of a block
+  const size_t slabs = (M + kColSlabRows - 1) / kColSlabRows;
+  size_t stretches = (2048 + slabs - 1) / slabs;
+  const size_t most = (K + 2 * round - 1) / (2 * round);
+  if (stretches > most) stretches = most;
+  if (stretches < 1) stretches = 1;
+  size_t cols = (K + stretches - 1) / stretches;
+  cols = (cols + round - 1) / round * round;  // whole rounds of the block's waves
+  stretches = (K + cols - 1) / cols;
+  if (slabs * stretches > kMaxGrid || slabs > 0xffffffffu) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+  float *partials = static_cast<float *>(stream_alloc(stretches * M * sizeof(float), stream));
+  if (!partials) return fail(TCU_ERR_RUNTIME, std::string(what) + ": no temporary device memory for the partial sums");
+  const unsigned grid = (unsigned)(slabs * stretches);
+  const half8_t *xv = static_cast<const half8_t *>(x);
+#define TCU_GEMV_COL(W_, G_)                                                                                                              \
+  do {                                                                                                                                    \
+    if (options().nontemporal) launch(gemv_col_partials_kernel<W_, G_, true>, grid, W_ * 64u, stream, a, lda, xv, partials, M, K, (unsigned)slabs, cols); \
+    else launch(gemv_col_partials_kernel<W_, G_, false>, grid, W_ * 64u, stream, a, lda, xv, partials, M, K, (unsigned)slabs, cols);      \
+  } while (0)
+  if (waves == 8 && groups == 1) TCU_GEMV_COL(8, 1);
+  else if (waves == 8) TCU_GEMV_COL(8, 2);
+  else if (groups == 1) TCU_GEMV_COL(4, 1);
+  else TCU_GEMV_COL(4, 2);
+#undef TCU_GEMV_COL
+  launch(gemv_col_finish_kernel<OUT>, (unsigned)((M + 255) / 256), 256u, stream, static_cast<const float *>(partials), yy, M, (unsigned)stretches, alpha, beta);
+  stream_free(partials, stream);
+  return TCU_OK;
+}
+
 inline int gemv_dispatch(const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
   return gemv_dispatch_typed<float>("tcu_gemv_f16_f32", A, x, y, M, K, alpha, beta, variant, stream);
 }

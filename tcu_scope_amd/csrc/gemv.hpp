@@ -260,4 +260,98 @@ __global__ __launch_bounds__(kMaxBlock) void gemv_generic_kernel(const uint16_t 
   if (lane == 63) gemv_update(y + row, acc, alpha, beta);
 }
 
+// ---- A column-major ------------------------------------------------------------------------------------------
+// y = alpha * A x + beta * y with element (m, k) of A at A[m + k * lda]: the layout of the reference's
+// compute_wmma_gemv_naive (src/gemv/wmma_naive.cu:33-36, 61: lda = M_GLOBAL, fragments loaded col_major) and of the
+// cuBLAS call beside it.  A column is contiguous, so the product is a sum of columns scaled by x[k]: a wave owns
+// kColSlabRows consecutive rows (a lane 8 of them: one 16-byte load per column, the wave 1 KiB) and every WPB-th
+// group of 8 columns of its block's stretch of K; the waves of a block add up in LDS and the block writes one fp32
+// partial sum per row; gemv_col_finish_kernel adds the partials of a row in the order of the stretches and applies
+// alpha, beta and y.  Every sum is taken in a fixed order.
+constexpr int kColSlabRows = 512;
+
+template <int WPB, int GROUPS, bool NT>
+__global__ __launch_bounds__(WPB * 64) void gemv_col_partials_kernel(const uint16_t *__restrict__ A, size_t lda, const half8_t *__restrict__ x, float *__restrict__ partials, size_t M, size_t K,
+                                                                     unsigned slabs, size_t cols_per_block) {
+  __shared__ float sums[WPB][kColSlabRows];
+  const int lane = lane_id(), wave = wave_in_block();
+  const size_t slab = blockIdx.x % slabs, stretch = blockIdx.x / slabs;
+  const size_t r0 = slab * kColSlabRows + (size_t)lane * 8;
+  const int valid = r0 >= M ? 0 : (M - r0 >= 8 ? 8 : (int)(M - r0));
+  const size_t k_lo = stretch * cols_per_block, k_hi = k_lo + cols_per_block < K ? k_lo + cols_per_block : K;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+  // GROUPS groups of 8 columns per wave and round (8 * GROUPS loads in flight); K is a multiple of 8: whole groups
+  for (size_t kb = k_lo + (size_t)wave * 8 * GROUPS; kb < k_hi; kb += (size_t)WPB * 8 * GROUPS) {
+    half8_t xs[GROUPS], a[GROUPS][8];
+#pragma unroll
+    for (int g = 0; g < GROUPS; g++) {
+      const size_t kg = kb + (size_t)g * 8;
+      const bool there = kg < k_hi;  // wave-uniform
+      xs[g] = there ? x[kg / 8] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const uint16_t *col = A + (kg + j) * lda + r0;
+        a[g][j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if (there && valid == 8) {
+          a[g][j] = load_chunk<NT>(reinterpret_cast<const half8_t *>(col));
+        } else if (there) {
+#pragma unroll
+          for (int i = 0; i < 8; i++)
+            if (i < valid) a[g][j][i] = __builtin_bit_cast(half_t, col[i]);
+        }
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < GROUPS; g++) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const float xk = (float)xs[g][j];
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = __builtin_fmaf((float)a[g][j][i], xk, acc[i]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) sums[wave][lane * 8 + i] = acc[i];
+  __syncthreads();
+  for (int r = (int)threadIdx.x; r < kColSlabRows; r += WPB * 64) {
+    const size_t row = slab * kColSlabRows + r;
+    if (row >= M) break;
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WPB; w++) s += sums[w][r];
+    partials[stretch * M + row] = s;
+  }
+}
+
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemv_col_finish_kernel(const float *__restrict__ partials, OUT *__restrict__ y, size_t M, unsigned stretches, float alpha, float beta) {
+  const size_t row = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= M) return;
+  float s = 0.0f;
+  unsigned c = 0;
+  for (; c + 8 <= stretches; c += 8) {  // eight loads in flight, added in the order of the stretches
+    float p[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) p[i] = partials[(size_t)(c + i) * M + row];
+#pragma unroll
+    for (int i = 0; i < 8; i++) s += p[i];
+  }
+  for (; c < stretches; c++) s += partials[(size_t)c * M + row];
+  gemv_update(y + row, s, alpha, beta);
+}
+
+// any M, K, lda, alignment: a thread per row, the threads of a wave read 128 contiguous bytes of a column
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemv_col_generic_kernel(const uint16_t *__restrict__ A, size_t lda, const uint16_t *__restrict__ x, OUT *__restrict__ y, size_t M, size_t K, float alpha,
+                                                               float beta) {
+  const size_t row = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= M) return;
+  float s = 0.0f;
+  for (size_t k = 0; k < K; k++) s = __builtin_fmaf((float)__builtin_bit_cast(half_t, A[k * lda + row]), (float)__builtin_bit_cast(half_t, x[k]), s);
+  gemv_update(y + row, s, alpha, beta);
+}
+
 }  // namespace tcu

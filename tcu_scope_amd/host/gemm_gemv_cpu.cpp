@@ -32,6 +32,11 @@ BENCHMARK(TCU_WAVE_HGEMV)->Apply(GemvArgs)->UseManualTime();
 BENCHMARK(CUDA_WMMA_GEMV_ACCURACY)->Apply(GemvArgs)->UseManualTime();
 BENCHMARK(CUDA_WMMA_GEMV_SHAREDMEM)->Apply(GemvArgs)->UseManualTime();
 BENCHMARK(TCU_WAVE_GEMV)->Apply(GemvArgs)->UseManualTime();
+// the same product with A in the reference's own layout (column-major, lda = M: src/gemv/wmma_naive.cu:33-36)
+static void TCU_COL_MAJOR_GEMV(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_AUTO, "TCU_COL_MAJOR_GEMV", false, true); }
+static void TCU_COL_MAJOR_HGEMV(benchmark::State &state) { harness::run_gemv(state, TCU_VARIANT_AUTO, "TCU_COL_MAJOR_HGEMV", true, true); }
+BENCHMARK(TCU_COL_MAJOR_GEMV)->Apply(GemvArgs)->UseManualTime();
+BENCHMARK(TCU_COL_MAJOR_HGEMV)->Apply(GemvArgs)->UseManualTime();
 
 // The reference's CPU verification loop as a benchmark: N = 2^20 in segments of 16 (seed 0),
 // one thread (as the reference wrote it) and all host threads.

@@ -484,12 +484,15 @@ void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, i
   });
 }
 
-void run_gemv(benchmark::State &state, int variant, const char *name, bool half_out) {
+void run_gemv(benchmark::State &state, int variant, const char *name, bool half_out, bool col_major) {
   guarded(state, [&] {
     const size_t M = state.range(0), K = state.range(1);
     const float alpha = 1.0f, beta = 0.0f;
     const size_t out_size = half_out ? 2 : 4;  // bytes per element of y
-    const auto gemv = half_out ? tcu_gemv_f16_f16 : tcu_gemv_f16_f32;
+    const auto gemv = [half_out, col_major](const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant, void *stream) {
+      if (col_major) return half_out ? tcu_gemv_col_major_f16_f16(A, M, x, y, M, K, alpha, beta, stream) : tcu_gemv_col_major_f16_f32(A, M, x, y, M, K, alpha, beta, stream);
+      return half_out ? tcu_gemv_f16_f16(A, x, y, M, K, alpha, beta, variant, stream) : tcu_gemv_f16_f32(A, x, y, M, K, alpha, beta, variant, stream);
+    };
     DeviceBuffer A(M * K * 2), x(K * 2), y(M * out_size);
     TCU_CHECK(tcu_generate_f16(A.get(), M * K, flags().seed, TCU_DIST_NORMAL, 0, nullptr));
     TCU_CHECK(tcu_generate_f16(x.get(), K, flags().seed + 1, TCU_DIST_NORMAL, 0, nullptr));
@@ -510,7 +513,7 @@ void run_gemv(benchmark::State &state, int variant, const char *name, bool half_
       }
       for (size_t m = 0; m < M; m++) {
         double s = 0;
-        for (size_t k = 0; k < K; k++) s += (double)half_to_float(hA[m * K + k]) * half_to_float(hx[k]);
+        for (size_t k = 0; k < K; k++) s += (double)half_to_float(hA[col_major ? k * M + m : m * K + k]) * half_to_float(hx[k]);
         if (std::fabs(hy[m] - s) > 1e-2 * std::max(std::fabs(s), std::sqrt((double)K))) throw std::runtime_error(std::string(name) + ": row " + std::to_string(m) + " differs from the fp64 dot product");
       }
     }

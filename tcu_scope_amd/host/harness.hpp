@@ -104,7 +104,8 @@ inline size_t single_pass_partition(size_t segment_size, int waves_per_block) {
 void run_full_reduce(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
 void run_full_scan(benchmark::State &state, int strategy, size_t segment_size, int waves_per_block, const char *name);
 // half_out: y (GEMV) or C and D (GEMM) in fp16, the reference's H* benchmarks
-void run_gemv(benchmark::State &state, int variant, const char *name, bool half_out = false);
+// col_major: A column-major with lda = M (tcu_gemv_col_major_*; `variant` is not used)
+void run_gemv(benchmark::State &state, int variant, const char *name, bool half_out = false, bool col_major = false);
 void run_gemm(benchmark::State &state, int variant, const char *name, bool half_out = false);
 // two computations of one product compared under the reference's agreement rule
 // (src/gemm/accuracy.cu:259-268, src/gemv/accuracy.cu:314-323); counters: errors, max_abs_diff, max_rel_diff

@@ -23,6 +23,12 @@ int emu_full_scan_f16(const void *in, void *out, size_t n, void *ws, size_t *ws_
   return tcu::full_scan_dispatch(in, out, n, ws, ws_bytes, strategy, seg, wpb, nullptr);
 }
 int emu_gemv_f16_f32(const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant) { return tcu::gemv_dispatch(A, x, y, M, K, alpha, beta, variant, nullptr); }
+int emu_gemv_col_major_f16_f32(const void *A, size_t lda, const void *x, void *y, size_t M, size_t K, float alpha, float beta) {
+  return tcu::gemv_col_major_dispatch<float>("tcu_gemv_col_major_f16_f32", A, lda, x, y, M, K, alpha, beta, nullptr);
+}
+int emu_gemv_col_major_f16_f16(const void *A, size_t lda, const void *x, void *y, size_t M, size_t K, float alpha, float beta) {
+  return tcu::gemv_col_major_dispatch<tcu::half_t>("tcu_gemv_col_major_f16_f16", A, lda, x, y, M, K, alpha, beta, nullptr);
+}
 int emu_gemv_f16_f16(const void *A, const void *x, void *y, size_t M, size_t K, float alpha, float beta, int variant) { return tcu::hgemv_dispatch(A, x, y, M, K, alpha, beta, variant, nullptr); }
 int emu_gemm_f16_f16(const void *A, const void *B, const void *C, void *D, size_t M, size_t N, size_t K, float alpha, float beta, int variant) {
   return tcu::hgemm_dispatch(A, B, C, D, M, N, K, alpha, beta, variant, nullptr);

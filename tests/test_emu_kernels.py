@@ -38,6 +38,8 @@ def emu():
     L.emu_gemv_f16_f32.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci]
     L.emu_gemm_f16_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
     L.emu_gemv_f16_f16.argtypes = [vp, vp, vp, sz, sz, cf, cf, ci]
+    L.emu_gemv_col_major_f16_f32.argtypes = [vp, sz, vp, vp, sz, sz, cf, cf]
+    L.emu_gemv_col_major_f16_f16.argtypes = [vp, sz, vp, vp, sz, sz, cf, cf]
     L.emu_gemm_f16_f16.argtypes = [vp, vp, vp, vp, sz, sz, sz, cf, cf, ci]
     L.emu_set_option.argtypes = [ctypes.c_char_p, ci]
     L.emu_seg_reduce_offsets_f16.argtypes = [vp, vp, sz, vp, vp, ci, sz]
@@ -360,6 +362,22 @@ def test_gemv_gemm_and_generator(emu, oracle):
             rc = emu.emu_gemv_f16_f16(Ai.ctypes.data, xi.ctypes.data, yh.ctypes.data, M, K, 1.5, -0.5, v)
             ref = oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0h.astype(np.float32))
             assert rc == 0 and oracle.check_f16(yh[:M], ref, K)[0] == 0, (M, K, v)
+    # A column-major with a leading dimension: 512-row slabs with a ragged last one, several stretches of K, and the
+    # scalar kernel (lda or K not a multiple of 8); the oracle's row-major product of the transposed copy is the reference
+    for M, K, lda in ((64, 512, 64), (1000, 264, 1008), (513, 8, 520), (1030, 328, 1032), (37, 24, 41), (5, 7, 5)):
+        At = oracle.generate_f16(K * lda, 3, oracle.DIST_NORMAL).reshape(K, lda)  # row k = column k of A, lda - M values of padding
+        x = oracle.generate_f16(K, 4, oracle.DIST_NORMAL)
+        A = np.ascontiguousarray(At[:, :M].T).reshape(-1)
+        y0 = np.linspace(-1, 1, M).astype(np.float32)
+        Ati, xi = copy_in(At.reshape(-1)), copy_in(x)
+        y = copy_in(y0, np.float32)
+        assert emu.emu_gemv_col_major_f16_f32(Ati.ctypes.data, lda, xi.ctypes.data, y.ctypes.data, M, K, 1.5, -0.5) == 0, emu.emu_last_error()
+        assert oracle.check_f32_rel(y[:M], oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0), 1e-4, float(np.sqrt(K)))[0] == 0, (M, K, lda)
+        y0h = y0.astype(np.float16)
+        yh = copy_in(y0h.view(np.uint16))
+        assert emu.emu_gemv_col_major_f16_f16(Ati.ctypes.data, lda, xi.ctypes.data, yh.ctypes.data, M, K, 1.5, -0.5) == 0
+        assert oracle.check_f16(yh[:M], oracle.gemv_f64(A, x, M, K, 1.5, -0.5, y0h.astype(np.float32)), K)[0] == 0, (M, K, lda)
+    assert emu.emu_gemv_col_major_f16_f32(Ati.ctypes.data, 3, xi.ctypes.data, y.ctypes.data, 5, 7, 1.0, 0.0) == 1  # lda < M
     for M, N, K in ((128, 128, 64), (256, 512, 64), (128, 256, 96), (64, 32, 48), (33, 17, 20)):
         A, B = oracle.generate_f16(M * K, 5, oracle.DIST_SMALLINT), oracle.generate_f16(N * K, 6, oracle.DIST_SMALLINT)
         C0 = (np.arange(M * N) % 7).astype(np.float32)

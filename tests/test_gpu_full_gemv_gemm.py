@@ -213,6 +213,42 @@ def test_gemv(tcu, oracle, M, K):
             assert bad == 0, ("fp16 y", v.name, alpha, beta, bad, worst, first)
 
 
+@pytest.mark.parametrize("M,K,lda", [(4096, 4096, 4096), (1000, 264, 1008), (2051, 1160, 2056), (513, 8, 520), (37, 24, 41), (5, 7, 5), (16384, 16384, 16384)])
+def test_gemv_col_major(tcu, oracle, M, K, lda):
+    """tcu_gemv_col_major_f16_f32 / _f16 (A as the reference's kernels hold it: element (m, k) at A[m + k*lda]) against the
+    fp64 product (1e-4 at the scale sqrt(K), as for the row-major entry points), with rows of padding between the columns,
+    ragged last slabs, the scalar kernel (lda or K not a multiple of 8), and against tcu_gemv_f16_f32 on the transposed
+    copy; the same call twice gives the same bits (every sum is taken in a fixed order)."""
+    import torch
+
+    At = oracle.generate_f16(K * lda, 3, oracle.DIST_NORMAL).reshape(K, lda)
+    x = oracle.generate_f16(K, 4, oracle.DIST_NORMAL)
+    A = np.ascontiguousarray(At[:, :M].T).reshape(-1)
+    y0 = np.linspace(-1, 1, M).astype(np.float32)
+    Atd, xd = to_dev(At.reshape(-1)).view(K, lda)[:, :M], to_dev(x)
+    for alpha, beta in [(1.0, 0.0), (1.5, -0.5)]:
+        y = torch.from_numpy(y0.copy()).cuda()
+        tcu.gemv_col_major(Atd, xd, alpha, beta, y=y)
+        ref = oracle.gemv_f64(A, x, M, K, alpha, beta, y0)
+        bad, worst, first = oracle.check_f32_rel(y.cpu().numpy(), ref, 1e-4, float(np.sqrt(K)))
+        assert bad == 0, (alpha, beta, bad, worst, first)
+        again = torch.from_numpy(y0.copy()).cuda()
+        tcu.gemv_col_major(Atd, xd, alpha, beta, y=again)
+        assert torch.equal(again, y)
+        y0h = y0.astype(np.float16)
+        yh = torch.from_numpy(y0h.copy()).cuda()
+        tcu.gemv_col_major(Atd, xd, alpha, beta, y=yh)
+        ref = oracle.gemv_f64(A, x, M, K, alpha, beta, y0h.astype(np.float32))
+        bad, worst, first = oracle.check_f16(yh.cpu().numpy().view(np.uint16), ref, K, ulps=1.0, abs_per_sqrt=1e-4)
+        assert bad == 0, ("fp16 y", alpha, beta, bad, worst, first)
+    if K % 8 == 0:
+        row_major = tcu.gemv(to_dev(A).view(M, K), xd)
+        col_major = tcu.gemv_col_major(Atd, xd)
+        assert torch.allclose(row_major, col_major, rtol=0, atol=1e-4 * float(np.sqrt(K)))
+    with pytest.raises(ValueError):
+        tcu.gemv_col_major(Atd.t(), xd)  # columns not contiguous
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 256, 256), (512, 384, 160), (384, 640, 1088), (96, 64, 48), (33, 17, 20)])
 def test_gemm_small_exact_and_normal(tcu, oracle, M, N, K):
     import torch

@@ -72,7 +72,7 @@ def test_harness_runs_verifies_and_reports(tmp_path):
     filt = ("(CUDA_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16<1, 4>|256<1, 4>|16N<4>|256N<4>|256N_BLOCK<4>)|CUB_(WARP|BLOCK)_SEGMENTED_(REDUCTION|PREFIXSUM)<(256, 16|512, 32, BLOCK_(SCAN|REDUCE)_RAKING)>"
             "|TCU_AUTO_SEGMENTED_(REDUCTION|PREFIXSUM))/.*num_elements:4194304/"
             "|CUDA_WMMA_FULL_(REDUCTION_(2KERS_BASE_16|ATOMIC_W_BLOCK_SYNC)|PREFIXSUM_(3KERS|CG))<8 \\* 256, 4>/num_elements:4194304/"
-            "|CUDA_WMMA_H?GEM[MV](_NAIVE)?/M:512/|TCU_WAVE_H?GEMV/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/"
+            "|CUDA_WMMA_H?GEM[MV](_NAIVE)?/M:512/|TCU_(WAVE|COL_MAJOR)_H?GEMV/M:512/|CPU_SEQUENTIAL_SEGMENTED_REDUCTION/num_segments:65536/"
             "|CUDA_UNSAFE_WMMA_SEGMENTED_(REDUCTION|PREFIXSUM)_(16N<4>|256N_BLOCK<4>)/.*num_elements:4194304/"
             "|CUB_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/|CUB_DEVICE_SEGMENTED_REDUCTION/.*segment_size:256/num_elements:4194304/|CUBLAS_(WMMA_H?GEMM|GEMV)/M:512/|HIPBLASLT_H?GEMM/M:512/"
             "|(THRUST|TCU_BY_KEY)_SEGMENTED_(REDUCTION|PREFIXSUM)/.*segment_size:(16|2048)/num_elements:4194304/|THRUST_FULL_(REDUCTION|PREFIXSUM)/num_elements:4194304/")
@@ -82,7 +82,7 @@ def test_harness_runs_verifies_and_reports(tmp_path):
     assert "ERROR OCCURRED" not in p.stdout, p.stdout
     data = json.loads(out.read_text())
     rows = data["benchmarks"]
-    assert len(rows) >= 52
+    assert len(rows) >= 54
     for r in rows:
         assert r["iterations"] >= 1 and r["real_time"] > 0 and r["flops"] > 0, r
         assert r["name"].endswith("/manual_time")
