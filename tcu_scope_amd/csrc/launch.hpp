@@ -51,6 +51,25 @@ inline std::atomic<unsigned long> &stream_alloc_count() {
   static std::atomic<unsigned long> n{0};
   return n;
 }
+// A block that a stream gives back is kept for that stream's next request (up to kSpareBlocks blocks per process):
+// work enqueued on one stream runs in order, so the next user of the block on the same stream cannot overtake the
+// last one, and the pool's two calls (about 10 us of host time per request, which a caller that waits for every
+// call sees in full) are skipped.  A request the spare does not satisfy goes to the pool; a returned block that
+// finds no room goes back to it.
+struct StreamBlocks {
+  static constexpr int kSpareBlocks = 8, kOutstanding = 64;
+  struct Block {
+    void *p = nullptr, *stream = nullptr;
+    size_t bytes = 0;
+    int dev = 0;
+  };
+  std::mutex mutex;
+  Block spare[kSpareBlocks], out[kOutstanding];
+};
+inline StreamBlocks &stream_blocks() {
+  static StreamBlocks b;
+  return b;
+}
 inline void *stream_alloc(size_t bytes, void *stream) {
   stream_alloc_count()++;
   constexpr int kMaxDevices = 64;
@@ -68,6 +87,23 @@ inline void *stream_alloc(size_t bytes, void *stream) {
     return nullptr;
   }
   if (dev < 0 || dev >= kMaxDevices) return nullptr;
+  if (bytes == 0) bytes = 1;
+  StreamBlocks &sb = stream_blocks();
+  {
+    std::lock_guard<std::mutex> lock(sb.mutex);
+    for (auto &s : sb.spare) {
+      if (s.p && s.stream == stream && s.dev == dev && s.bytes >= bytes) {
+        for (auto &o : sb.out) {
+          if (!o.p) {  // remembered so that stream_free knows its size; no room to remember: the pool serves the request
+            o = s;
+            s = StreamBlocks::Block{};
+            return o.p;
+          }
+        }
+        break;
+      }
+    }
+  }
   std::lock_guard<std::mutex> lock(pools_mutex);
   if (!pools[dev]) {
     hipMemPoolProps props = {};
@@ -89,9 +125,56 @@ inline void *stream_alloc(size_t bytes, void *stream) {
     (void)hipGetLastError();  // the caller reports the failure or does without; a later launch check must not see it
     return nullptr;
   }
+  std::lock_guard<std::mutex> lock2(sb.mutex);
+  for (auto &o : sb.out) {
+    if (!o.p) {
+      o.p = p;
+      o.stream = stream;
+      o.bytes = bytes;
+      o.dev = dev;
+      break;
+    }
+  }
   return p;
 }
-inline void stream_free(void *p, void *stream) { (void)hipFreeAsync(p, static_cast<hipStream_t>(stream)); }
+inline void stream_free(void *p, void *stream) {
+  if (!p) return;
+  StreamBlocks &sb = stream_blocks();
+  void *evicted = nullptr, *evicted_stream = nullptr;
+  bool kept = false;
+  {
+    std::lock_guard<std::mutex> lock(sb.mutex);
+    for (auto &o : sb.out) {
+      if (o.p != p) continue;
+      StreamBlocks::Block b = o;
+      o = StreamBlocks::Block{};
+      if (b.stream != stream) break;  // given back on another stream than it was taken on: the pool orders that
+      // this stream's spare, else a free place, else the place of the smallest block if that is smaller
+      StreamBlocks::Block *at = nullptr;
+      for (auto &s : sb.spare)
+        if (s.p && s.stream == stream && s.dev == b.dev) at = &s;
+      if (!at)
+        for (auto &s : sb.spare)
+          if (!s.p && !at) at = &s;
+      if (!at) {
+        at = &sb.spare[0];
+        for (auto &s : sb.spare)
+          if (s.bytes < at->bytes) at = &s;
+      }
+      if (at->p && at->bytes >= b.bytes) break;  // what is kept is at least as large
+      evicted = at->p;
+      evicted_stream = at->stream;
+      *at = b;
+      kept = true;
+      break;
+    }
+  }
+  if (evicted) {
+    if (evicted_stream == stream) (void)hipFreeAsync(evicted, static_cast<hipStream_t>(stream));
+    else (void)hipFree(evicted);  // that stream may be gone by now: not in its order, but after all work on the device
+  }
+  if (!kept) (void)hipFreeAsync(p, static_cast<hipStream_t>(stream));
+}
 
 }  // namespace tcu
 #endif  // TCU_LAUNCH_HPP
