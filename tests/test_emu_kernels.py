@@ -364,7 +364,7 @@ def test_gemv_gemm_and_generator(emu, oracle):
             assert rc == 0 and oracle.check_f16(yh[:M], ref, K)[0] == 0, (M, K, v)
     # A column-major with a leading dimension: 512-row slabs with a ragged last one, several stretches of K, and the
     # scalar kernel (lda or K not a multiple of 8); the oracle's row-major product of the transposed copy is the reference
-    for M, K, lda in ((64, 512, 64), (1000, 264, 1008), (513, 8, 520), (1030, 328, 1032), (37, 24, 41), (5, 7, 5)):
+    for M, K, lda in ((64, 512, 64), (520, 136, 528), (513, 8, 520), (37, 24, 41), (5, 7, 5)):
         At = oracle.generate_f16(K * lda, 3, oracle.DIST_NORMAL).reshape(K, lda)  # row k = column k of A, lda - M values of padding
         x = oracle.generate_f16(K, 4, oracle.DIST_NORMAL)
         A = np.ascontiguousarray(At[:, :M].T).reshape(-1)
@@ -486,7 +486,7 @@ def test_segments_given_by_keys(emu, oracle, bits):
     kt = np.int32 if bits == 32 else np.int64
     rng = np.random.default_rng(bits)
     part = 4 * 16 * 512
-    for n, mean_run in ((1, 1), (7, 2), (513, 1), (part - 3, 40), (part + 1, 5000), (3 * part + 77, 3), (3 * part + 77, 300), (2 * part, 10 ** 9)):
+    for n, mean_run in ((1, 1), (7, 2), (513, 1), (part - 3, 40), (part + 1, 5000), (2 * part + 77, 3), (2 * part + 77, 300), (2 * part, 10 ** 9)):
         keys = run_keys(rng, n, mean_run)
         if bits == 32:
             keys = keys % (1 << 20)
