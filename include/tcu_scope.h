@@ -232,7 +232,7 @@ int tcu_gemv_f16_f32(const void *d_A, const void *d_x, void *d_y, size_t M, size
  * the reference's own kernels and its cuBLAS baseline take A (src/gemv/wmma_naive.cu:33-36, 61: lda = M_GLOBAL,
  * fragments loaded col_major), so a caller that holds the reference's buffers passes them as they are.  y: M values of
  * fp32 (_f32) or fp16 (_f16).  Columns are read 1 KiB at a time and scaled by x[k]; the sums of stretches of K meet in
- * M floats per stretch of stream-ordered temporary memory (up to 64 stretches) and are added in a fixed order.  K a
+ * M floats per stretch of stream-ordered temporary memory (about 1024 / (M / 512) stretches) and are added in a fixed order.  K a
  * multiple of 8, lda a multiple of 8 and 16-byte aligned A and x take the fast kernels, anything else a scalar one. */
 int tcu_gemv_col_major_f16_f32(const void *d_A, size_t lda, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, void *stream);
 int tcu_gemv_col_major_f16_f16(const void *d_A, size_t lda, const void *d_x, void *d_y, size_t M, size_t K, float alpha, float beta, void *stream);

@@ -32,7 +32,8 @@ extern "C" {
  *   "by_key_waves"    waves per block of the two large launches of tcu_seg_reduce_by_key_f16 (1 .. 16; 0 = default 1)
  *   "by_key_key_tiles" KiB of keys a wave of its first launch has in flight: 4, 8 or 16 (0 = default 16)
  *   "scan_lds_tiles"  0/1, default 1: full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves)
- *   "gemv_col_shape"  column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2); default 42
+ *   "gemv_col_shape"  column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2); default 82
+ *   "gemv_col_blocks" column-major GEMV: about this many blocks (slabs of 512 rows x stretches of K); default 1024
  *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step
  *                     (1/2/4/8) and waves per block of the block GEMV kernel (rows of 8 KiB and more);
  *                     "gemv_waves" also sets the waves that split K in the strip kernels (TCU_VARIANT_MFMA_16N)

@@ -43,7 +43,8 @@ struct Options {
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
   bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
-  int gemv_col_shape = 42;     // column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2)
+  int gemv_col_blocks = 1024;  // column-major GEMV: about this many blocks (slabs of 512 rows x stretches of K)
+  int gemv_col_shape = 82;     // column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2)
   bool gemv_strip_lds = true;  // strip GEMV (TCU_VARIANT_MFMA_16N): stage the strip through LDS where K is a multiple of 512
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
   int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
@@ -74,6 +75,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_rows") o.gemv_rows = value;
   else if (n == "gemv_tiles") o.gemv_tiles = value;
   else if (n == "gemv_waves") o.gemv_waves = value;
+  else if (n == "gemv_col_blocks") o.gemv_col_blocks = value < 1 ? 1 : value;
   else if (n == "gemv_col_shape") o.gemv_col_shape = value;
   else if (n == "gemv_strip_lds") o.gemv_strip_lds = value != 0;
   else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
@@ -1179,13 +1181,13 @@ inline int gemv_col_major_dispatch(const char *what, const void *A, size_t lda, 
     launch(gemv_col_generic_kernel<OUT>, (unsigned)grid, 256u, stream, a, lda, static_cast<const uint16_t *>(x), yy, M, K, alpha, beta);
     return TCU_OK;
   }
-  // slabs of 512 rows; K is cut into stretches so that about 2048 blocks run and a wave still takes two rounds or more
-  // (16384 x 16384: 32 slabs x 64 stretches of 256 columns)
+  // slabs of 512 rows; K is cut into stretches so that about 1024 blocks of 8 waves run and a wave still takes two rounds or
+  // more (16384 x 16384: 32 slabs x 32 stretches of 512 columns; 1024 ... 8192 blocks of 4 or 8 waves: 88-106 us)
   const int shape = options().gemv_col_shape;  // waves per block * 10 + groups of 8 columns per wave and round
   const unsigned waves = shape / 10 == 8 ? 8u : 4u, groups = shape % 10 == 1 ? 1u : 2u;
   const size_t round = (size_t)8 * groups * waves;  // columns per round of a block
   const size_t slabs = (M + kColSlabRows - 1) / kColSlabRows;
-  size_t stretches = (2048 + slabs - 1) / slabs;
+  size_t stretches = ((size_t)options().gemv_col_blocks + slabs - 1) / slabs;
   const size_t most = (K + 2 * round - 1) / (2 * round);
   if (stretches > most) stretches = most;
   if (stretches < 1) stretches = 1;
