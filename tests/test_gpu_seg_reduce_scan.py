@@ -479,6 +479,31 @@ def test_offsets_one_segment_beyond_2_to_the_31(tcu, oracle):
     assert torch.equal(sums.view(torch.int16), want.view(torch.int16))
 
 
+def test_temporary_memory_across_streams(tcu, oracle):
+    """The paths that take temporary device memory keep the block a stream gave back for that stream's next request:
+    twelve streams (more than the library keeps blocks for), growing and shrinking requests on one stream, and calls
+    that alternate between streams must all give the results of the default stream."""
+    import torch
+
+    seg = 1 << 20
+    g = oracle.generate_f16(8 * seg, 31, oracle.DIST_GRID)
+    gd = to_dev(g)
+    want = {k: oracle.seg_reduce_f64(g[:k * seg], k, seg).astype(np.float16).view(np.uint16) for k in (1, 2, 4, 8)}
+    streams = [torch.cuda.Stream() for _ in range(12)]
+    torch.cuda.synchronize()
+    outs = []
+    for rep in range(3):
+        for i, st in enumerate(streams):
+            k = (1, 4, 2, 8)[(i + rep) % 4]  # the same stream asks for more, then for less
+            with torch.cuda.stream(st):
+                outs.append((k, tcu.seg_reduce(gd[:k * seg], seg, stream=st)))
+    for k in (8, 1, 4):
+        outs.append((k, tcu.seg_reduce(gd[:k * seg], seg)))
+    torch.cuda.synchronize()
+    for k, out in outs:
+        assert np.array_equal(to_host(out), want[k]), k
+
+
 def test_time_next_launch(tcu):
     """tcu_time_next_launch: the events are stamped by the kernel itself, only the next launch carries them, and the
     duration lies between what the bytes need at 8 TB/s and the wall-clock time of the call."""
