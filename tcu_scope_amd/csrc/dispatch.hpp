@@ -41,7 +41,7 @@ struct Options {
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
   bool gemm_staged_epilogue = true;   // 16x16x32 big-tile kernel: turn the outputs through LDS so that rows are written whole (C and D 16-byte aligned)
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
-  bool scan_lds_tiles = true;  // full scan AUTO: park 4 extra tiles per wave in LDS
+  int scan_lds_tiles = -1;     // full scan AUTO: park 4 extra tiles per wave in LDS: 1 always, 0 never, -1 where it measures faster (around 2^28 elements)
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
   int gemv_col_blocks = 1024;  // column-major GEMV: about this many blocks (slabs of 512 rows x stretches of K)
   int gemv_col_shape = 82;     // column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2)
@@ -78,7 +78,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemv_col_blocks") o.gemv_col_blocks = value < 1 ? 1 : value;
   else if (n == "gemv_col_shape") o.gemv_col_shape = value;
   else if (n == "gemv_strip_lds") o.gemv_strip_lds = value != 0;
-  else if (n == "scan_lds_tiles") o.scan_lds_tiles = value != 0;
+  else if (n == "scan_lds_tiles") o.scan_lds_tiles = value < 0 ? -1 : (value != 0);
   else if (n == "gemm_bk64") o.gemm_bk64 = value != 0;
   else if (n == "offsets_scan_chain") o.offsets_scan_chain = value != 0;
   else if (n == "by_key_reduce_chain") o.by_key_reduce_chain = value != 0;
@@ -898,8 +898,10 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
   const bool mfma = (strategy & TCU_FULL_MFMA) != 0;
   strategy &= ~TCU_FULL_MFMA;
   if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
-  // AUTO with the default partition: the kernel that parks 4 more tiles per wave in LDS
-  const bool lds_held = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && options().scan_lds_tiles && !mfma;
+  // AUTO with the default partition: the kernel that parks 4 more tiles per wave in LDS: 193 against 201 us at 2^28 elements, but 390 against 383 at 2^29, 760 against 744 at 2^30
+  // and 64.5 against 62.3 at 2^26, so only around 2^28
+  const bool lds_pays = options().scan_lds_tiles < 0 ? n > ((size_t)1 << 27) && n < ((size_t)1 << 29) : options().scan_lds_tiles != 0;
+  const bool lds_held = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && lds_pays && !mfma;
   if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
   const bool nt = options().nontemporal;
   if (strategy == TCU_FULL_SINGLE_PASS) {

@@ -71,7 +71,7 @@ def test_argument_validation_needs_no_gpu(lib):
     for name in (b"static_order", b"scan_lds_tiles", b"gemm_big_tiles", b"gemm_direct_lds", b"gemm_bk64", b"gemm_staged_epilogue", b"gemm_depth", b"gemm_split_tail", b"compute_units", b"gemv_rows", b"gemv_tiles", b"gemv_waves", b"lookback_poll_limit",
                  b"test_mute_partition", b"scan_store_policy", b"by_key_reduce_chain", b"by_key_waves", b"by_key_key_tiles", b"offsets_scan_chain", b"gemv_col_shape", b"gemv_col_blocks"):
         assert lib.tcu_set_option(name, 0) == 0  # every switch the header documents exists
-    for name, default in ((b"scan_lds_tiles", 1), (b"gemm_big_tiles", -1), (b"gemm_direct_lds", -1), (b"gemm_depth", 4), (b"gemm_staged_epilogue", 1), (b"gemm_split_tail", 1), (b"compute_units", 256), (b"lookback_poll_limit", -1), (b"scan_store_policy", 2), (b"offsets_scan_chain", 1), (b"gemv_col_shape", 82), (b"gemv_col_blocks", 1024), (b"xcd_run", 7),
+    for name, default in ((b"scan_lds_tiles", -1), (b"gemm_big_tiles", -1), (b"gemm_direct_lds", -1), (b"gemm_depth", 4), (b"gemm_staged_epilogue", 1), (b"gemm_split_tail", 1), (b"compute_units", 256), (b"lookback_poll_limit", -1), (b"scan_store_policy", 2), (b"offsets_scan_chain", 1), (b"gemv_col_shape", 82), (b"gemv_col_blocks", 1024), (b"xcd_run", 7),
                           (b"xcd_run", -1)):
         assert lib.tcu_set_option(name, default) == 0
     assert lib.tcu_set_option(b"no_such_option", 1) == 1

@@ -260,7 +260,10 @@ def test_full_array_kernels(emu, oracle):
         w64 = oracle.seg_scan_f64(x, 1, n)
         xi = copy_in(x)
         # 0x100 = TCU_FULL_MFMA: the single-pass kernels on the matrix unit
-        for strategy, seg, wpb in ((0, 0, 0), (1, 2048, 4), (1, 1024, 1), (2, 0, 0), (2, 256, 2), (0x100, 0, 0), (0x101, 2048, 4), (0x101, 512, 1)):
+        # -1 as the first entry's last field: AUTO with 4 more tiles per wave parked in LDS, which the library itself only takes around 2^28 elements
+        for strategy, seg, wpb in ((0, 0, -1), (0, 0, 0), (1, 2048, 4), (1, 1024, 1), (2, 0, 0), (2, 256, 2), (0x100, 0, 0), (0x101, 2048, 4), (0x101, 512, 1)):
+            emu.emu_set_option(b"scan_lds_tiles", 1 if wpb < 0 else -1)
+            wpb = max(wpb, 0)
             for op, fn in (("reduce", emu.emu_full_reduce_f16), ("scan", emu.emu_full_scan_f16)):
                 need = sz(0)
                 rc = fn(xi.ctypes.data, None, n, None, ctypes.byref(need), strategy, seg, wpb)

@@ -32,6 +32,12 @@ def test_full_reduce_and_scan(tcu, oracle, n):
             continue
         expect_ok(oracle, red, ref[-1:], n, f"full reduce n={n} strategy={int(strategy):#x} seg={seg}")
         expect_ok(oracle, sc, ref, n, f"full scan n={n} strategy={int(strategy):#x} seg={seg}")
+    # AUTO with 4 more tiles per wave parked in LDS, which the library itself only takes around 2^28 elements
+    try:
+        tcu.set_option("scan_lds_tiles", 1)
+        expect_ok(oracle, to_host(tcu.full_scan(xd)), ref, n, f"full scan n={n} with tiles parked in LDS")
+    finally:
+        tcu.set_option("scan_lds_tiles", -1)
 
 
 def test_full_exact_grid_bitwise_and_repeatable(tcu, oracle):
@@ -112,6 +118,7 @@ def test_a_wait_that_expires_gives_nan_not_wrong_numbers(tcu, oracle):
         tcu.set_option("test_mute_partition", mute)
         # (strategy, segment_size, waves) -> halves per partition
         for strategy, seg, w, part in [(S.SINGLE_PASS, 0, 0, 65536), (S.SINGLE_PASS, 8192, 4, 8192), (S.AUTO, 0, 0, 98304), (S.SINGLE_PASS | tcu.FULL_MFMA, 0, 0, 65536)]:
+            tcu.set_option("scan_lds_tiles", 1 if part == 98304 else -1)  # AUTO with tiles parked in LDS: forced, the library takes it around 2^28 elements only
             ws = torch.zeros(tcu.binding.full_workspace_bytes("scan", n, strategy, seg, w) // 4, dtype=torch.int32, device="cuda")
             got = to_host(tcu.full_scan(xd, strategy, seg, w, workspace=ws))
             # word 1 of the workspace counts the waits that gave up: the partition behind the silent one for certain,
@@ -137,6 +144,7 @@ def test_a_wait_that_expires_gives_nan_not_wrong_numbers(tcu, oracle):
         expect_ok(oracle, th[1:], refs[-1:], seg, "segmented look-back scan: total of the other segment")
     finally:
         tcu.set_option("test_mute_partition", 0)
+        tcu.set_option("scan_lds_tiles", -1)
         tcu.set_option("lookback_poll_limit", -1)
     # and with the defaults restored the same calls are right again
     ws = torch.ones(tcu.binding.full_workspace_bytes("scan", n, S.SINGLE_PASS) // 4, dtype=torch.int32, device="cuda")
