@@ -1320,7 +1320,17 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
     // the transfer kernel with 128 x 128 tiles (two blocks per compute unit) unless the register-staged
     // kernel is asked for (gemm_direct_lds = 0) or K is beyond the 32-bit lane offsets
     if (options().gemm_direct_lds != 0 && K <= ((size_t)1 << 22)) {
-      if (K % 64 == 0)
+      // K a multiple of 64 and outputs aligned to four: the three-A-two-B-buffer loop on 16x16x32 MFMAs with the
+      // epilogue through LDS, as for the big tiles (gemm_direct_lds = 64 keeps the 32x32x16 kernel selectable)
+      const bool al4 = ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & (4 * sizeof(OUT) - 1)) == 0;
+      const int direct_lds = options().gemm_direct_lds;
+      if ((direct_lds < 0 || direct_lds == 66) && K % 64 == 0 && al4) {
+        const bool staged = options().gemm_staged_epilogue && ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & 15u) == 0;
+        if (staged)
+          launch(gemm_dlds_a3b2_m16_t128_kernel<OUT, true>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+        else
+          launch(gemm_dlds_a3b2_m16_t128_kernel<OUT, false>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      } else if (K % 64 == 0)
         launch(gemm_dlds_kernel<64, 2, OUT, 128>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
       else
         launch(gemm_dlds_kernel<32, 4, OUT, 128>, (unsigned)grid, 256u, stream, a, b, c, d, M, N, K, alpha, beta);

@@ -674,25 +674,25 @@ __global__ __launch_bounds__(256) void gemm_dlds_a3b2_kernel(const half8_t *__re
 // row (lane & 15) and the four adjacent columns 4 * (lane >> 4) .. + 3 of every tile, i.e. one
 // 128-bit (fp32) or 64-bit (fp16) access per tile.  CRow16 holds a lane's C values of one row
 // of eight tiles.
-template <typename OUT>
+template <typename OUT, int W8>
 struct CRow16 {
   using word_t = typename std::conditional<sizeof(OUT) == 4, float4_t, uint2_t>::type;
-  word_t v[8];
+  word_t v[W8];
 };
-template <typename OUT>
-TCU_DEVICE void gemm_load_c_row16(CRow16<OUT> &c, const OUT *C, size_t ldc, size_t row0, size_t col0, int lane) {
-  using word_t = typename CRow16<OUT>::word_t;
+template <typename OUT, int W8>
+TCU_DEVICE void gemm_load_c_row16(CRow16<OUT, W8> &c, const OUT *C, size_t ldc, size_t row0, size_t col0, int lane) {
+  using word_t = typename CRow16<OUT, W8>::word_t;
   const word_t *p = reinterpret_cast<const word_t *>(C + (row0 + (lane & 15)) * ldc + col0 + 4 * (lane >> 4));
 #pragma unroll
-  for (int j = 0; j < 8; j++) c.v[j] = __builtin_nontemporal_load(p + j * 4);
+  for (int j = 0; j < W8; j++) c.v[j] = __builtin_nontemporal_load(p + j * 4);
 }
-// D = alpha * acc + beta * c for one row of eight tiles; c is not read when beta == 0
-template <typename OUT>
-TCU_DEVICE void gemm_store_row16(OUT *D, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8], const CRow16<OUT> &c, int lane, float alpha, float beta) {
-  using word_t = typename CRow16<OUT>::word_t;
+// D = alpha * acc + beta * c for one row of W8 tiles; c is not read when beta == 0
+template <typename OUT, int W8>
+TCU_DEVICE void gemm_store_row16(OUT *D, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[W8], const CRow16<OUT, W8> &c, int lane, float alpha, float beta) {
+  using word_t = typename CRow16<OUT, W8>::word_t;
   word_t *p = reinterpret_cast<word_t *>(D + (row0 + (lane & 15)) * ldc + col0 + 4 * (lane >> 4));
 #pragma unroll
-  for (int j = 0; j < 8; j++) {
+  for (int j = 0; j < W8; j++) {
     float4_t r = alpha * acc[j];
     if constexpr (sizeof(OUT) == 4) {
       if (beta != 0.0f) r = gemm_axpby(alpha, acc[j], beta, c.v[j]);
@@ -710,33 +710,35 @@ TCU_DEVICE void gemm_store_row16(OUT *D, size_t ldc, size_t row0, size_t col0, c
     }
   }
 }
-// The whole strip: eight rows of tiles, each row's C values read just before its stores (C may
+// The whole strip: W8 rows of W8 tiles, each row's C values read just before its stores (C may
 // be the same buffer as D: a lane reads only elements it will itself write).  Reading one to
 // three rows ahead of the stores measured the same or up to 1 % slower (8192^3, same run).
-template <typename OUT>
-TCU_DEVICE void gemm_store_strip16(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8][8], int lane, float alpha, float beta) {
+template <typename OUT, int W8>
+TCU_DEVICE void gemm_store_strip16(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[W8][W8], int lane, float alpha, float beta) {
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    CRow16<OUT> c;
+  for (int i = 0; i < W8; i++) {
+    CRow16<OUT, W8> c;
     if (beta != 0.0f) gemm_load_c_row16(c, C, ldc, row0 + i * 16, col0, lane);
     gemm_store_row16(D, ldc, row0 + i * 16, col0, acc[i], c, lane, alpha, beta);
   }
 }
 
 // The same strip with every row of tiles turned through LDS first, so that global memory sees whole rows: a
-// row of eight tiles is 16 rows of 128 outputs; the lanes park alpha * acc in `stage` (two buffers of
-// kStageRowFloats * 16 floats per wave, rows padded by four floats), and read it back with consecutive lanes
-// along a row: 32 lanes x 4 fp32 outputs (512 bytes of one row, two rows per instruction) or 16 lanes x 8 fp16
-// outputs (256 bytes, four rows per instruction), where the direct form writes 64 / 32 bytes of 16 rows
-// per instruction.  C is read in the same shape, by the lane that writes the same elements of D.
-constexpr int kStageRowFloats = 128 + 4;
-constexpr int kStageWaveFloats = 2 * 16 * kStageRowFloats;
-template <typename OUT>
-TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[8][8], int lane, float alpha, float beta, float *stage) {
-  constexpr int PER_LANE = sizeof(OUT) == 4 ? 4 : 8;   // outputs per lane and access (16 bytes)
-  constexpr int LANES_PER_ROW = 128 / PER_LANE;        // 32 or 16
-  constexpr int ROWS_PER_ACCESS = 64 / LANES_PER_ROW;  // 2 or 4
-  constexpr int ACCESSES = 16 / ROWS_PER_ACCESS;       // per row of tiles: 8 or 4
+// row of W8 tiles is 16 rows of 16 * W8 outputs; the lanes park alpha * acc in `stage` (two buffers of
+// gemm_stage_row_floats(W8) * 16 floats per wave, rows padded by four floats), and read it back with consecutive
+// lanes along a row.  W8 = 8: 32 lanes x 4 fp32 outputs (512 bytes of one row, two rows per instruction) or 16 lanes
+// x 8 fp16 outputs (256 bytes, four rows per instruction); W8 = 4: 256 bytes of four rows or 128 bytes of eight;
+// the direct form writes 64 / 32 bytes of 16 rows per instruction.  C is read in the same shape, by the lane that
+// writes the same elements of D.
+constexpr int gemm_stage_row_floats(int w8) { return 16 * w8 + 4; }
+constexpr int gemm_stage_wave_floats(int w8) { return 2 * 16 * gemm_stage_row_floats(w8); }
+template <typename OUT, int W8>
+TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[W8][W8], int lane, float alpha, float beta, float *stage) {
+  constexpr int kStageRowFloats = gemm_stage_row_floats(W8);
+  constexpr int PER_LANE = sizeof(OUT) == 4 ? 4 : 8;       // outputs per lane and access (16 bytes)
+  constexpr int LANES_PER_ROW = 16 * W8 / PER_LANE;        // W8 = 8: 32 or 16; W8 = 4: 16 or 8
+  constexpr int ROWS_PER_ACCESS = 64 / LANES_PER_ROW;      // 2 or 4; 4 or 8
+  constexpr int ACCESSES = 16 / ROWS_PER_ACCESS;           // per row of tiles: 8 or 4; 4 or 2
   using word_t = typename std::conditional<sizeof(OUT) == 4, float4_t, uint4_t>::type;
   const int wr = lane & 15, wq = lane >> 4;  // accumulator layout: row, group of four columns
   const int rr = lane / LANES_PER_ROW, rc = (lane % LANES_PER_ROW) * PER_LANE;
@@ -749,14 +751,14 @@ TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size
     for (int t = 0; t < ACCESSES; t++) c[0][t] = __builtin_nontemporal_load(reinterpret_cast<const word_t *>(C + at0 + (size_t)(ROWS_PER_ACCESS * t) * ldc));
   }
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
+  for (int i = 0; i < W8; i++) {
     float *buf = stage + (i & 1) * (16 * kStageRowFloats);
-    if (beta != 0.0f && i + 1 < 8) {
+    if (beta != 0.0f && i + 1 < W8) {
 #pragma unroll
       for (int t = 0; t < ACCESSES; t++) c[(i + 1) & 1][t] = __builtin_nontemporal_load(reinterpret_cast<const word_t *>(C + at0 + (size_t)(16 * (i + 1) + ROWS_PER_ACCESS * t) * ldc));
     }
 #pragma unroll
-    for (int j = 0; j < 8; j++) *reinterpret_cast<float4_t *>(buf + wr * kStageRowFloats + 16 * j + 4 * wq) = alpha * acc[i][j];
+    for (int j = 0; j < W8; j++) *reinterpret_cast<float4_t *>(buf + wr * kStageRowFloats + 16 * j + 4 * wq) = alpha * acc[i][j];
     wave_lds_fence();
 #pragma unroll
     for (int t = 0; t < ACCESSES; t++) {
@@ -797,12 +799,18 @@ TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size
 // One tile (or, with share != nullptr, the K steps step0 .. step0 + steps - 1 of one tile, whose raw fp32
 // accumulators go to `share` as a 256 x 256 row-major tile).  May be called several times by a block:
 // every wave waits for its own transfers before it leaves, and nothing reads LDS after the last barrier.
-template <typename OUT, bool STAGED>
+// W8 = 8: the 256 x 256 block tile; W8 = 4: a 128 x 128 block tile (waves of 64 x 64 = 4 x 4 accumulators, 80 KiB of
+// LDS, two blocks per compute unit), for outputs too small to fill the chip with the big tiles.
+template <typename OUT, bool STAGED, int W8 = 8>
 TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t N, size_t K, size_t tile_m, size_t tile_n, size_t step0, size_t steps,
                                    float *share, float alpha, float beta) {
   constexpr int BK = 64, ROWH = BK, CPR = 8, RPT = 8, RS = 1, SUB = 2, NA = 3, NB = 2;
-  constexpr int OPH = kGemmBigBM * ROWH;     // halves per operand per stage
-  constexpr int TPW = kGemmBigBM / RPT / 4;  // transfer instructions per wave, operand and step (8)
+  constexpr int TILE = 32 * W8, WT = 16 * W8;  // block tile, wave tile
+  constexpr int NM = W8 * W8;                  // MFMAs per substep
+  constexpr int OPH = TILE * ROWH;             // halves per operand per stage
+  constexpr int TPW = TILE / RPT / 4;          // transfer instructions per wave, operand and step (8 or 4)
+  constexpr int TEVERY = NM / 2 / TPW;         // one transfer every so many MFMAs of a substep's second half
+  static_assert(W8 == 8 || W8 == 4, "fragment reads (one before every other MFMA) and transfers must fit a substep");
   __shared__ __attribute__((aligned(1024))) half_t lds_a[NA][OPH];
   __shared__ __attribute__((aligned(1024))) half_t lds_b[NB][OPH];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -816,18 +824,18 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
     goff[t] = (uint32_t)(((size_t)row * k_chunks + chunk) * 16);
   }
   constexpr lds_addr_t STAGE = OPH * 2, TBYTES = 1024, STEPB = BK * 2;
-  const char *ga = reinterpret_cast<const char *>(A + tile_m * kGemmBigBM * k_chunks) + step0 * STEPB;
-  const char *gb = reinterpret_cast<const char *>(B + tile_n * kGemmBigBN * k_chunks) + step0 * STEPB;
+  const char *ga = reinterpret_cast<const char *>(A + tile_m * TILE * k_chunks) + step0 * STEPB;
+  const char *gb = reinterpret_cast<const char *>(B + tile_n * TILE * k_chunks) + step0 * STEPB;
   const lds_addr_t ta = wave_uniform(lds_address_of(&lds_a[0][0]) + wave * TPW * TBYTES);
   const lds_addr_t tb = wave_uniform(lds_address_of(&lds_b[0][0]) + wave * TPW * TBYTES);
   auto issue_a = [&](size_t step, int buf, int t) { load_chunk_to_lds(ga + (step < steps ? step : steps - 1) * STEPB, goff[t], ta + buf * STAGE + t * TBYTES); };
   auto issue_b = [&](size_t step, int buf, int t) { load_chunk_to_lds(gb + (step < steps ? step : steps - 1) * STEPB, goff[t], tb + buf * STAGE + t * TBYTES); };
 
-  float4_t acc[8][8];
+  float4_t acc[W8][W8];
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+  for (int i = 0; i < W8; i++)
 #pragma unroll
-    for (int j = 0; j < 8; j++)
+    for (int j = 0; j < W8; j++)
 #pragma unroll
       for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
 
@@ -846,13 +854,13 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
   // fragment of row r, k chunk kc: slot kc ^ f(r); the lane supplies row (lane & 15) of a
   // 16-row tile and chunk (lane >> 4) of the substep's four; rows of a lane differ by multiples of 16
   const int frow = lane & 15, kq = lane >> 4, fsw = (frow >> RS) & (CPR - 1);
-  const int fa0 = (wm * 128 + frow) * ROWH, fb0 = (wn * 128 + frow) * ROWH;
+  const int fa0 = (wm * WT + frow) * ROWH, fb0 = (wn * WT + frow) * ROWH;
   int ko[SUB];
 #pragma unroll
   for (int kk = 0; kk < SUB; kk++) ko[kk] = ((4 * kk + kq) ^ fsw) * 8;
-  half8_t fa[2][8], fb[2][8];
+  half8_t fa[2][W8], fb[2][W8];
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
+  for (int i = 0; i < W8; i++) {
     fa[0][i] = *reinterpret_cast<const half8_t *>(&lds_a[0][fa0 + i * 16 * ROWH + ko[0]]);
     fb[0][i] = *reinterpret_cast<const half8_t *>(&lds_b[0][fb0 + i * 16 * ROWH + ko[0]]);
   }
@@ -860,18 +868,18 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
   for (size_t s = 0; s < steps; s++) {
     const int na = ca + 1 == NA ? 0 : ca + 1, nb = cb ^ 1;
     const int fill_a = ca == 0 ? NA - 1 : ca - 1;  // A buffer of step s - 1 = of step s + 2
-    // substep 0: MFMA t works on tile (t / 8, t % 8); fragment k of substep 1 (order: A0 B0..B7 A1..A7)
-    // is read before MFMA 2k
+    // substep 0: MFMA t works on tile (t / W8, t % W8); fragment k of substep 1 (order: A0 B0..B7 A1..A7 for
+    // W8 = 8) is read before MFMA 2k
 #pragma unroll
-    for (int t = 0; t < 64; t++) {
-      if (t < 32 && t % 2 == 0) {
+    for (int t = 0; t < NM; t++) {
+      if (t < 4 * W8 && t % 2 == 0) {
         const int k = t / 2;
         if (k == 0) fa[1][0] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + ko[1]]);
-        else if (k <= 8) fb[1][k - 1] = *reinterpret_cast<const half8_t *>(&lds_b[cb][fb0 + (k - 1) * 16 * ROWH + ko[1]]);
-        else fa[1][k - 8] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + (k - 8) * 16 * ROWH + ko[1]]);
+        else if (k <= W8) fb[1][k - 1] = *reinterpret_cast<const half8_t *>(&lds_b[cb][fb0 + (k - 1) * 16 * ROWH + ko[1]]);
+        else fa[1][k - W8] = *reinterpret_cast<const half8_t *>(&lds_a[ca][fa0 + (k - W8) * 16 * ROWH + ko[1]]);
       }
-      if (t >= 32 && t % 4 == 0) issue_a(s + 2, fill_a, (t - 32) / 4);  // A tile of step s + 2 under the second half
-      acc[t / 8][t % 8] = mfma_16x16x32(fb[0][t % 8], fa[0][t / 8], acc[t / 8][t % 8]);
+      if (t >= NM / 2 && (t - NM / 2) % TEVERY == 0) issue_a(s + 2, fill_a, (t - NM / 2) / TEVERY);  // A tile of step s + 2 under the second half
+      acc[t / W8][t % W8] = mfma_16x16x32(fb[0][t % W8], fa[0][t / W8], acc[t / W8][t % W8]);
       sched_fence();
     }
     // substep 1: own transfers of step s + 1 done (the A tile of step s + 2 may still fly), barrier,
@@ -881,37 +889,47 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
     block_barrier_lds_only();
     sched_fence();
 #pragma unroll
-    for (int t = 0; t < 64; t++) {
-      if (t < 32 && t % 2 == 0) {
+    for (int t = 0; t < NM; t++) {
+      if (t < 4 * W8 && t % 2 == 0) {
         const int k = t / 2;
         if (k == 0) fa[0][0] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + ko[0]]);
-        else if (k <= 8) fb[0][k - 1] = *reinterpret_cast<const half8_t *>(&lds_b[nb][fb0 + (k - 1) * 16 * ROWH + ko[0]]);
-        else fa[0][k - 8] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + (k - 8) * 16 * ROWH + ko[0]]);
+        else if (k <= W8) fb[0][k - 1] = *reinterpret_cast<const half8_t *>(&lds_b[nb][fb0 + (k - 1) * 16 * ROWH + ko[0]]);
+        else fa[0][k - W8] = *reinterpret_cast<const half8_t *>(&lds_a[na][fa0 + (k - W8) * 16 * ROWH + ko[0]]);
       }
-      if (t >= 32 && t % 4 == 0) issue_b(s + 2, cb, (t - 32) / 4);  // B tile of step s + 2 into the B buffer of step s
-      acc[t / 8][t % 8] = mfma_16x16x32(fb[1][t % 8], fa[1][t / 8], acc[t / 8][t % 8]);
+      if (t >= NM / 2 && (t - NM / 2) % TEVERY == 0) issue_b(s + 2, cb, (t - NM / 2) / TEVERY);  // B tile of step s + 2 into the B buffer of step s
+      acc[t / W8][t % W8] = mfma_16x16x32(fb[1][t % W8], fa[1][t / W8], acc[t / W8][t % W8]);
       sched_fence();
     }
     ca = na;
     cb = nb;
   }
   wait_vector_loads<0>();  // the re-reads past the last step must land before the block's LDS is released
+  constexpr int kStageWaveFloats = gemm_stage_wave_floats(W8);
   if (share != nullptr) {
-    if constexpr (STAGED) {  // raw accumulators, whole rows of the 256 x 256 share (it is 16-byte aligned)
+    if constexpr (STAGED) {  // raw accumulators, whole rows of the TILE x TILE share (it is 16-byte aligned)
       block_barrier_lds_only();
-      gemm_store_strip16_staged<float>(share, nullptr, kGemmBigBN, wm * 128, wn * 128, acc, lane, 1.0f, 0.0f, reinterpret_cast<float *>(&lds_a[0][0]) + wave * kStageWaveFloats);
+      gemm_store_strip16_staged<float>(share, nullptr, TILE, wm * WT, wn * WT, acc, lane, 1.0f, 0.0f, reinterpret_cast<float *>(&lds_a[0][0]) + wave * kStageWaveFloats);
       block_barrier_lds_only();  // the block's next piece of work starts its transfers only after every wave has read its outputs back
     } else {
-      gemm_store_strip16<float>(share, nullptr, kGemmBigBN, wm * 128, wn * 128, acc, lane, 1.0f, 0.0f);
+      gemm_store_strip16<float>(share, nullptr, TILE, wm * WT, wn * WT, acc, lane, 1.0f, 0.0f);
     }
   } else if constexpr (STAGED) {
     block_barrier_lds_only();  // the other waves have read their last fragments: the A buffers can hold outputs now
     static_assert(4 * kStageWaveFloats * sizeof(float) <= sizeof(lds_a), "staging area of four waves");
-    gemm_store_strip16_staged(D, C, N, tile_m * kGemmBigBM + wm * 128, tile_n * kGemmBigBN + wn * 128, acc, lane, alpha, beta, reinterpret_cast<float *>(&lds_a[0][0]) + wave * kStageWaveFloats);
+    gemm_store_strip16_staged(D, C, N, tile_m * TILE + wm * WT, tile_n * TILE + wn * WT, acc, lane, alpha, beta, reinterpret_cast<float *>(&lds_a[0][0]) + wave * kStageWaveFloats);
     block_barrier_lds_only();  // a block that goes on to another piece of work starts its transfers only after every wave has read its outputs back
   } else {
-    gemm_store_strip16(D, C, N, tile_m * kGemmBigBM + wm * 128, tile_n * kGemmBigBN + wn * 128, acc, lane, alpha, beta);
+    gemm_store_strip16(D, C, N, tile_m * TILE + wm * WT, tile_n * TILE + wn * WT, acc, lane, alpha, beta);
   }
+}
+
+// The same loop on 128 x 128 block tiles (M and N multiples of 128, K of 64, C and D aligned to four outputs): one tile
+// per block, two blocks per compute unit.
+template <typename OUT, bool STAGED>
+__global__ __launch_bounds__(256, 2) void gemm_dlds_a3b2_m16_t128_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+  size_t tile_m, tile_n;
+  gemm_tile_of_block(M / 128, N / 128, blockIdx.x, &tile_m, &tile_n);
+  gemm_a3b2_m16_tile<OUT, STAGED, 4>(A, B, C, D, N, K, tile_m, tile_n, 0, K / 64, static_cast<float *>(nullptr), alpha, beta);
 }
 
 // Blocks 0 .. full_tiles-1 take one tile each.  With T tiles on a chip that runs `units` blocks at a

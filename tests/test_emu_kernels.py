@@ -460,15 +460,24 @@ def test_gemv_gemm_and_generator(emu, oracle):
             rc = emu.emu_gemm_f16_f16(Asi.ctypes.data, Bsi.ctypes.data, Chs.ctypes.data, Dhs.ctypes.data, Ms, Ns, Ks, 0.5, 2.0, V_BLOCK)
             assert rc == 0 and np.array_equal(Dhs.reshape(Ms, Ns), refs.astype(np.float16).view(np.uint16)), ("split tail fp16", Ms, Ns, Ks)
         assert emu.emu_set_option(b"compute_units", 256) == 0 and emu.emu_set_option(b"gemm_split_tail", 1) == 0
-        # 128 x 128 tiles: the transfer kernel (K step 64 and 32) and the register-staged one
+        # 128 x 128 tiles: the 16x16x32 kernel (K a multiple of 64; outputs through LDS or straight from the accumulators,
+        # fp16 outputs in place), the 32x32x16 transfer kernel (K step 64 and 32) and the register-staged one
         assert emu.emu_set_option(b"gemm_big_tiles", 0) == 0
-        for direct_lds, Ks in ((-1, 192), (-1, 96), (0, 96)):
-            assert emu.emu_set_option(b"gemm_direct_lds", direct_lds) == 0
+        for direct_lds, Ks, staged in ((-1, 192, 1), (-1, 192, 0), (-1, 64, 1), (64, 192, 1), (-1, 96, 1), (0, 96, 1)):
+            assert emu.emu_set_option(b"gemm_direct_lds", direct_lds) == 0 and emu.emu_set_option(b"gemm_staged_epilogue", staged) == 0
             A2, B2 = oracle.generate_f16(M * Ks, 9, oracle.DIST_SMALLINT), oracle.generate_f16(N * Ks, 10, oracle.DIST_SMALLINT)
             A2i, B2i = copy_in(A2), copy_in(B2)
+            ref2 = oracle.gemm_f64(A2, B2, M, N, Ks, 1.5, 2.0, C0)
             D = aligned(M * N, np.float32, -777)
             rc = emu.emu_gemm_f16_f32(A2i.ctypes.data, B2i.ctypes.data, Ci.ctypes.data, D.ctypes.data, M, N, Ks, 1.5, 2.0, V_BLOCK)
-            assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A2, B2, M, N, Ks, 1.5, 2.0, C0)), (direct_lds, Ks)
+            assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), ref2), (direct_lds, Ks, staged)
+            if direct_lds == -1 and Ks % 64 == 0:
+                Dh = copy_in(C0.astype(np.float16).view(np.uint16))  # in place: C == D
+                rc = emu.emu_gemm_f16_f16(A2i.ctypes.data, B2i.ctypes.data, Dh.ctypes.data, Dh.ctypes.data, M, N, Ks, 1.5, 2.0, V_BLOCK)
+                assert rc == 0 and np.array_equal(Dh.reshape(M, N), ref2.astype(np.float16).view(np.uint16)), ("fp16", Ks, staged)
+                D = aligned(M * N, np.float32, -777)  # beta = 0: C is not read
+                rc = emu.emu_gemm_f16_f32(A2i.ctypes.data, B2i.ctypes.data, None, D.ctypes.data, M, N, Ks, 1.5, 0.0, V_BLOCK)
+                assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A2, B2, M, N, Ks, 1.5, 0.0, C0)), ("beta 0", Ks, staged)
     finally:
         for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1), (b"compute_units", 256), (b"gemm_split_tail", 1), (b"gemm_staged_epilogue", 1)):
             emu.emu_set_option(name, val)

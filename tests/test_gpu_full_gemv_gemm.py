@@ -376,11 +376,13 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             ref = oracle.gemm_f64(A, B, Ms, Ns, Ks, 0.5, -1.0, Cs, row0=tm * 256 + 37, rows=4)
             assert np.array_equal(got[1][0][tm * 256 + 37:tm * 256 + 41].astype(np.float64), ref), ("split tail", tm)
             assert np.array_equal(got[1][1][tm * 256 + 37:tm * 256 + 41], ref.astype(np.float16).view(np.uint16)), ("split tail fp16", tm)
-        # 128 x 128 tiles: the transfer kernel (K step 64 and 32) and the register-staged one
+        # 128 x 128 tiles: the 16x16x32 kernel (K a multiple of 64; outputs through LDS and straight from the accumulators),
+        # the 32x32x16 transfer kernel (K step 64 and 32) and the register-staged one
         tcu.set_option("gemm_big_tiles", 0)
         tcu.set_option("gemm_bk64", 0)
-        for direct_lds, K in ((-1, 64), (-1, 448), (-1, 224), (0, 224)):
+        for direct_lds, K, staged in ((-1, 64, 1), (-1, 448, 1), (-1, 448, 0), (64, 448, 1), (-1, 224, 1), (0, 224, 1)):
             tcu.set_option("gemm_direct_lds", direct_lds)
+            tcu.set_option("gemm_staged_epilogue", staged)
             A = oracle.generate_f16(M * K, 21, oracle.DIST_SMALLINT)
             B = oracle.generate_f16(N * K, 22, oracle.DIST_SMALLINT)
             Ad, Bd = to_dev(A).view(M, K), to_dev(B).view(N, K)
@@ -388,8 +390,13 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd, variant=tcu.Variant.BLOCK_LDS)
             Dh = tcu.gemm(Ad, Bd, 1.0, 0.0, variant=tcu.Variant.BLOCK_LDS, out_dtype=torch.float16)
             torch.cuda.synchronize()
-            assert np.array_equal(Cd.cpu().numpy().astype(np.float64), oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)), ("128 tiles", direct_lds, K)
-            assert np.array_equal(Dh.cpu().numpy().view(np.uint16), oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0).astype(np.float16).view(np.uint16)), ("128 tiles fp16", direct_lds, K)
+            Ch = torch.from_numpy(C0.astype(np.float16)).cuda().view(M, N)
+            tcu.gemm(Ad, Bd, 2.0, -1.0, C=Ch, out=Ch, variant=tcu.Variant.BLOCK_LDS)  # fp16 in place
+            torch.cuda.synchronize()
+            ref1 = oracle.gemm_f64(A, B, M, N, K, 2.0, -1.0, C0)
+            assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("128 tiles", direct_lds, K, staged)
+            assert np.array_equal(Dh.cpu().numpy().view(np.uint16), oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0).astype(np.float16).view(np.uint16)), ("128 tiles fp16", direct_lds, K, staged)
+            assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("128 tiles fp16 in place", direct_lds, K, staged)
     finally:
         tcu.set_option("gemm_split_tail", 1)
         tcu.set_option("gemm_staged_epilogue", 1)
@@ -419,8 +426,15 @@ def test_gemm_kernels_round_alike(tcu):
             for name, variant, staged in (("direct kernel", tcu.Variant.MFMA_16N, 1), ("tiled, through LDS", tcu.Variant.AUTO, 1), ("tiled, from the accumulators", tcu.Variant.AUTO, 0)):
                 tcu.set_option("gemm_staged_epilogue", staged)
                 got[name] = tcu.gemm(A, B, 1.1, 1.2, C=C, variant=variant).view(bits)
+            # the same loop on 128 x 128 block tiles adds a given output's products in the same order
+            tcu.set_option("gemm_big_tiles", 0)
+            for staged in (1, 0):
+                tcu.set_option("gemm_staged_epilogue", staged)
+                got["128 tiles", staged] = tcu.gemm(A, B, 1.1, 1.2, C=C).view(bits)
+            tcu.set_option("gemm_big_tiles", 1)
             torch.cuda.synchronize()
             assert torch.equal(got["tiled, through LDS"], got["tiled, from the accumulators"]), dt
+            assert torch.equal(got["tiled, through LDS"], got["128 tiles", 1]) and torch.equal(got["tiled, through LDS"], got["128 tiles", 0]), dt
             if dt == torch.float32:
                 assert torch.equal(got["direct kernel"], got["tiled, through LDS"])
             else:  # the compiler may narrow the fused multiply-add of one kernel in a single rounding: exact ties can fall the other way
