@@ -45,14 +45,16 @@ extern "C" {
  *   "gemm_direct_lds" -1/0/3/4/64/65/66, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
  *                     buffers; 64 = K step 64, two buffers; 65 = K step 64, three buffers for A and two for B;
  *                     66 = as 65 on 16x16x32 instead of 32x32x16 MFMAs (C and D aligned to four outputs, else 65);
- *                     0 = register-staged kernel; -1 = 66 where K is a multiple of 64, else 4
+ *                     0 = register-staged kernel; -1 = 66 where K is a multiple of 64, else 4.  128 x 128 tiles:
+ *                     -1 and 66 = the 16x16x32 loop of 66 (K a multiple of 64, C and D aligned to four outputs),
+ *                     other values above 0 = 32x32x16 transfers with K step 64 (two buffers) or 32 (four)
  *   "gemm_split_tail" 0/1/2, default 1: the K steps of the tiles of a last, partly filled round of the big-tile GEMM
  *                     grid are spread over all compute units (fp32 shares in stream-ordered temporary memory, added
  *                     in a fixed order by a second kernel): never, where it pays (round at most a third full,
  *                     K >= 4096), or whenever there is such a round
  *   "compute_units"   blocks of the big-tile GEMM kernel the device runs at a time (set by tcu_init; for tests)
- *   "gemm_staged_epilogue" 0/1, default 1: the big-tile GEMM kernel on 16x16x32 MFMAs turns its outputs through LDS and
- *                     writes (and reads C in) whole rows of a wave's 128 columns, 16 bytes per lane, where C and D are
+ *   "gemm_staged_epilogue" 0/1, default 1: the GEMM kernels on 16x16x32 MFMAs turn their outputs through LDS and
+ *                     write (and read C in) whole rows of a wave's 128 or 64 columns, 16 bytes per lane, where C and D are
  *                     16-byte aligned; 0 = straight from the accumulator layout (64 / 32 bytes of 16 rows per store)
  *   "gemm_bk64"       0/1, default 0: K step 64 instead of 32 in the register-staged kernel
  *   "gemm_depth"      1..4, default 4: prefetch depth of the register-staged kernel
