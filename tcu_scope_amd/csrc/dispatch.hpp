@@ -47,6 +47,7 @@ struct Options {
   int gemv_col_shape = 82;     // column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2)
   bool gemv_strip_lds = true;  // strip GEMV (TCU_VARIANT_MFMA_16N): stage the strip through LDS where K is a multiple of 512
   int gemm_depth = 4;          // global-load prefetch depth of the K-step-32 kernel (1..4)
+  int scan_lds_pad = -1;       // KiB of LDS a block of the segmented block scan asks for and leaves unused (caps the blocks a compute unit holds); -1 = AUTO's table
   int compute_units = 256;     // blocks of the big-tile GEMM kernel the device runs at a time (one per compute unit; set by tcu_init)
   int gemm_split_tail = 1;     // spread the K steps of the tiles of a last, partly filled round of the GEMM grid over all compute units: 0 never, 1 where it pays, 2 always
   int many_totals = 65536;     // multi-kernel sequences: from this many per-segment totals on, the step over the totals is itself a multi-block launch
@@ -87,6 +88,7 @@ inline int set_option(const char *name, int value) {
   else if (n == "gemm_staged_epilogue") o.gemm_staged_epilogue = value != 0;
   else if (n == "gemm_split_tail") o.gemm_split_tail = value < 0 ? 0 : (value > 2 ? 2 : value);
   else if (n == "compute_units") o.compute_units = value < 1 ? 1 : value;
+  else if (n == "scan_lds_pad") o.scan_lds_pad = value < 0 ? -1 : value;
   else if (n == "xcd_run") o.xcd_run = value < 0 ? -1 : value;
   else if (n == "many_totals") o.many_totals = value < 1 ? 65536 : value;
   else if (n == "lookback_poll_limit") o.lookback_poll_limit = value < 0 ? kDefaultPollLimit : (unsigned)value;
@@ -173,6 +175,7 @@ struct Plan {
   bool block;  // block-per-segment kernel
   int u, w;
   unsigned c = 0;  // consecutive blocks per XCD (xcd_run_piece)
+  unsigned pad = 0;  // KiB of LDS a block asks for and leaves unused, to cap the blocks per compute unit (block scan: 52 = three, 39 = four)
 };
 // the run length a launch uses: the option when set, else the plan's (only when the plan's shape is the one launched)
 inline unsigned xcd_run_for(const Plan &plan, bool plan_shape) {
@@ -183,6 +186,11 @@ inline unsigned xcd_run_for(const Plan &plan, bool plan_shape) {
 // tiles per wave, waves per block and XCD run length with the outputs of the launches taken in turn;
 // profiles/seg_launch_shape_sweeps.md).  From 2^26 elements on one table serves every N but for the entries marked;
 // below 2^25 a launch lasts 6-13 us and is bound by how fast blocks start, so fewer and larger blocks win.
+// the unused LDS a block scan asks for, in bytes: the option when set, else the plan's (only with the plan's shape)
+inline unsigned lds_pad_for(const Plan &plan, bool plan_shape) {
+  if (options().scan_lds_pad >= 0) return (unsigned)options().scan_lds_pad * 1024u;
+  return plan_shape ? plan.pad * 1024u : 0u;
+}
 inline Plan auto_plan_reduce(size_t S, size_t N) {
   if (N < ((size_t)1 << 25)) {
     if (S <= 1024) return {false, 2, 1, 128};
@@ -213,9 +221,13 @@ inline Plan auto_plan_scan(size_t S, size_t N) {
   if (S <= 512) return {false, 2, 1, 512};
   if (S == 1024) return {true, 1, 1, 128};
   if (S == 2048) return {true, 2, 2, 256};
-  if (S == 4096) return N <= ((size_t)1 << 26) ? Plan{true, 2, 8, 0} : Plan{true, 2, 4, 128};
-  if (S == 8192) return N >= ((size_t)1 << 30) ? Plan{true, 2, 16, 32} : Plan{true, 2, 8, 32};
-  if (S == 16384) return {true, 4, 8, 8};
+  // 4096 ... 16384: blocks of 16 KiB with three or four of them on a compute unit (48 - 64 KiB in flight per unit) run
+  // 2 - 3.5 % faster than the same or larger blocks at full occupancy (2^28: 157.3 / 159.1 / 162.7 us against 162.9 /
+  // 164.0 / 166.6); at 2^30 the two shorter sizes keep their uncapped shapes (646.6 and 653.7 us, level or ahead)
+  const size_t G = (size_t)1 << 30;
+  if (S == 4096) return N >= G ? Plan{true, 2, 4, 128} : (N <= G / 16 ? Plan{true, 4, 4, 32, 39} : Plan{true, 2, 8, 8, 52});
+  if (S == 8192) return N >= G ? Plan{true, 2, 16, 32} : (N < G / 4 ? Plan{true, 4, 4, 32, 39} : Plan{true, 4, 4, 8, 39});
+  if (S == 16384) return N < G / 8 ? Plan{true, 4, 4, 8, 39} : Plan{true, 4, 4, 8, 52};
   if (S == 32768) return {true, 8, 8, 16};
   // 65536 and beyond: 8 tiles per wave, 0.72-0.74 against 0.68-0.71 for 4 (N = 2^28); the XCD runs by measurement per size
   if (S == 262144) return {true, 8, 16, 8};
@@ -640,6 +652,7 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
     const BlockShape shape = block_shape(tiles_per_seg, u, wpb, variant == TCU_VARIANT_MFMA_16N_BLOCK ? 16u : 1u);
     const size_t grid = (num_segments + shape.spb - 1) / shape.spb;
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+    next_launch_lds_pad() = lds_pad_for(plan, plan_fits && u == plan.u && wpb == plan.w);
     if (policy == kStoreStream)
       TCU_SWITCH_U_MFMA(seg_scan_block_kernel, shape.u, a.mfma, kStoreStream, (unsigned)grid, block, stream, in, out, totals, n_chunks, num_segments, tiles_per_seg, shape.spb, shape.group, run);
     else if (policy == kStoreAlternate)

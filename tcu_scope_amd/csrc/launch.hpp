@@ -28,15 +28,63 @@ inline LaunchEvents &next_launch_events() {
   return e;
 }
 
+// Bytes of LDS that the next launch of this host thread asks for beyond what its kernel declares.  The kernel
+// does not touch them: they cap how many of its blocks a compute unit holds at a time (160 KiB of LDS per unit),
+// i.e. the bytes the unit has in flight, which copy-shaped kernels with blocks of several waves are sensitive to.
+inline unsigned &next_launch_lds_pad() {
+  static thread_local unsigned n = 0;
+  return n;
+}
+// The pad a kernel can take: never more than the compute unit has left beside the kernel's own LDS; requests
+// beyond 48 KiB need the kernel's limit raised once per device.  What was found out about a kernel is kept per host
+// thread (the launch goes to the current device, as every launch of the library does).
+inline unsigned usable_lds_pad(const void *kernel, unsigned pad) {
+  struct Known { const void *kernel; int device; unsigned own, raised_to; };
+  static thread_local Known known[32];
+  static thread_local int n_known = 0;
+  constexpr unsigned kLdsPerUnit = 160u * 1024u, kNeedsRaise = 48u * 1024u;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  Known *k = nullptr;
+  for (int i = 0; i < n_known; i++)
+    if (known[i].kernel == kernel && known[i].device == device) k = &known[i];
+  if (!k) {
+    hipFuncAttributes attr{};
+    if (hipFuncGetAttributes(&attr, kernel) != hipSuccess) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    Known fresh{kernel, device, (unsigned)attr.sharedSizeBytes, 0u};
+    if (n_known < 32) k = &(known[n_known++] = fresh);
+    else k = &(known[0] = fresh);
+  }
+  if (k->own + 1024u >= kLdsPerUnit) return 0;
+  if (pad > kLdsPerUnit - 1024u - k->own) pad = kLdsPerUnit - 1024u - k->own;
+  if (pad > kNeedsRaise && pad > k->raised_to) {
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pad) != hipSuccess) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    k->raised_to = pad;
+  }
+  return pad;
+}
+
 template <typename... KArgs, typename... Args>
 inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void *stream, Args... args) {
   launch_count()++;
   LaunchEvents &ev = next_launch_events();
+  unsigned pad = next_launch_lds_pad();
+  next_launch_lds_pad() = 0;
+  if (pad) pad = usable_lds_pad(reinterpret_cast<const void *>(kernel), pad);
   if (ev.start || ev.stop) {
-    hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, static_cast<hipStream_t>(stream), ev.start, ev.stop, 0, static_cast<KArgs>(args)...);
+    hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), pad, static_cast<hipStream_t>(stream), ev.start, ev.stop, 0, static_cast<KArgs>(args)...);
     ev = LaunchEvents{};
   } else {
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, static_cast<hipStream_t>(stream), static_cast<KArgs>(args)...);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), pad, static_cast<hipStream_t>(stream), static_cast<KArgs>(args)...);
   }
 }
 

@@ -421,8 +421,13 @@ inline void spin_pause() { emu::yield(); }
 #ifndef TCU_LAUNCH_HPP
 #define TCU_LAUNCH_HPP
 namespace tcu {
+inline unsigned &next_launch_lds_pad() {  // occupancy hint of the real launch: nothing to emulate
+  static thread_local unsigned n = 0;
+  return n;
+}
 template <typename... KArgs, typename... Args>
 inline void launch(void (*kernel)(KArgs...), unsigned grid, unsigned block, void *, Args... args) {
+  next_launch_lds_pad() = 0;
   emu::launch(grid, block, [=]() { kernel(static_cast<KArgs>(args)...); });
 }
 // launches run to completion before they return here, so plain host memory is "stream ordered"
