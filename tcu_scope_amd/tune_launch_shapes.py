@@ -5,13 +5,15 @@ machine change.
 For one operation and element count, every segment size of the list is run with every combination of kernel family
 (wave kernels: WAVE_SHUFFLE, block kernels: BLOCK_LDS), 1 KiB tiles in flight per wave (1, 2, 4, 8), waves per block
 (1 ... 16) and XCD run length (blocks of one XCD on consecutive pieces of the array: 0, 8, 32, 128, 512), and once
-with AUTO.  The cases are shuffled anew for every repetition; a launch is timed by a pair of HIP events that the
+with AUTO.  With --pads the block kernels of the scan are also run with that many KiB of LDS requested and left
+unused per block (option scan_lds_pad), which caps the blocks a compute unit holds (160 KiB per unit: 39 = four
+blocks, 52 = three, 79 = two).  The cases are shuffled anew for every repetition; a launch is timed by a pair of HIP events that the
 kernel's own dispatch stamps (tcu_time_next_launch); two inputs alternate and the outputs are taken in turn
 (three buffers up to 2^28 elements, two beyond), so that nothing is served from or absorbed by the 256 MiB
 memory-side cache.  The median over the repetitions is reported as time and as a fraction of 8 TB/s (algorithmic
 bytes: reduce 2N + 2N/S, scan 4N).
 
-    python -m tcu_scope_amd.tune_launch_shapes --op scan --n-log2 28 [--sizes 16,256,...] [--markdown out.md]
+    python -m tcu_scope_amd.tune_launch_shapes --op scan --n-log2 28 [--sizes 16,256,...] [--pads 0,39,52] [--markdown out.md]
 """
 import argparse
 import random
@@ -23,6 +25,7 @@ def main():
     ap.add_argument("--op", choices=("reduce", "scan"), default="scan")
     ap.add_argument("--n-log2", type=int, default=28)
     ap.add_argument("--sizes", default=",".join(str(16 << i) for i in range(11)), help="segment sizes, comma separated")
+    ap.add_argument("--pads", default="0", help="KiB of unused LDS per block of the scan's block kernels, comma separated (0 = none)")
     ap.add_argument("--repetitions", type=int, default=5)
     ap.add_argument("--top", type=int, default=6, help="how many shapes to list per segment size")
     ap.add_argument("--markdown", default=None, help="append the table to this file")
@@ -36,14 +39,16 @@ def main():
     stream = torch.cuda.current_stream()
     kind, n = args.op, 1 << args.n_log2
     sizes = [int(s) for s in args.sizes.split(",")]
+    pads = [int(p) for p in args.pads.split(",")] if kind == "scan" else [0]
     inputs = [t.generate(n, s, t.Dist.UNIFORM) for s in (1, 2)]
     n_out = 3 if args.n_log2 <= 28 else 2
     outs = [torch.empty(n if kind == "scan" else n // min(sizes), dtype=torch.float16, device="cuda") for _ in range(n_out)]
     run = t.seg_scan if kind == "scan" else t.seg_reduce
     launches = [0]
 
-    def once(S, variant, u, w, c, events=None):
+    def once(S, variant, u, w, c, pad, events=None):
         t.set_option("xcd_run", c)
+        t.set_option("scan_lds_pad", pad)
         if events is not None:
             t.time_next_launch(*events)
         i = launches[0]
@@ -52,14 +57,15 @@ def main():
 
     cases = []
     for S in sizes:
-        cases.append((S, t.Variant.AUTO, 0, 0, -1))
+        cases.append((S, t.Variant.AUTO, 0, 0, -1, -1))
         for u in (1, 2, 4, 8):
             for w in (1, 2, 4, 8, 16):
                 for c in (0, 8, 32, 128, 512):
                     if S <= 512 or u * 512 <= S * 16:  # a wave takes at most 16 segments of a tile or more
-                        cases.append((S, t.Variant.WAVE_SHUFFLE, u, w, c))
+                        cases.append((S, t.Variant.WAVE_SHUFFLE, u, w, c, 0))
                     if S >= 512 and u * w * 512 <= max(S, 512) * 4:  # a block takes at most 4 segments at a time
-                        cases.append((S, t.Variant.BLOCK_LDS, u, w, c))
+                        for pad in pads:
+                            cases.append((S, t.Variant.BLOCK_LDS, u, w, c, pad))
     times = {}
     try:
         for _ in range(args.repetitions):
@@ -82,11 +88,12 @@ def main():
                 times.setdefault(case, []).append(a.elapsed_time(b) * 1e3)
     finally:
         t.set_option("xcd_run", -1)
+        t.set_option("scan_lds_pad", -1)
 
     def name(k):
         if k[1] == t.Variant.AUTO:
             return "AUTO"
-        return f"{'wave' if k[1] == t.Variant.WAVE_SHUFFLE else 'block'} {k[2]} x {k[3]}, run {k[4]}"
+        return f"{'wave' if k[1] == t.Variant.WAVE_SHUFFLE else 'block'} {k[2]} x {k[3]}, run {k[4]}" + (f", pad {k[5]}" if k[5] else "")
 
     lines = [f"### {kind}, N = 2^{args.n_log2} ({args.repetitions} shuffled repetitions, median kernel time in us, fraction of 8 TB/s)", "",
              "| segment size | AUTO | " + " | ".join(f"#{i + 1}" for i in range(args.top)) + " |", "|---|---|" + "---|" * args.top]
