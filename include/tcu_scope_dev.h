@@ -23,6 +23,11 @@ extern "C" {
  *                     launch: half of it is exactly that cache) runs 9 % faster, because those lines never have to
  *                     reach HBM; a scan whose output must reach HBM (outputs taken in turn, or 2 GiB of output) runs
  *                     1-3 % slower with it
+ *   "scan_lds_pad"    KiB of LDS that a block of the segmented block scan (segments of 512 halves and more) asks for and
+ *                     never touches, which caps the blocks a compute unit holds (160 KiB per unit: 39 = four blocks,
+ *                     52 = three, 79 = two); -1 (default) = AUTO's table, which caps blocks of 16 KiB at three or four
+ *                     per unit for segments of 4096 ... 16384 halves; 0 = never.  Requests beyond what a unit has left
+ *                     beside the kernel's own LDS are clipped
  *   "static_order"    0/1, default 0: full scan takes partitions in block-index order instead of by ticket
  *   "offsets_scan_chain" 0/1, default 1: tcu_seg_scan_offsets_f16 with expected segments beyond 65536 halves in one pass (a
  *                     segment's slices meet through decoupled look-back) instead of slice sums followed by a second read
