@@ -267,6 +267,35 @@ def test_scan_in_place_and_structure(tcu, oracle):
     assert np.array_equal(np.delete(a, 7, 0), np.delete(b, 7, 0)) and not np.array_equal(a[7], b[7])
 
 
+@pytest.mark.parametrize("seg", [4096, 8192, 16384])
+def test_scan_blocks_capped_per_compute_unit(tcu, oracle, seg):
+    """AUTO's block scan asks for LDS it never touches, so that a compute unit holds three or four of its blocks
+    (option scan_lds_pad, KiB; -1 = AUTO's table).  The request changes how many blocks run side by side and nothing
+    else: at 2^27 elements (and a segment count that no block shape divides) the outputs are the same bits with the
+    table's cap, without one, with two blocks per unit and with a request beyond what a unit has (clipped), and they
+    agree with the oracle; an explicit launch shape takes the option too."""
+    nseg = (1 << 27) // seg + 3
+    n = nseg * seg
+    x = oracle.generate_f16(n, 31, oracle.DIST_UNIFORM)
+    xd = to_dev(x)
+    got = {}
+    try:
+        for pad in (-1, 0, 79, 400):
+            tcu.set_option("scan_lds_pad", pad)
+            got[pad] = to_host(tcu.seg_scan(xd, seg))
+        for pad in (39, 0):  # another shape adds a segment's pieces in another order, so it is compared with itself
+            tcu.set_option("scan_lds_pad", pad)
+            got["explicit", pad] = to_host(tcu.seg_scan(xd, seg, variant=tcu.Variant.BLOCK_LDS, tiles_per_wave=2, waves_per_block=8))
+    finally:
+        tcu.set_option("scan_lds_pad", -1)
+    for key in (0, 79, 400):
+        assert np.array_equal(got[-1], got[key]), (seg, key)
+    assert np.array_equal(got["explicit", 39], got["explicit", 0]), seg
+    w = 1 << 22  # the oracle on the first and on the last stretch
+    for first in (0, n - w):
+        expect_ok(oracle, got[-1][first:first + w], oracle.seg_scan_f64(x[first:first + w], w // seg, seg), seg, (seg, first))
+
+
 def test_device_generator_matches_oracle(tcu, oracle):
     n = (1 << 20) + 13
     for dist in (tcu.Dist.UNIFORM, tcu.Dist.GRID, tcu.Dist.SMALLINT):
