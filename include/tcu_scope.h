@@ -150,7 +150,10 @@ int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_s
  * threads) race on it and must be serialised by the caller; calls on the same stream are fine.
  * The descriptors are spaced 256 bytes apart while the call has at most 4096 partitions (2^28 halves) and
  * closer beyond that, which costs a few per cent of speed.  The array is cleared by a kernel at the start of
- * every call.  No counterpart in the reference,
+ * every call.  For segments of 4096 ... 16384 halves the block scan's launch asks for LDS it leaves unused
+ * (it caps the blocks per compute unit); the first such launch of a kernel by a host thread on a device reads the
+ * kernel's attributes and raises its limit of dynamic LDS once (hipFuncGetAttributes, hipFuncSetAttribute: host-side
+ * calls that allocate nothing and put nothing on the stream).  No counterpart in the reference,
  * whose kernels take no temporary memory. */
 int tcu_seg_scan_f16_noalloc(const void *d_in, void *d_out, void *d_totals, size_t num_segments, size_t segment_size, int variant, int tiles_per_wave, int waves_per_block, void *stream);
 
