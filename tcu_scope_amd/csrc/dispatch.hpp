@@ -37,7 +37,7 @@ struct Options {
   bool nontemporal = true;
   int scan_store_policy = kStoreStream;     // stores of the segmented scans and of the copy probe while `nontemporal` is on: kStoreAlternate or kStoreStream
   bool static_order = false;
-  int gemm_big_tiles = -1;     // 256 x 256 block tiles: 1 wherever M and N allow, 0 never, -1 where there are at least 128 of them
+  int gemm_big_tiles = -1;     // 256 x 256 block tiles: 1 wherever M and N allow, 0 never, -1 where there are at least 128 of them (and 192 x 192 tiles where they fill the chip better); 192: 192 x 192 tiles wherever M and N allow
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
   bool gemm_staged_epilogue = true;   // 16x16x32 big-tile kernel: turn the outputs through LDS so that rows are written whole (C and D 16-byte aligned)
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
@@ -70,7 +70,7 @@ inline int set_option(const char *name, int value) {
   if (n == "nontemporal") o.nontemporal = value != 0;
   else if (n == "scan_store_policy") o.scan_store_policy = value == kStoreStream ? kStoreStream : kStoreAlternate;
   else if (n == "static_order") o.static_order = value != 0;
-  else if (n == "gemm_big_tiles") o.gemm_big_tiles = value < 0 ? -1 : (value != 0);
+  else if (n == "gemm_big_tiles") o.gemm_big_tiles = value < 0 ? -1 : (value == 192 ? 192 : (value != 0));
   else if (n == "gemm_direct_lds") o.gemm_direct_lds = value;
   else if (n == "gemm_depth") o.gemm_depth = value;
   else if (n == "gemv_rows") o.gemv_rows = value;
@@ -1256,6 +1256,33 @@ inline int gemm_dispatch_typed(const char *what, const void *A, const void *B, c
   // fewer than 128 tiles of 256 x 256 leave more than half of the 256 compute units idle: the
   // 128 x 128 kernel then wins (2048^3: 37.8 vs 51.9 us; 2560^3, 100 tiles: 55.8 vs 62.4; 3072^3, 144 tiles: 126 vs 72.5)
   const bool big_tiles = options().gemm_big_tiles > 0 || (options().gemm_big_tiles < 0 && (M / kGemmBigBM) * (N / kGemmBigBN) >= 128);
+  // 192 x 192 tiles where they fill the chip's rounds better than the 256 x 256 ones: a round of them costs
+  // 0.5625 of the work and 17 % for the smaller tile (9216^3: 157 against 240 us per round); the big tiles are priced
+  // with their split tail (a last round at most a third full costs its share and a fix-up).  3072^3: 256 tiles in one
+  // round, 61.9 us, against 144 of 256 compute units busy for 70.5 (fp16 outputs 56.4 against 63.4); 6144^3 and up: level
+  // or behind.  gemm_big_tiles = 192 forces them, 0 and 1 leave them out.
+  if (al && K > 0 && variant != TCU_VARIANT_MFMA_16N && M % 192 == 0 && N % 192 == 0 && K % 64 == 0 && K <= ((size_t)1 << 22) && options().gemm_direct_lds < 0 &&
+      ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & (4 * sizeof(OUT) - 1)) == 0) {
+    const size_t units = (size_t)options().compute_units, t192 = (M / 192) * (N / 192);
+    bool take = options().gemm_big_tiles == 192;
+    if (options().gemm_big_tiles < 0 && M % kGemmBigBM == 0 && N % kGemmBigBN == 0) {
+      const size_t t256 = (M / kGemmBigBM) * (N / kGemmBigBN), full = t256 / units, tail = t256 % units;
+      if (t256 >= 128) {
+        const double last = tail == 0 ? 0.0 : ((tail * 3 <= units && K >= 4096) ? (double)tail / (double)units + 0.15 : 1.0);
+        const double cost256 = ((double)full + last) * 65536.0, cost192 = (double)((t192 + units - 1) / units) * 36864.0 * 1.17;
+        take = cost192 < cost256;
+      }
+    }
+    if (take) {
+      if (t192 > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");
+      const bool staged = options().gemm_staged_epilogue && ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(D)) & 15u) == 0;
+      if (staged)
+        launch(gemm_dlds_a3b2_m16_t192_kernel<OUT, true>, (unsigned)t192, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      else
+        launch(gemm_dlds_a3b2_m16_t192_kernel<OUT, false>, (unsigned)t192, 256u, stream, a, b, c, d, M, N, K, alpha, beta);
+      return TCU_OK;
+    }
+  }
   if (lds_ok && variant != TCU_VARIANT_MFMA_16N && M % kGemmBigBM == 0 && N % kGemmBigBN == 0 && big_tiles) {
     const size_t grid = (M / kGemmBigBM) * (N / kGemmBigBN);
     if (grid > kMaxGrid) return fail(TCU_ERR_UNSUPPORTED, std::string(what) + ": grid exceeds the launch limit");

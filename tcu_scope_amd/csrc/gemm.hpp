@@ -737,30 +737,33 @@ template <typename OUT, int W8>
 TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size_t row0, size_t col0, const float4_t (&acc)[W8][W8], int lane, float alpha, float beta, float *stage) {
   constexpr int kStageRowFloats = gemm_stage_row_floats(W8);
   constexpr int PER_LANE = sizeof(OUT) == 4 ? 4 : 8;       // outputs per lane and access (16 bytes)
-  constexpr int LANES_PER_ROW = 16 * W8 / PER_LANE;        // W8 = 8: 32 or 16; W8 = 4: 16 or 8
-  constexpr int ROWS_PER_ACCESS = 64 / LANES_PER_ROW;      // 2 or 4; 4 or 8
-  constexpr int ACCESSES = 16 / ROWS_PER_ACCESS;           // per row of tiles: 8 or 4; 4 or 2
+  constexpr int LANES_PER_ROW = 16 * W8 / PER_LANE;        // W8 = 8: 32 or 16; W8 = 4: 16 or 8; W8 = 6: 24 or 12
+  constexpr int ROWS_PER_ACCESS = 64 / LANES_PER_ROW >= 8 ? 8 : 64 / LANES_PER_ROW >= 4 ? 4 : 2;  // 2 or 4; 4 or 8; 2 or 4
+  constexpr int ACCESSES = 16 / ROWS_PER_ACCESS;           // per row of tiles: 8 or 4; 4 or 2; 8 or 4
+  constexpr int ACTIVE = ROWS_PER_ACCESS * LANES_PER_ROW;  // lanes that move outputs: all 64, or 48 of them where W8 = 6
   using word_t = typename std::conditional<sizeof(OUT) == 4, float4_t, uint4_t>::type;
   const int wr = lane & 15, wq = lane >> 4;  // accumulator layout: row, group of four columns
-  const int rr = lane / LANES_PER_ROW, rc = (lane % LANES_PER_ROW) * PER_LANE;
+  const bool active = ACTIVE == 64 || lane < ACTIVE;
+  const int rr = active ? lane / LANES_PER_ROW : 0, rc = (lane % LANES_PER_ROW) * PER_LANE;  // an idle lane keeps its addresses inside the tile
   const size_t at0 = (row0 + rr) * ldc + col0 + rc;  // access t of row of tiles i: at0 + (16 i + ROWS_PER_ACCESS t) * ldc
   // the C values of a row of tiles are requested one row of tiles ahead, all at once (one wait per load would
   // leave the epilogue bound by latency); C may be D: a lane reads only what it will itself write, rows later
   word_t c[2][ACCESSES];
-  if (beta != 0.0f) {
+  if (beta != 0.0f && active) {
 #pragma unroll
     for (int t = 0; t < ACCESSES; t++) c[0][t] = __builtin_nontemporal_load(reinterpret_cast<const word_t *>(C + at0 + (size_t)(ROWS_PER_ACCESS * t) * ldc));
   }
 #pragma unroll
   for (int i = 0; i < W8; i++) {
     float *buf = stage + (i & 1) * (16 * kStageRowFloats);
-    if (beta != 0.0f && i + 1 < W8) {
+    if (beta != 0.0f && i + 1 < W8 && active) {
 #pragma unroll
       for (int t = 0; t < ACCESSES; t++) c[(i + 1) & 1][t] = __builtin_nontemporal_load(reinterpret_cast<const word_t *>(C + at0 + (size_t)(16 * (i + 1) + ROWS_PER_ACCESS * t) * ldc));
     }
 #pragma unroll
     for (int j = 0; j < W8; j++) *reinterpret_cast<float4_t *>(buf + wr * kStageRowFloats + 16 * j + 4 * wq) = alpha * acc[i][j];
     wave_lds_fence();
+    if (active) {
 #pragma unroll
     for (int t = 0; t < ACCESSES; t++) {
       const int r = t * ROWS_PER_ACCESS + rr;
@@ -785,6 +788,7 @@ TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size
         __builtin_nontemporal_store(o, d);
       }
     }
+    }
   }
 }
 
@@ -801,7 +805,9 @@ TCU_DEVICE void gemm_store_strip16_staged(OUT *D, const OUT *C, size_t ldc, size
 // accumulators go to `share` as a 256 x 256 row-major tile).  May be called several times by a block:
 // every wave waits for its own transfers before it leaves, and nothing reads LDS after the last barrier.
 // W8 = 8: the 256 x 256 block tile; W8 = 4: a 128 x 128 block tile (waves of 64 x 64 = 4 x 4 accumulators, 80 KiB of
-// LDS, two blocks per compute unit), for outputs too small to fill the chip with the big tiles.
+// LDS, two blocks per compute unit), for outputs too small to fill the chip with the big tiles; W8 = 6: a 192 x 192
+// block tile (waves of 96 x 96, 120 KiB of LDS), for outputs that 256 x 256 tiles cut into much less than a round of
+// the chip and 192 x 192 tiles into about one (3072^2: 144 against 256 tiles on 256 compute units).
 template <typename OUT, bool STAGED, int W8 = 8>
 TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t N, size_t K, size_t tile_m, size_t tile_n, size_t step0, size_t steps,
                                    float *share, float alpha, float beta) {
@@ -811,7 +817,8 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
   constexpr int OPH = TILE * ROWH;             // halves per operand per stage
   constexpr int TPW = TILE / RPT / 4;          // transfer instructions per wave, operand and step (8 or 4)
   constexpr int TEVERY = NM / 2 / TPW;         // one transfer every so many MFMAs of a substep's second half
-  static_assert(W8 == 8 || W8 == 4, "fragment reads (one before every other MFMA) and transfers must fit a substep");
+  static_assert(W8 == 8 || W8 == 6 || W8 == 4, "fragment reads (one before every other MFMA) and transfers must fit a substep");
+  static_assert(4 * W8 <= NM && (NM / 2) % TPW == 0, "fragment reads and transfers per substep");
   __shared__ __attribute__((aligned(1024))) half_t lds_a[NA][OPH];
   __shared__ __attribute__((aligned(1024))) half_t lds_b[NB][OPH];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -922,6 +929,15 @@ TCU_DEVICE void gemm_a3b2_m16_tile(const half8_t *__restrict__ A, const half8_t 
   } else {
     gemm_store_strip16(D, C, N, tile_m * TILE + wm * WT, tile_n * TILE + wn * WT, acc, lane, alpha, beta);
   }
+}
+
+// The same loop on 192 x 192 block tiles (M and N multiples of 192, K of 64, C and D aligned to four outputs): one tile
+// per block, one block per compute unit.
+template <typename OUT, bool STAGED>
+__global__ __launch_bounds__(256) void gemm_dlds_a3b2_m16_t192_kernel(const half8_t *__restrict__ A, const half8_t *__restrict__ B, const OUT *C, OUT *D, size_t M, size_t N, size_t K, float alpha, float beta) {
+  size_t tile_m, tile_n;
+  gemm_tile_of_block(M / 192, N / 192, blockIdx.x, &tile_m, &tile_n);
+  gemm_a3b2_m16_tile<OUT, STAGED, 6>(A, B, C, D, N, K, tile_m, tile_n, 0, K / 64, static_cast<float *>(nullptr), alpha, beta);
 }
 
 // The same loop on 128 x 128 block tiles (M and N multiples of 128, K of 64, C and D aligned to four outputs): one tile

@@ -478,6 +478,24 @@ def test_gemv_gemm_and_generator(emu, oracle):
                 D = aligned(M * N, np.float32, -777)  # beta = 0: C is not read
                 rc = emu.emu_gemm_f16_f32(A2i.ctypes.data, B2i.ctypes.data, None, D.ctypes.data, M, N, Ks, 1.5, 0.0, V_BLOCK)
                 assert rc == 0 and np.array_equal(D.reshape(M, N).astype(np.float64), oracle.gemm_f64(A2, B2, M, N, Ks, 1.5, 0.0, C0)), ("beta 0", Ks, staged)
+        # 192 x 192 tiles (waves of 96 x 96; 48 of 64 lanes move the outputs that went through LDS): six and two tiles,
+        # one and three K steps, outputs through LDS and straight from the accumulators, fp16 outputs in place, beta = 0
+        assert emu.emu_set_option(b"gemm_big_tiles", 192) == 0 and emu.emu_set_option(b"gemm_direct_lds", -1) == 0
+        for M3, N3, K3, staged in ((384, 576, 192, 1), (384, 576, 192, 0), (384, 192, 64, 1)):
+            assert emu.emu_set_option(b"gemm_staged_epilogue", staged) == 0
+            A3, B3 = oracle.generate_f16(M3 * K3, 17, oracle.DIST_SMALLINT), oracle.generate_f16(N3 * K3, 18, oracle.DIST_SMALLINT)
+            C3 = (np.arange(M3 * N3) % 5).astype(np.float32)
+            A3i, B3i = copy_in(A3), copy_in(B3)
+            ref3 = oracle.gemm_f64(A3, B3, M3, N3, K3, 1.5, 2.0, C3)
+            D3 = copy_in(C3, np.float32)  # in place
+            rc = emu.emu_gemm_f16_f32(A3i.ctypes.data, B3i.ctypes.data, D3.ctypes.data, D3.ctypes.data, M3, N3, K3, 1.5, 2.0, V_AUTO)
+            assert rc == 0 and np.array_equal(D3.reshape(M3, N3).astype(np.float64), ref3), ("192 tiles", M3, N3, K3, staged)
+            Dh3 = copy_in(C3.astype(np.float16).view(np.uint16))
+            rc = emu.emu_gemm_f16_f16(A3i.ctypes.data, B3i.ctypes.data, Dh3.ctypes.data, Dh3.ctypes.data, M3, N3, K3, 1.5, 2.0, V_AUTO)
+            assert rc == 0 and np.array_equal(Dh3.reshape(M3, N3), ref3.astype(np.float16).view(np.uint16)), ("192 tiles fp16", M3, N3, K3, staged)
+            D3 = aligned(M3 * N3, np.float32, -777)
+            rc = emu.emu_gemm_f16_f32(A3i.ctypes.data, B3i.ctypes.data, None, D3.ctypes.data, M3, N3, K3, 1.5, 0.0, V_AUTO)
+            assert rc == 0 and np.array_equal(D3.reshape(M3, N3).astype(np.float64), oracle.gemm_f64(A3, B3, M3, N3, K3, 1.5, 0.0, C3)), ("192 tiles beta 0", M3, N3, K3, staged)
     finally:
         for name, val in ((b"gemm_direct_lds", -1), (b"gemm_bk64", 0), (b"gemm_depth", 4), (b"gemm_big_tiles", -1), (b"compute_units", 256), (b"gemm_split_tail", 1), (b"gemm_staged_epilogue", 1)):
             emu.emu_set_option(name, val)

@@ -397,6 +397,27 @@ def test_gemm_big_tile_pipeline_shapes(tcu, oracle):
             assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("128 tiles", direct_lds, K, staged)
             assert np.array_equal(Dh.cpu().numpy().view(np.uint16), oracle.gemm_f64(A, B, M, N, K, 1.0, 0.0, C0).astype(np.float16).view(np.uint16)), ("128 tiles fp16", direct_lds, K, staged)
             assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("128 tiles fp16 in place", direct_lds, K, staged)
+        # 192 x 192 tiles, forced (the default takes them where they fill the chip better than 256 x 256 ones): M and N need
+        # not be multiples of 128
+        tcu.set_option("gemm_big_tiles", 192)
+        tcu.set_option("gemm_direct_lds", -1)
+        M3, N3 = 576, 960
+        C3 = (np.arange(M3 * N3) % 5).astype(np.float32)
+        for K, staged in ((64, 1), (448, 1), (448, 0)):
+            tcu.set_option("gemm_staged_epilogue", staged)
+            A = oracle.generate_f16(M3 * K, 23, oracle.DIST_SMALLINT)
+            B = oracle.generate_f16(N3 * K, 24, oracle.DIST_SMALLINT)
+            Ad, Bd = to_dev(A).view(M3, K), to_dev(B).view(N3, K)
+            Cd = torch.from_numpy(C3.copy()).cuda().view(M3, N3)
+            tcu.gemm(Ad, Bd, 2.0, -1.0, C=Cd, out=Cd)
+            Dh = tcu.gemm(Ad, Bd, 1.0, 0.0, out_dtype=torch.float16)
+            Ch = torch.from_numpy(C3.astype(np.float16)).cuda().view(M3, N3)
+            tcu.gemm(Ad, Bd, 2.0, -1.0, C=Ch, out=Ch)
+            torch.cuda.synchronize()
+            ref1 = oracle.gemm_f64(A, B, M3, N3, K, 2.0, -1.0, C3)
+            assert np.array_equal(Cd.cpu().numpy().astype(np.float64), ref1), ("192 tiles", K, staged)
+            assert np.array_equal(Dh.cpu().numpy().view(np.uint16), oracle.gemm_f64(A, B, M3, N3, K, 1.0, 0.0, C3).astype(np.float16).view(np.uint16)), ("192 tiles fp16", K, staged)
+            assert np.array_equal(Ch.cpu().numpy().view(np.uint16), ref1.astype(np.float16).view(np.uint16)), ("192 tiles fp16 in place", K, staged)
     finally:
         tcu.set_option("gemm_split_tail", 1)
         tcu.set_option("gemm_staged_epilogue", 1)
@@ -439,6 +460,22 @@ def test_gemm_kernels_round_alike(tcu):
                 assert torch.equal(got["direct kernel"], got["tiled, through LDS"])
             else:  # the compiler may narrow the fused multiply-add of one kernel in a single rounding: exact ties can fall the other way
                 assert int((got["direct kernel"].int() - got["tiled, through LDS"].int()).abs().max()) <= 1
+        # 192 x 192 tiles: the same loop again (768 = 3 x 256 = 4 x 192)
+        M = N = 768
+        A = tcu.generate(M * K, 8, tcu.Dist.NORMAL).view(M, K)
+        B = tcu.generate(N * K, 9, tcu.Dist.NORMAL).view(N, K)
+        for dt in (torch.float32, torch.float16):
+            C = tcu.generate(M * N, 7, tcu.Dist.UNIFORM).view(M, N).to(dt)
+            bits = torch.int32 if dt == torch.float32 else torch.int16
+            tcu.set_option("gemm_staged_epilogue", 1)
+            tcu.set_option("gemm_big_tiles", 1)
+            want = tcu.gemm(A, B, 1.1, 1.2, C=C).view(bits)
+            tcu.set_option("gemm_big_tiles", 192)
+            for staged in (1, 0):
+                tcu.set_option("gemm_staged_epilogue", staged)
+                got192 = tcu.gemm(A, B, 1.1, 1.2, C=C).view(bits)
+                torch.cuda.synchronize()
+                assert torch.equal(want, got192), ("192 tiles", dt, staged)
     finally:
         tcu.set_option("gemm_staged_epilogue", 1)
         tcu.set_option("gemm_big_tiles", -1)
