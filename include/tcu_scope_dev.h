@@ -45,8 +45,10 @@ extern "C" {
  *                     "gemv_waves" also sets the waves that split K in the strip kernels (TCU_VARIANT_MFMA_16N)
  *   "gemv_strip_lds"  0/1, default 1: TCU_VARIANT_MFMA_16N stages the 16-row strip through LDS where K is a
  *                     multiple of 512 (0: operands straight from global memory at every K)
- *   "gemm_big_tiles"  -1/0/1, default -1: 256 x 256 block tiles wherever M and N allow (1), never (0), or
- *                     where the output has at least 128 of them (-1; smaller outputs take 128 x 128 tiles)
+ *   "gemm_big_tiles"  -1/0/1/192, default -1: 256 x 256 block tiles wherever M and N allow (1), never (0), or
+ *                     where the output has at least 128 of them (-1; smaller outputs take 128 x 128 tiles, and outputs
+ *                     that 192 x 192 tiles cut into fuller rounds of the chip take those, e.g. 3072 x 3072); 192 = 192 x 192
+ *                     tiles wherever M and N are multiples of 192 and K of 64
  *   "gemm_direct_lds" -1/0/3/4/64/65/66, default -1: 3 or 4 = global -> LDS transfers, K step 32, that many LDS
  *                     buffers; 64 = K step 64, two buffers; 65 = K step 64, three buffers for A and two for B;
  *                     66 = as 65 on 16x16x32 instead of 32x32x16 MFMAs (C and D aligned to four outputs, else 65);

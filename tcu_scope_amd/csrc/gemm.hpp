@@ -17,7 +17,8 @@
 //                        one on v_mfma_f32_16x16x32_f16 (less power per multiply-add), the
 //                        others on 32x32x16.  gemm_dlds_a3b2_m16_t128_kernel (and gemm_dlds_kernel
 //                        with TILE = 128) run the same loops on 128 x 128 block tiles, two blocks per
-//                        compute unit, for outputs too small to fill the chip with the big tiles.
+//                        compute unit, for outputs too small to fill the chip with the big tiles;
+//                        gemm_dlds_a3b2_m16_t192_kernel on 192 x 192 tiles where those fill it better.
 //   gemm_direct_kernel : one 32 x 32 tile per wave, fragments loaded straight from global
 //                        memory (reference compute_gemm_naive, src/gemm/wmma_naive.cu:33-88).
 //   gemm_generic_kernel: any M, N, K; one thread per output element.
