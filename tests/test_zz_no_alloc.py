@@ -119,3 +119,35 @@ def test_noalloc_other_paths_and_limit(tcu, oracle):
         tcu.seg_scan_noalloc(small, 1 << 21, small, num_segments=(1 << 12) + 1)
     assert e.value.status == 2 and "scratch" in str(e.value)
     # exactly at the limit the host side accepts the size; not launched here (that would need 16 GiB)
+
+
+def test_noalloc_in_a_captured_graph(tcu, oracle):
+    """What the entry point is for: its launches recorded into a HIP graph (no allocation, no memset node) and replayed.
+    Three segment sizes: the wave kernel, the block scan with its LDS request (whose kernel may meet its first launch,
+    and with it the host-side attribute calls, inside the capture) and the look-back path with its clearing kernel.
+    Three replays with the program's own eager work and synchronisations between them, each checked bit for bit
+    against the rounded fp64 prefix (inputs on the k/2048 grid)."""
+    import torch
+
+    n = 1 << 23
+    x16 = oracle.generate_f16(n, 77, oracle.DIST_GRID)
+    xd = to_dev(x16)
+    sizes = (256, 8192, 1 << 22)
+    want = {s: oracle.seg_scan_f64(x16, n // s, s).astype(np.float16).view(np.uint16) for s in sizes}
+    outs = {s: torch.empty(n, dtype=torch.float16, device="cuda") for s in sizes}
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for s in sizes:
+                tcu.seg_scan_noalloc(xd, s, outs[s], stream=side)
+    for replay in range(3):
+        for s in sizes:
+            outs[s].fill_(float("nan"))
+        eager = to_host(tcu.seg_scan(xd, 2048))  # eager work of the program between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for s in sizes:
+            assert np.array_equal(to_host(outs[s]), want[s]), (replay, s)
+        assert np.array_equal(eager, oracle.seg_scan_f64(x16, n // 2048, 2048).astype(np.float16).view(np.uint16))
