@@ -36,9 +36,23 @@ inline Dim3 g_threadIdx, g_blockIdx, g_blockDim, g_gridDim;
 
 struct Fiber {
   ucontext_t ctx;
-  std::vector<char> stack;
   bool done = false;
 };
+// Fiber stacks are taken once and used again by every block of every launch: a fresh, zero-filled 256 KiB per thread
+// and block was most of the emulator's run time (page faults).
+constexpr size_t kFiberStackBytes = 256 * 1024;
+inline char *fiber_stack(unsigned thread) {
+  static std::vector<char *> pool;
+  while (pool.size() <= thread) {
+    char *p = static_cast<char *>(malloc(kFiberStackBytes));
+    if (!p) {
+      fprintf(stderr, "emu: out of memory for fiber stacks\n");
+      abort();
+    }
+    pool.push_back(p);
+  }
+  return pool[thread];
+}
 struct WaveSync {
   int arrived = 0;
   unsigned gen = 0;
@@ -118,10 +132,9 @@ inline void launch(unsigned grid, unsigned block, std::function<void()> body) {
     g_blockIdx.x = bi;
     for (unsigned t = 0; t < block; t++) {
       Fiber &f = blk.fibers[t];
-      f.stack.resize(256 * 1024);
       getcontext(&f.ctx);
-      f.ctx.uc_stack.ss_sp = f.stack.data();
-      f.ctx.uc_stack.ss_size = f.stack.size();
+      f.ctx.uc_stack.ss_sp = fiber_stack(t);
+      f.ctx.uc_stack.ss_size = kFiberStackBytes;
       f.ctx.uc_link = nullptr;
       makecontext(&f.ctx, (void (*)())fiber_entry, 0);
     }
