@@ -1,7 +1,7 @@
 """Randomised cases over the CPU emulation of the kernels (see test_emu_kernels.py): random segment sizes, variants,
-launch shapes, offsets arrays, key arrays and full-array strategies against the oracle, every operand between guard
-pages.  The default run is a fixed seed and a few dozen cases; TCU_EMU_RANDOM_SEED / TCU_EMU_RANDOM_CASES run a longer
-campaign by hand (5400 cases over 10 seeds passed when this file was written)."""
+launch shapes, offsets arrays, key arrays, full-array strategies and GEMM shapes / tile families against the oracle, every
+operand between guard pages.  The default run is a fixed seed and a few dozen cases; TCU_EMU_RANDOM_SEED / TCU_EMU_RANDOM_CASES run a longer
+campaign by hand (5400 cases over 10 seeds passed when this file was written; 1050 more over 5 seeds with the GEMM cases)."""
 import ctypes
 import os
 
@@ -11,7 +11,7 @@ import test_emu_kernels as T
 from test_emu_kernels import aligned, copy_in, emu  # noqa: F401  (emu is the fixture)
 
 SEED = int(os.environ.get("TCU_EMU_RANDOM_SEED", "2024"))
-CASES = int(os.environ.get("TCU_EMU_RANDOM_CASES", "48"))
+CASES = int(os.environ.get("TCU_EMU_RANDOM_CASES", "84"))
 sz = ctypes.c_size_t
 
 
@@ -136,10 +136,43 @@ def by_key_case(rng, emu, oracle):
     assert np.array_equal(so, want_scan[np.append(starts[1:], n) - 1]), ("run sums",) + tag
 
 
+def gemm_case(rng, emu, oracle):
+    """Random tile family (128 / 192 / 256 / none of them), K step, epilogue and scalars; integer-valued inputs, so the
+    fp32 result is exact and the fp16 result is its one rounding."""
+    unit = int(rng.choice([32, 64, 128, 192, 256]))
+    M, N = unit * int(rng.integers(1, 4 if unit >= 128 else 7)), unit * int(rng.integers(1, 4 if unit >= 128 else 7))
+    K = int(rng.choice([16, 32, 48, 64, 96, 128, 192, 320]))
+    big, staged = int(rng.choice([-1, 0, 1, 192])), int(rng.integers(0, 2))
+    alpha, beta = float(rng.choice([1.0, 0.5, 2.0, -1.5])), float(rng.choice([0.0, 1.0, -2.0]))
+    variant = int(rng.choice([T.V_AUTO, T.V_AUTO, T.V_BLOCK, T.V_MFMA_16N]))
+    tag = (M, N, K, big, staged, alpha, beta, variant)
+    A, B = oracle.generate_f16(M * K, int(rng.integers(1, 1000)), oracle.DIST_SMALLINT), oracle.generate_f16(N * K, int(rng.integers(1, 1000)), oracle.DIST_SMALLINT)
+    C0 = (np.arange(M * N) % 7 - 3).astype(np.float32)
+    ref = oracle.gemm_f64(A, B, M, N, K, alpha, beta, C0)
+    Ai, Bi = copy_in(A), copy_in(B)
+    try:
+        assert emu.emu_set_option(b"gemm_big_tiles", big) == 0 and emu.emu_set_option(b"gemm_staged_epilogue", staged) == 0
+        D = copy_in(C0, np.float32)  # in place
+        rc = emu.emu_gemm_f16_f32(Ai.ctypes.data, Bi.ctypes.data, D.ctypes.data, D.ctypes.data, M, N, K, alpha, beta, variant)
+        assert rc in (0, 2), (rc, emu.emu_last_error()) + tag  # 2: a kernel family that does not take this shape
+        if rc == 0:
+            assert np.array_equal(D.reshape(M, N).astype(np.float64), ref), ("fp32",) + tag
+        Ch = copy_in(C0.astype(np.float16).view(np.uint16))
+        Dh = aligned(M * N, np.uint16, 0x7e00)
+        rc = emu.emu_gemm_f16_f16(Ai.ctypes.data, Bi.ctypes.data, Ch.ctypes.data, Dh.ctypes.data, M, N, K, alpha, beta, variant)
+        assert rc in (0, 2), (rc, emu.emu_last_error()) + tag
+        if rc == 0:
+            # by value: with beta == 0 a negative alpha times an exact zero sum is -0.0, which the fp64 reference writes as +0.0
+            assert np.array_equal(Dh.view(np.float16).reshape(M, N), ref.astype(np.float16)), ("fp16",) + tag
+    finally:
+        emu.emu_set_option(b"gemm_big_tiles", -1)
+        emu.emu_set_option(b"gemm_staged_epilogue", 1)
+
+
 def test_random_cases(emu, oracle):
     emu.emu_seg_scan_by_key_f16.argtypes = [ctypes.c_void_p] * 3 + [sz, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(sz)]
     emu.emu_seg_reduce_by_key_f16.argtypes = [ctypes.c_void_p] * 5 + [sz, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(sz)]
     rng = np.random.default_rng(SEED)
-    kinds = (fixed_size_case, any_size_case, offsets_reduce_case, offsets_scan_case, full_array_case, by_key_case)
+    kinds = (fixed_size_case, any_size_case, offsets_reduce_case, offsets_scan_case, full_array_case, by_key_case, gemm_case)
     for i in range(CASES):
         kinds[i % len(kinds)](rng, emu, oracle)
