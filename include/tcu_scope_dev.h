@@ -37,7 +37,7 @@ extern "C" {
  *   "by_key_waves"    waves per block of the two large launches of tcu_seg_reduce_by_key_f16 (1 .. 16; 0 = default 1)
  *   "by_key_key_tiles" KiB of keys a wave of its first launch has in flight: 4, 8 or 16 (0 = default 16)
  *   "scan_lds_tiles"  full scan AUTO parks 4 extra tiles per wave in LDS (partitions of 98304 halves): 1 always, 0 never,
- *                     -1 (default) where it measures faster, i.e. between 2^27 and 2^29 elements
+ *                     -1 (default) where it measures faster, i.e. up to 2^27 elements
  *   "gemv_col_shape"  column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2); default 82
  *   "gemv_col_blocks" column-major GEMV: about this many blocks (slabs of 512 rows x stretches of K); default 1024
  *   "gemv_rows", "gemv_tiles", "gemv_waves"  0 = default: rows per block (1/2/4/8), tiles per wave and step

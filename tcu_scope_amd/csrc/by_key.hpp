@@ -65,9 +65,11 @@ TCU_DEVICE float look_back_flagged(const unsigned long long *desc, long long par
   float prefix = 0.0f;
   long long base = part - 1;
   unsigned polls = 0;
+  unsigned long long d = 0;
+  bool reload = true;  // per lane, as in look_back: a poll repeats only the reads that found nothing and still matter
   while (true) {
     const long long idx = base - lane;
-    const unsigned long long d = idx >= 0 ? atomic_load_u64(desc + ((size_t)idx << wait.desc_shift)) : (unsigned long long)kKeyStatusPrefix << 32;
+    if (reload) d = idx >= 0 ? atomic_load_u64(desc + ((size_t)idx << wait.desc_shift)) : (unsigned long long)kKeyStatusPrefix << 32;
     const unsigned hi = (unsigned)(d >> 32);
     const unsigned long long is_stop = ballot(hi >= kKeyStatusPrefix);
     const unsigned long long is_empty = ballot(hi == 0u);
@@ -78,6 +80,7 @@ TCU_DEVICE float look_back_flagged(const unsigned long long *desc, long long par
         note_expired_wait(wait, lane);
         return __builtin_nanf("");
       }
+      reload = hi == 0u && ((needed >> lane) & 1ull) != 0;
       spin_pause();
       continue;
     }
@@ -86,6 +89,7 @@ TCU_DEVICE float look_back_flagged(const unsigned long long *desc, long long par
     prefix += readlane(val, 63);
     if (first_stop < 64) return prefix;
     base -= 64;
+    reload = true;
   }
 }
 // Both walks of the reduction in one loop, so that their polls travel together: the value walk as above, and

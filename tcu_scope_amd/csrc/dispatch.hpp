@@ -41,7 +41,7 @@ struct Options {
   bool gemm_bk64 = false;      // K step 64 (prefetch depth <= 2) instead of 32
   bool gemm_staged_epilogue = true;   // 16x16x32 big-tile kernel: turn the outputs through LDS so that rows are written whole (C and D 16-byte aligned)
   int gemm_direct_lds = -1;    // 3 or 4: global -> LDS transfers, K step 32, that many LDS buffers; 64: K step 64, two buffers; 65: K step 64, three A and two B buffers; 66: as 65 on 16x16x32 MFMAs; 0: register-staged kernel; -1: by shape
-  int scan_lds_tiles = -1;     // full scan AUTO: park 4 extra tiles per wave in LDS: 1 always, 0 never, -1 where it measures faster (around 2^28 elements)
+  int scan_lds_tiles = -1;     // full scan AUTO: park 4 extra tiles per wave in LDS: 1 always, 0 never, -1 where it measures faster (up to 2^27 elements)
   int gemv_rows = 0, gemv_tiles = 0, gemv_waves = 0;  // block GEMV shape (rows per block, tiles per wave and step, waves); 0 = default
   int gemv_col_blocks = 1024;  // column-major GEMV: about this many blocks (slabs of 512 rows x stretches of K)
   int gemv_col_shape = 82;     // column-major GEMV: waves per block (4 or 8) * 10 + groups of 8 columns per wave and round (1 or 2)
@@ -913,9 +913,10 @@ inline int full_scan_dispatch(const void *d_in, void *d_out, size_t n, void *d_w
   const bool mfma = (strategy & TCU_FULL_MFMA) != 0;
   strategy &= ~TCU_FULL_MFMA;
   if (strategy < TCU_FULL_AUTO || strategy > TCU_FULL_MULTI_KERNEL) return fail(TCU_ERR_INVALID_ARG, std::string(what) + ": unknown strategy");
-  // AUTO with the default partition: the kernel that parks 4 more tiles per wave in LDS: 193 against 201 us at 2^28 elements, but 390 against 383 at 2^29, 760 against 744 at 2^30
-  // and 64.5 against 62.3 at 2^26, so only around 2^28
-  const bool lds_pays = options().scan_lds_tiles < 0 ? n > ((size_t)1 << 27) && n < ((size_t)1 << 29) : options().scan_lds_tiles != 0;
+  // AUTO with the default partition: the kernel that parks 4 more tiles per wave in LDS, against the one that holds its tiles in registers only: 20.7 against 21.7 us at 2^24
+  // elements, 61.2 against 62.1 at 2^26, 104.4 against 106.5 at 2^27, but 200.7 against 193.5 at 2^28, 381 against 366 at 2^29 and 733 against 711 at 2^30 (since a look-back
+  // poll repeats only the reads that found nothing, the register kernel gained 3.5 % and the other 1 %), so up to 2^27
+  const bool lds_pays = options().scan_lds_tiles < 0 ? n <= ((size_t)1 << 27) : options().scan_lds_tiles != 0;
   const bool lds_held = strategy == TCU_FULL_AUTO && segment_size == 0 && waves_per_block == 0 && lds_pays && !mfma;
   if (strategy == TCU_FULL_AUTO) strategy = TCU_FULL_SINGLE_PASS;
   const bool nt = options().nontemporal;

@@ -181,9 +181,11 @@ TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long 
   float prefix = 0.0f;
   long long base = part - 1;
   unsigned polls = 0;
+  unsigned long long d = 0;
+  bool reload = true;  // per lane: a poll repeats only the reads that found nothing and still matter
   while (true) {
     const long long idx = base - lane;
-    const unsigned long long d = idx >= floor ? atomic_load_u64(desc + ((size_t)idx << wait.desc_shift)) : kFlagPrefix;
+    if (reload) d = idx >= floor ? atomic_load_u64(desc + ((size_t)idx << wait.desc_shift)) : kFlagPrefix;
     const unsigned flag = (unsigned)(d >> 32);
     const unsigned long long is_prefix = ballot(flag == 2u);
     const unsigned long long is_empty = ballot(flag == 0u);
@@ -194,6 +196,9 @@ TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long 
         note_expired_wait(wait, lane);
         return __builtin_nanf("");
       }
+      // an aggregate that was read stays valid when its descriptor turns into a prefix (the look-back then
+      // merely walks on to older descriptors), so only the empty ones in front of the nearest prefix are read again
+      reload = flag == 0u && ((needed >> lane) & 1ull) != 0;
       spin_pause();
       continue;
     }
@@ -202,6 +207,7 @@ TCU_DEVICE float look_back(const unsigned long long *desc, long long part, long 
     prefix += readlane(val, 63);
     if (first_prefix < 64) return prefix;
     base -= 64;
+    reload = true;
   }
 }
 
