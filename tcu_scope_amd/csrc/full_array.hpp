@@ -104,9 +104,9 @@ constexpr unsigned kDescShift = 5;
 // sum over lanes of the published values at p[lane], lane < count (count <= 64); false if a
 // value never showed up
 TCU_DEVICE bool gather_published(const unsigned long long *p, unsigned count, int lane, float *sum, const WaitPolicy &wait) {
-  unsigned long long d = kPublished;
+  unsigned long long d = (unsigned)lane < count ? 0ull : kPublished;
   for (unsigned polls = 0;; polls++) {
-    if ((unsigned)lane < count) d = atomic_load_u64(p + lane);
+    if ((d >> 32) != 1ull) d = atomic_load_u64(p + lane);  // only what has not shown up yet is read again
     if (ballot((d >> 32) == 1ull) == ~0ull) break;
     if (polls >= wait.poll_limit) {
       note_expired_wait(wait, lane);
