@@ -225,11 +225,13 @@ inline Plan auto_plan_scan(size_t S, size_t N) {
   // 1.5 - 3 % faster than the same or larger blocks at full occupancy (2^28, identical launches back to back: 160.5 /
   // 159.3 / 162.9 us against 162.9 / 164.1 / 166.4; shuffled with other launches 157.3 / 159.1 / 162.7 against 162.9 /
   // 164.0 / 166.6).  Beyond 2^28 elements the two shorter sizes keep their uncapped shapes (2^29 back to back: level
-  // or 2 % behind), the longest its capped one up to 2^29 (325.7 against 332.7 us; 2^30: level within its scatter)
+  // or 2 % behind), the longest its capped one up to 2^29 (325.7 against 332.7 us).  At 2^30 the shapes with runs of 8
+  // blocks per XCD alternate between 660 and 720 us from launch to launch inside a fixed sequence of launches (which of two
+  // input and output buffers a launch gets), those with runs of 32 stay at 670 - 685: 2 tiles x 16 waves, as for 8192
   const size_t G = (size_t)1 << 30;
   if (S == 4096) return N > G / 4 ? Plan{true, 2, 4, 128} : (N <= G / 16 ? Plan{true, 4, 4, 32, 39} : Plan{true, 2, 8, 8, 52});
   if (S == 8192) return N >= G ? Plan{true, 2, 16, 32} : (N > G / 4 ? Plan{true, 2, 8, 32} : (N < G / 4 ? Plan{true, 4, 4, 32, 39} : Plan{true, 4, 4, 8, 39}));
-  if (S == 16384) return N >= G ? Plan{true, 4, 8, 8} : Plan{true, 4, 4, 8, 52};
+  if (S == 16384) return N >= G ? Plan{true, 2, 16, 32} : Plan{true, 4, 4, 8, 52};
   if (S == 32768) return {true, 8, 8, 16};
   // 65536 and beyond: 8 tiles per wave, 0.72-0.74 against 0.68-0.71 for 4 (N = 2^28); the XCD runs by measurement per size
   if (S == 262144) return {true, 8, 16, 8};
