@@ -18,7 +18,9 @@
  *   - temporary device memory: the kernels of the common sizes need none.  A few paths take
  *     some in stream order from a memory pool the library keeps per device (it is given back
  *     to the pool when the enqueued work has run, and the pool keeps it for the next call):
- *     tcu_seg_reduce_f16 with segments of 2^20 halves and more and tcu_seg_scan_f16 from 2^21
+ *     tcu_seg_reduce_f16 and tcu_seg_scan_f16 with TCU_VARIANT_AUTO where they cut segments into partitions: segments
+ *     of 2^20 (reduction) / 2^21 (scan) halves and more, segments of 2^17 halves and more when there are fewer than 256
+ *     of them, and segments of 2^19 halves and more from 2^30 elements on
  *     (reduction: 4 bytes per 4096 input halves, and a thousandth of that again for segments
  *     beyond 2^25; scan: 256 bytes per 65536 input halves), the *_offsets_f16 entry points with
  *     expected segment lengths beyond 65536 halves (reduction 4, scan up to 256 bytes per 65536 halves), and tcu_gemm_* when the
@@ -142,7 +144,8 @@ int tcu_seg_scan_f16(const void *d_in, void *d_out, void *d_totals, size_t num_s
 /* tcu_seg_scan_f16 for callers that cannot allocate device memory (code under HIP graph
  * capture, serving loops, harnesses that forbid hipMalloc): same arguments, same kernels, same
  * results, but the partition descriptors of the look-back path (TCU_VARIANT_AUTO with segments of
- * 2^21 halves and more, the only path of tcu_seg_scan_f16 that takes temporary memory) live in a
+ * 2^21 halves and more, of 2^17 and more when there are fewer than 256 of them, of 2^19 and more from 2^30
+ * elements on: the only path of tcu_seg_scan_f16 that takes temporary memory) live in a
  * 1 MiB + 256 B array that is part of the library's device code, so this entry point never calls
  * an allocating routine.  Limit: num_segments * segment_size <= 2^33 halves on that path (131072
  * partitions of 65536 halves; larger calls return TCU_ERR_UNSUPPORTED).  Each GPU holds one such

@@ -344,6 +344,16 @@ inline void launch_reduce_small_s(int lps_log2, int u, unsigned grid, unsigned b
 // the single-pass look-back scan with the look-back stopped at segment starts.  Both need a
 // few bytes per partition of temporary device memory, taken in stream order.
 constexpr size_t kHugeReduceSegment = (size_t)1 << 20, kHugeScanSegment = (size_t)1 << 21, kHugePartHalves = 65536;
+// Below those sizes a block walks a segment by itself, which also loses where the segments are too few to give every
+// compute unit one (a block walks 1 MiB in about 40 us whatever the others do: N = 2^26 in segments of 2^19 halves
+// reduces in 43.9 us walking and in 24.0 us cut into partitions, N = 2^26 in segments of 2^20 scans in 105 against 61 us),
+// and, less, from 2^30 elements on in segments of 2^19 halves and more (reduce 317 against 298 - 307 us, scan 726 against
+// 712 and 730 against 704); with 256 segments and more of up to 2^18 halves the walking block is level or ahead.
+inline bool is_pow2_size(size_t x) { return x && !(x & (x - 1)); }
+inline bool few_long_segments(size_t S, size_t num_segments) { return S >= ((size_t)1 << 17) && num_segments < 256; }
+inline bool many_elements_long_segments(size_t S, size_t num_segments) { return S >= ((size_t)1 << 19) && num_segments * S >= ((size_t)1 << 30); }
+inline bool reduce_cuts_segments(size_t S, size_t num_segments) { return S >= kHugeReduceSegment || (is_pow2_size(S) && (few_long_segments(S, num_segments) || many_elements_long_segments(S, num_segments))); }
+inline bool scan_cuts_segments(size_t S, size_t num_segments) { return S >= kHugeScanSegment || (is_pow2_size(S) && (few_long_segments(S, num_segments) || many_elements_long_segments(S, num_segments))); }
 
 // The partition sums (full-array reduction, segments of 2^20 halves and more) take the launch shape that the
 // segmented reduction of 4096-half segments measures fastest: blocks of 4 waves x 2 tiles, every XCD on 128
@@ -449,7 +459,7 @@ inline int seg_reduce_dispatch(const void *d_in, void *d_out, size_t num_segment
     launch(seg_reduce_generic_kernel, (unsigned)grid, (unsigned)gw * 64u, stream, static_cast<const uint16_t *>(d_in), out, num_segments, S);
     return TCU_OK;
   }
-  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeReduceSegment) return seg_reduce_huge(in, out, num_segments, S, nt, stream);
+  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && reduce_cuts_segments(S, num_segments)) return seg_reduce_huge(in, out, num_segments, S, nt, stream);
   const size_t n_chunks = N / 8;
   const Plan plan = auto_plan_reduce(S, N);
   // A segment shorter than a tile cannot be shared by the waves of a block: below 512 halves the block families
@@ -641,7 +651,7 @@ inline int seg_scan_dispatch(const void *d_in, void *d_out, void *d_totals, size
     launch(seg_scan_generic_kernel, (unsigned)grid, (unsigned)gw * 64u, stream, static_cast<const uint16_t *>(d_in), static_cast<uint16_t *>(d_out), totals, num_segments, S);
     return TCU_OK;
   }
-  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && S >= kHugeScanSegment) return seg_scan_huge(what, in, out, totals, num_segments, S, nt, stream, scratch);
+  if (variant == TCU_VARIANT_AUTO && !tiles_per_wave && !waves_per_block && scan_cuts_segments(S, num_segments)) return seg_scan_huge(what, in, out, totals, num_segments, S, nt, stream, scratch);
   const size_t n_chunks = N / 8;
   const Plan plan = auto_plan_scan(S, N);
   const bool use_block = S >= kTileHalves && (variant == TCU_VARIANT_AUTO ? plan.block : is_block_variant(variant));  // as in the reduction

@@ -114,7 +114,7 @@ def test_segmented_kernels_bit_exact_on_grid_inputs(emu, oracle, seg, variants, 
 
 
 def test_segments_larger_than_a_block_can_walk(emu, oracle):
-    """AUTO cuts segments of 2^20 (reduce) / 2^21 (scan) halves and more into 65536-half partitions:
+    """AUTO cuts segments of 2^20 (reduce) / 2^21 (scan) halves and more into partitions:
     partition sums + per-segment finish, and the look-back scan restarted at segment starts."""
     seg, nseg = 1 << 20, 2
     x = oracle.generate_f16(nseg * seg, 5, oracle.DIST_GRID)
@@ -132,6 +132,18 @@ def test_segments_larger_than_a_block_can_walk(emu, oracle):
     assert emu.emu_seg_scan_f16(xi.ctypes.data, out.ctypes.data, tot.ctypes.data, nseg, seg, V_AUTO, 0, 0) == 0, emu.emu_last_error()
     assert np.array_equal(out[:nseg * seg], want) and np.all(out[nseg * seg:] == 0xFFFF)
     assert np.array_equal(tot[:nseg], want.reshape(nseg, seg)[:, -1]) and np.all(tot[nseg:] == 0xFFFF)
+    # fewer segments than compute units: AUTO cuts them into partitions from 2^17 halves on (a block that walks such a
+    # segment alone would leave most of the chip idle)
+    seg, nseg = 1 << 17, 3
+    x = oracle.generate_f16(nseg * seg, 7, oracle.DIST_GRID)
+    want = oracle.seg_scan_f64(x, nseg, seg).astype(np.float16).view(np.uint16)
+    xi = copy_in(x)
+    red = aligned(nseg + 8, np.uint16, 0xFFFF)
+    assert emu.emu_seg_reduce_f16(xi.ctypes.data, red.ctypes.data, nseg, seg, V_AUTO, 0, 0) == 0, emu.emu_last_error()
+    assert np.array_equal(red[:nseg], want.reshape(nseg, seg)[:, -1]) and np.all(red[nseg:] == 0xFFFF)
+    out = aligned(nseg * seg + 64, np.uint16, 0xFFFF)
+    assert emu.emu_seg_scan_f16(xi.ctypes.data, out.ctypes.data, None, nseg, seg, V_AUTO, 0, 0) == 0, emu.emu_last_error()
+    assert np.array_equal(out[:nseg * seg], want) and np.all(out[nseg * seg:] == 0xFFFF)
 
 
 def ragged_offsets(rng, n, nseg, max_len):

@@ -351,15 +351,17 @@ def test_full_size_seg_scan(tcu, oracle, seg):
             assert torch.equal(tcu.seg_scan(gd, seg, variant=v), base), f"grid inputs: {v.name} differs from WAVE_SHUFFLE"
 
 
-@pytest.mark.parametrize("seg_log2", [20, 21, 24, 28])
-def test_segments_larger_than_a_block_can_walk(tcu, oracle, seg_log2):
-    """AUTO on segments of 2^20 halves and more (partition sums / look-back scan restarted at
-    segment starts), up to the whole 2^28 array as one segment: uniform inputs within the
-    tolerance, exact-grid inputs bit for bit, per-segment totals, repeated calls."""
+@pytest.mark.parametrize("seg_log2,n_log2", [(17, 24), (19, 24), (17, 26), (20, 24), (21, 24), (24, 24), (28, 28)])
+def test_segments_larger_than_a_block_can_walk(tcu, oracle, seg_log2, n_log2):
+    """AUTO on segments that are cut into partitions (partition sums / look-back scan restarted at segment starts):
+    2^20 (reduce) and 2^21 (scan) halves and more, up to the whole 2^28 array as one segment, and segments from 2^17
+    halves on when there are fewer of them than compute units (128 and 32 segments here; 512 segments of 2^17 halves
+    stay with the block that walks a segment): uniform inputs within the tolerance, exact-grid inputs bit for bit,
+    per-segment totals, repeated calls."""
     import torch
 
     seg = 1 << seg_log2
-    n = max(1 << 24, seg) if seg_log2 < 28 else seg
+    n = 1 << n_log2
     nseg = n // seg
     x = oracle.generate_f16(n, 3, oracle.DIST_UNIFORM)
     xd = to_dev(x)
