@@ -32,7 +32,7 @@ def test_full_reduce_and_scan(tcu, oracle, n):
             continue
         expect_ok(oracle, red, ref[-1:], n, f"full reduce n={n} strategy={int(strategy):#x} seg={seg}")
         expect_ok(oracle, sc, ref, n, f"full scan n={n} strategy={int(strategy):#x} seg={seg}")
-    # AUTO with 4 more tiles per wave parked in LDS, which the library itself only takes around 2^28 elements
+    # AUTO with 4 more tiles per wave parked in LDS, which the library itself only takes up to 2^27 elements
     try:
         tcu.set_option("scan_lds_tiles", 1)
         expect_ok(oracle, to_host(tcu.full_scan(xd)), ref, n, f"full scan n={n} with tiles parked in LDS")
@@ -118,7 +118,7 @@ def test_a_wait_that_expires_gives_nan_not_wrong_numbers(tcu, oracle):
         tcu.set_option("test_mute_partition", mute)
         # (strategy, segment_size, waves) -> halves per partition
         for strategy, seg, w, part in [(S.SINGLE_PASS, 0, 0, 65536), (S.SINGLE_PASS, 8192, 4, 8192), (S.AUTO, 0, 0, 98304), (S.SINGLE_PASS | tcu.FULL_MFMA, 0, 0, 65536)]:
-            tcu.set_option("scan_lds_tiles", 1 if part == 98304 else -1)  # AUTO with tiles parked in LDS: forced, the library takes it around 2^28 elements only
+            tcu.set_option("scan_lds_tiles", 1 if part == 98304 else -1)  # AUTO with tiles parked in LDS: forced, the library takes it up to 2^27 elements only
             ws = torch.zeros(tcu.binding.full_workspace_bytes("scan", n, strategy, seg, w) // 4, dtype=torch.int32, device="cuda")
             got = to_host(tcu.full_scan(xd, strategy, seg, w, workspace=ws))
             # word 1 of the workspace counts the waits that gave up: the partition behind the silent one for certain,
